@@ -119,17 +119,16 @@ def test_maxpool(case):
         assert torch.equal(po.maxpool_bwd(y, dy, x, ks, st, pad, "first").to(torch.int32), ref.to(torch.int8).to(torch.int32))
         assert torch.equal(co.maxpool_bwd(y, dy, x, ks, st, pad, "first"), po.maxpool_bwd(y, dy, x, ks, st, pad, "first"))
         assert torch.equal(co.maxpool_bwd(y, dy, x, ks, st, pad, "all"), po.maxpool_bwd(y, dy, x, ks, st, pad, "all"))
-    # 2x2/s2 without ties: both rules coincide and dx sums to dy per window
-    x = torch.arange(N * H * W * C).reshape(N, H, W, C).remainder(251).sub(125).to(torch.int8)
-    if ks == 2 and st == 2:
-        perm = torch.randperm(x.numel(), generator=g)
-        x = x.flatten()[perm].reshape(N, H, W, C)
+    # no ties inside any (n, c) plane: both rules coincide; without window overlap dx sums to dy
+    planes = torch.stack([torch.randperm(H * W, generator=g) for _ in range(N * C)]).reshape(N, C, H, W)
+    x = (planes - 60).permute(0, 2, 3, 1).contiguous().to(torch.int8)
     y = po.maxpool_fwd(x, ks, st, pad)
     dy = ri8(g, *y.shape, lo=-20, hi=20)
     a, b = po.maxpool_bwd(y, dy, x, ks, st, pad, "first"), po.maxpool_bwd(y, dy, x, ks, st, pad, "all")
+    assert torch.equal(a, b)
     if st >= ks:
         assert int(a.to(torch.int64).sum()) == int(dy.to(torch.int64).sum())
-        assert torch.equal(a, b)
+        assert int((a != 0).sum()) <= dy.numel()
 
 
 def test_ti_loss_shapes_and_sign():
