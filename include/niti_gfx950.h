@@ -1,0 +1,166 @@
+/*
+ * libniti_gfx950 -- C ABI of the MI355X (gfx950) int8 training hot path of NITI.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream (passed as void*),
+ * launches asynchronously on that stream and returns a status code (0 = success).  Nothing
+ * here allocates device memory: outputs and workspaces are the caller's.  Layouts follow the
+ * reference: activations NHWC int8, filters KRSC int8, conv results NPQK int32, GEMM
+ * operands row-major.  "Reference" below is wangmaolin/niti; paths are relative to it.
+ *
+ * Per-tensor range: kernels that take `absmax` atomically max |value| into *absmax (uint32,
+ * device memory, zeroed by the caller, e.g. with niti_fill_u32).  The requantisation kernels
+ * read it back on the device, so no host synchronisation is needed between a GEMM and its
+ * requantisation (the reference synchronises twice per tensor, ti_torch.py:369-377).
+ */
+#ifndef NITI_GFX950_H
+#define NITI_GFX950_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+enum {
+  NITI_OK = 0,
+  NITI_ERR_INVALID_ARG = 1, /* null pointer, non-positive size, misaligned pointer */
+  NITI_ERR_UNSUPPORTED = 2, /* shape outside what the kernels implement (message says which) */
+  NITI_ERR_WORKSPACE = 3,   /* workspace missing or too small */
+  NITI_ERR_LAUNCH = 4       /* HIP reported a launch error */
+};
+
+/* conv / gemm flags */
+#define NITI_EPI_F32_ROUNDTRIP 1u /* pass every int32 result through fp32 and back, as the
+                                     reference's CUTLASS epilogue does
+                                     (pytorch/cutlass-extension/cutlassconv_kernel.cu:78-85) */
+/* requant flags */
+#define NITI_RQ_RELU 1u /* clamp the int8 result at 0 (TiReLU.forward, ti_torch.py:272-279) */
+
+/* rounding method (ti_torch.py:23-69) / division meaning / bit-width evaluation / pool ties */
+enum { NITI_ROUND_NEAREST = 0, NITI_ROUND_STOCHASTIC = 1, NITI_ROUND_PSEUDO_STOCHASTIC = 2 };
+enum { NITI_DIV_FLOOR = 0, NITI_DIV_TRUNC = 1 };
+enum { NITI_BW_INT = 0, NITI_BW_F32 = 1 };
+enum { NITI_TIES_FIRST = 0, NITI_TIES_ALL = 1 };
+
+int niti_version(void);
+const char* niti_status_string(int status);
+/* message of the last failing call on this host thread ("" if none) */
+const char* niti_last_error(void);
+
+/* Host-side evaluation of the bit-width rule the kernels use (ti_torch.py:366-377):
+ * NITI_BW_INT: ceil(log2(r)) as exact integer arithmetic; NITI_BW_F32: the reference's
+ * int(ceil(log2f((float)r))) under a correctly rounded log2f.  r == 0 gives 0. */
+int niti_bitwidth(uint32_t r, int bw_mode);
+
+/* dst[0..n) = value */
+int niti_fill_u32(uint32_t* dst, int64_t n, uint32_t value, void* stream);
+
+/*
+ * Convolution forward (cross-correlation), replaces cutlassconv_cuda.sp_conv and
+ * .sp_conv_optimized (pytorch/cutlass-extension/cutlassconv.cpp:57-73,
+ * cutlassconv_kernel.cu:38-319):
+ *   y[n,p,q,k] = sum_{r,s,c} x[n, p*stride-pad+r, q*stride-pad+s, c] * w[k,r,s,c]
+ * x: [N,H,W,C] int8, w: [K,R,S,C] int8, y: [N,P,Q,K] int32, P=(H+2*pad-R)/stride+1.
+ * Requires C % 16 == 0 (the reference pads C the same way, ti_torch.py:178-183) and 16-byte
+ * aligned x, w, y.  absmax may be NULL.
+ */
+int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y, int N, int H, int W, int C, int K, int R,
+                         int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* stream);
+
+/*
+ * Data gradient, replaces the reference's fprop-on-flipped-weights rewrite
+ * (TiConv2d.backward, ti_torch.py:403-405):
+ *   dx[n,h,w,c] = sum_{r,s,k} err[n, h+pad-r, w+pad-s, k] * w[k,r,s,c]
+ * err: [N,P,Q,K] int8, w: [K,R,S,C] int8, dx: [N,H,W,C] int32.  Like the reference it is
+ * defined for stride 1 with 2*pad == R-1 == S-1 only; needs K % 16 == 0.
+ * Workspace: niti_conv2d_i8_dgrad_workspace() bytes (re-laid filter).
+ */
+size_t niti_conv2d_i8_dgrad_workspace(int C, int K, int R, int S);
+int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N, int H, int W, int C, int K, int R,
+                         int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/*
+ * Weight gradient, replaces the reference's fprop-on-transposed-operands rewrite
+ * (ti_torch.py:430-432) and, for the first layer, conv2d_weight_int8 -> group_conv
+ * (ti_torch.py:194-233):
+ *   dw[k,r,s,c] = sum_{n,p,q} err[n,p,q,k] * act[n, p+r-pad, q+s-pad, c]
+ * act: [N,H,W,C] int8, err: [N,P,Q,K] int8, dw: [K,R,S,C] int32.  Stride 1 only; any C, K, N.
+ * Workspace: niti_conv2d_i8_wgrad_workspace() bytes.  absmax may be NULL.
+ */
+size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad);
+int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int N, int H, int W, int C, int K,
+                         int R, int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/*
+ * int8 x int8 -> exact int32 GEMM, replaces int8mm_cuda.int8_mm
+ * (pytorch/int8mm-extension/int8mm.cpp:9-14, int8mm_kernel.cu:8-34):
+ *   c[m,n] = sum_k opA[m,k] * opB[k,n],  c row-major with leading dimension n.
+ * trans_a == 0: a is [m,k] row-major; 1: a is [k,m].  trans_b == 0: b is [k,n]; 1: b is [n,k].
+ * (trans_a=0, trans_b=1) streams both operands as stored; the other forms first re-lay the
+ * operand(s) into the workspace (niti_gemm_i8_workspace() bytes; 0 for the direct form when
+ * k % 16 == 0).
+ */
+size_t niti_gemm_i8_workspace(int trans_a, int trans_b, int m, int n, int k);
+int niti_gemm_i8(int trans_a, int trans_b, const int8_t* a, const int8_t* b, int32_t* c, int m, int n, int k,
+                 unsigned flags, uint32_t* absmax, void* workspace, size_t workspace_bytes, void* stream);
+
+/* max |x[i]| atomically folded into *absmax (RangeEstimate, ti_torch.py:369-377) */
+int niti_absmax_i32(const int32_t* x, int64_t n, uint32_t* absmax, void* stream);
+
+/*
+ * act_calc / err_calc / grad_calc (ti_torch.py:103-147) in one pass:
+ *   shift = bitwidth(*absmax) - target_bits
+ *   shift >= 1: y = clip(round_method(x, shift), +-127)   else: y = low byte of x (128 wraps)
+ *   *shift_out = max(shift, 0)                            (shift_out may be NULL)
+ * target_bits = 7 for activations and errors, GRAD_BITWIDTH (5/4/3) for gradients.
+ * rand: one int32 per element in [0, 2^shift), NITI_ROUND_STOCHASTIC only (stands in for the
+ * reference's device torch.randint, ti_torch.py:41).
+ */
+int niti_requant_i32_i8(const int32_t* x, int8_t* y, int64_t n, const uint32_t* absmax, int target_bits,
+                        int method, int div_mode, int bw_mode, const int32_t* rand, unsigned flags,
+                        int32_t* shift_out, void* stream);
+
+/*
+ * UpdateWeight.weight_update (ti_torch.py:16-21) fused with grad_calc:
+ *   g8 = grad_calc(g, mu);  w = clip(int16(w) - int16(g8), +-127)
+ * g8_out (int8, may be NULL) receives the rounded gradient.
+ */
+int niti_grad_update_i8(const int32_t* g, int8_t* w, int64_t n, const uint32_t* absmax, int mu, int method,
+                        int div_mode, int bw_mode, const int32_t* rand, int8_t* g8_out, int32_t* shift_out,
+                        void* stream);
+
+/* w = clip(int16(w) - int16(g), +-127)  (ti_torch.py:21) */
+int niti_weight_update_i8(int8_t* w, const int8_t* g, int64_t n, void* stream);
+
+/* y = max(x, 0) (ti_torch.py:278);  dx = act > 0 ? dy : 0 (ti_torch.py:289) */
+int niti_relu_i8_fwd(const int8_t* x, int8_t* y, int64_t n, void* stream);
+int niti_relu_i8_bwd(const int8_t* act, const int8_t* dy, int8_t* dx, int64_t n, void* stream);
+
+/*
+ * NHWC int8 max pooling, replaces int8pool_cuda.int8_pool / int8_pool_backward
+ * (pytorch/int8pool-extension/int8pool.cpp:37-57, int8pool_kernel.cu:28-138).
+ * x: [N,H,W,C], y/dy: [N,P,Q,C], dx: [N,H,W,C], P=(H+2*pad-ks)/stride+1.
+ * Backward routes dy to the position(s) of x equal to y: the first in (kh,kw) scan order
+ * (NITI_TIES_FIRST) or all of them (NITI_TIES_ALL); overlapping windows add.
+ */
+int niti_maxpool_i8_fwd(const int8_t* x, int8_t* y, int N, int H, int W, int C, int ks, int stride, int pad,
+                        void* stream);
+int niti_maxpool_i8_bwd(const int8_t* y, const int8_t* dy, const int8_t* x, int8_t* dx, int N, int H, int W, int C,
+                        int ks, int stride, int pad, int ties, void* stream);
+
+/*
+ * Grouped int8 convolution with float32 output, replaces int8conv_cuda.group_conv
+ * (pytorch/int8conv-extension/int8conv.cpp:35-44, int8conv_kernel.cu:248-334):
+ * x: [N,H,W,G*Cg] int8, w: [K,R,S,Cg] int8 (K % G == 0, filter k belongs to group k/(K/G)),
+ * y: [N,P,Q,K] float32 (integer-valued; exact while |sum| < 2^24).
+ */
+int niti_group_conv_i8_f32(const int8_t* x, const int8_t* w, float* y, int N, int H, int W, int C, int K, int R,
+                           int S, int Cg, int stride, int pad, int dilation, int groups, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* NITI_GFX950_H */

@@ -1,0 +1,74 @@
+"""ctypes binding of libniti_gfx950.so (the C ABI declared in include/niti_gfx950.h).
+
+The library is the only implementation of the hot path: if it cannot be loaded every op of
+this package raises, there is no fallback."""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+SO_PATH = os.path.join(_HERE, "libniti_gfx950.so")
+
+OK = 0
+EPI_F32_ROUNDTRIP = 1
+RQ_RELU = 1
+ROUND = {"round": 0, "sto": 1, "psto": 2}
+DIV = {"floor": 0, "trunc": 1}
+BW = {"int": 0, "f32": 1}
+TIES = {"first": 0, "all": 1}
+
+_vp, _i, _u, _i64, _sz = C.c_void_p, C.c_int, C.c_uint, C.c_int64, C.c_size_t
+
+# name -> (restype, argtypes); must list every symbol of include/niti_gfx950.h
+SIGNATURES = {
+    "niti_version": (_i, []),
+    "niti_status_string": (C.c_char_p, [_i]),
+    "niti_last_error": (C.c_char_p, []),
+    "niti_bitwidth": (_i, [C.c_uint32, _i]),
+    "niti_fill_u32": (_i, [_vp, _i64, C.c_uint32, _vp]),
+    "niti_conv2d_i8_fprop": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp]),
+    "niti_conv2d_i8_dgrad_workspace": (_sz, [_i] * 4),
+    "niti_conv2d_i8_dgrad": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp, _sz, _vp]),
+    "niti_conv2d_i8_wgrad_workspace": (_sz, [_i] * 8),
+    "niti_conv2d_i8_wgrad": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp, _sz, _vp]),
+    "niti_gemm_i8_workspace": (_sz, [_i] * 5),
+    "niti_gemm_i8": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _i, _u, _vp, _vp, _sz, _vp]),
+    "niti_absmax_i32": (_i, [_vp, _i64, _vp, _vp]),
+    "niti_requant_i32_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _u, _vp, _vp]),
+    "niti_grad_update_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "niti_weight_update_i8": (_i, [_vp, _vp, _i64, _vp]),
+    "niti_relu_i8_fwd": (_i, [_vp, _vp, _i64, _vp]),
+    "niti_relu_i8_bwd": (_i, [_vp, _vp, _vp, _i64, _vp]),
+    "niti_maxpool_i8_fwd": (_i, [_vp, _vp] + [_i] * 7 + [_vp]),
+    "niti_maxpool_i8_bwd": (_i, [_vp, _vp, _vp, _vp] + [_i] * 8 + [_vp]),
+    "niti_group_conv_i8_f32": (_i, [_vp, _vp, _vp] + [_i] * 12 + [_vp]),
+}
+
+_lib = None
+
+
+class NitiError(RuntimeError):
+    """A C-ABI call returned a non-zero status (the reference's extensions call exit() here)."""
+
+
+def lib() -> C.CDLL:
+    global _lib
+    if _lib is None:
+        if not os.path.exists(SO_PATH):
+            raise ImportError(
+                "niti_amd: %s is missing; build it with `python -m niti_amd.build` "
+                "(there is no fallback implementation)" % SO_PATH)
+        handle = C.CDLL(SO_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(status: int, what: str) -> None:
+    if status != OK:
+        l = lib()
+        raise NitiError("%s: %s (%s)" % (what, l.niti_status_string(status).decode(), l.niti_last_error().decode()))

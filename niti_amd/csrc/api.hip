@@ -1,0 +1,216 @@
+// extern "C" surface of libniti_gfx950: argument checking, workspace carving and the
+// composition of kernels behind each entry point declared in include/niti_gfx950.h.
+#include <stdarg.h>
+#include <string.h>
+
+#include "common.h"
+
+namespace niti {
+namespace {
+thread_local char g_err[512] = {0};
+
+__global__ void pad_rows_i8_kernel(const int8_t* __restrict__ src, int8_t* __restrict__ dst, int64_t rows, int k, int kpad) {
+  const int64_t total = rows * kpad;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += stride) {
+    const int64_t r = i / kpad;
+    const int c = static_cast<int>(i - r * kpad);
+    dst[i] = c < k ? src[r * k + c] : static_cast<int8_t>(0);
+  }
+}
+
+inline size_t round256(size_t v) { return (v + 255) & ~static_cast<size_t>(255); }
+inline int round16(int v) { return (v + 15) & ~15; }
+
+int pick_split(long long tiles, int kiters) {
+  // aim at ~3 workgroups per compute unit, keep at least 8 main-loop steps per slice
+  long long want = (768 + tiles - 1) / tiles;
+  long long maxs = kiters / 8;
+  if (maxs < 1) maxs = 1;
+  if (want > maxs) want = maxs;
+  if (want < 1) want = 1;
+  return static_cast<int>(want);
+}
+}  // namespace
+
+int fail(int status, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return status;
+}
+void clear_error() { g_err[0] = 0; }
+
+}  // namespace niti
+
+using namespace niti;
+
+extern "C" int niti_version(void) { return 100; }
+
+extern "C" const char* niti_status_string(int status) {
+  switch (status) {
+    case NITI_OK: return "ok";
+    case NITI_ERR_INVALID_ARG: return "invalid argument";
+    case NITI_ERR_UNSUPPORTED: return "unsupported shape";
+    case NITI_ERR_WORKSPACE: return "workspace too small";
+    case NITI_ERR_LAUNCH: return "kernel launch failed";
+    default: return "unknown status";
+  }
+}
+
+extern "C" const char* niti_last_error(void) { return g_err; }
+
+extern "C" int niti_bitwidth(uint32_t r, int bw_mode) { return bitwidth_of(r, bw_mode); }
+
+extern "C" int niti_fill_u32(uint32_t* dst, int64_t n, uint32_t value, void* stream) {
+  clear_error();
+  if (n < 0 || (n > 0 && dst == nullptr)) return fail(NITI_ERR_INVALID_ARG, "fill: bad arguments");
+  return launch_fill_u32(dst, n, value, static_cast<hipStream_t>(stream));
+}
+
+static int check_conv_dims(const char* who, int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0)
+    return fail(NITI_ERR_INVALID_ARG, "%s: non-positive extent (N=%d H=%d W=%d C=%d K=%d R=%d S=%d)", who, N, H, W, C, K, R, S);
+  if (stride <= 0 || pad < 0) return fail(NITI_ERR_INVALID_ARG, "%s: stride=%d pad=%d", who, stride, pad);
+  if (H + 2 * pad < R || W + 2 * pad < S) return fail(NITI_ERR_INVALID_ARG, "%s: filter larger than padded input", who);
+  return NITI_OK;
+}
+
+extern "C" int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y, int N, int H, int W, int C, int K,
+                                    int R, int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* stream) {
+  clear_error();
+  int st = check_conv_dims("conv_fprop", N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
+  if (x == nullptr || w == nullptr || y == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: null pointer");
+  if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: pointers must be 16-byte aligned");
+  const int P = (H + 2 * pad - R) / stride + 1, Q = (W + 2 * pad - S) / stride + 1;
+  ConvProblem p{x, w, y, absmax, N, H, W, C, K, R, S, stride, pad,
+                static_cast<long long>(P) * Q * K, static_cast<long long>(Q) * K, K, 1, 1, flags};
+  return launch_conv_igemm(p, static_cast<hipStream_t>(stream));
+}
+
+extern "C" size_t niti_conv2d_i8_dgrad_workspace(int C, int K, int R, int S) {
+  if (C <= 0 || K <= 0 || R <= 0 || S <= 0) return 0;
+  return round256(static_cast<size_t>(C) * R * S * K);
+}
+
+extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N, int H, int W, int C, int K,
+                                    int R, int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  clear_error();
+  int st = check_conv_dims("conv_dgrad", N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
+  if (err == nullptr || w == nullptr || dx == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_dgrad: null pointer");
+  if (stride != 1 || R != S || pad > R - 1)
+    return fail(NITI_ERR_UNSUPPORTED, "conv_dgrad: needs stride 1, square filter, pad <= R-1 (stride=%d R=%d S=%d pad=%d)", stride, R, S, pad);
+  if (K % 16 != 0) return fail(NITI_ERR_UNSUPPORTED, "conv_dgrad: K=%d must be a multiple of 16", K);
+  if (!aligned16(err) || !aligned16(dx)) return fail(NITI_ERR_INVALID_ARG, "conv_dgrad: pointers must be 16-byte aligned");
+  const size_t need = niti_conv2d_i8_dgrad_workspace(C, K, R, S);
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    return fail(NITI_ERR_WORKSPACE, "conv_dgrad: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  int8_t* wt = static_cast<int8_t*>(workspace);
+  st = launch_filter_flip_transpose(w, wt, K, R, S, C, s);
+  if (st != NITI_OK) return st;
+  const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
+  // fprop over the error map: "input" [N,P,Q,K], "filter" [C,R,S,K], padding R-1-pad -> [N,H,W,C]
+  ConvProblem p{err, wt, dx, absmax, N, P, Q, K, C, R, S, 1, R - 1 - pad,
+                static_cast<long long>(H) * W * C, static_cast<long long>(W) * C, C, 1, 1, flags};
+  return launch_conv_igemm(p, s);
+}
+
+extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad) {
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || pad < 0) return 0;
+  const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
+  if (P <= 0 || Q <= 0) return 0;
+  const size_t np = static_cast<size_t>(round16(N));
+  return round256(static_cast<size_t>(C) * H * W * np) + round256(static_cast<size_t>(K) * P * Q * np);
+}
+
+extern "C" int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int N, int H, int W, int C, int K,
+                                    int R, int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
+  clear_error();
+  int st = check_conv_dims("conv_wgrad", N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
+  if (act == nullptr || err == nullptr || dw == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_wgrad: null pointer");
+  if (stride != 1) return fail(NITI_ERR_UNSUPPORTED, "conv_wgrad: stride %d (only 1)", stride);
+  const size_t need = niti_conv2d_i8_wgrad_workspace(N, H, W, C, K, R, S, pad);
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    return fail(NITI_ERR_WORKSPACE, "conv_wgrad: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
+  const int np = round16(N);
+  int8_t* act_t = static_cast<int8_t*>(workspace);                                 // [C][H*W][np]
+  int8_t* err_t = act_t + round256(static_cast<size_t>(C) * H * W * np);           // [K][P*Q][np]
+  st = launch_transpose_outer_inner_i8(act, act_t, N, H * W, C, np, s);
+  if (st != NITI_OK) return st;
+  st = launch_transpose_outer_inner_i8(err, err_t, N, P * Q, K, np, s);
+  if (st != NITI_OK) return st;
+  const int64_t nout = static_cast<int64_t>(K) * R * S * C;
+  st = launch_fill_u32(reinterpret_cast<uint32_t*>(dw), nout, 0u, s);
+  if (st != NITI_OK) return st;
+  // The batch index becomes the reduction ("channel") index: images = C, filters = K, the
+  // error map plays the filter window; output (c, r, s, k) is scattered to dw[k][r][s][c].
+  const long long tiles = ((static_cast<long long>(C) * R * S + 127) / 128) * ((K + 127) / 128);
+  const long long kg = static_cast<long long>(P) * Q * np;
+  const int kiters = static_cast<int>((kg + 63) / 64);
+  int split = pick_split(tiles, kiters);
+  if (split < 2) split = 2;  // the scatter store path is the split-k one
+  ConvProblem p{act_t, err_t, dw, nullptr, C, H, W, np, K, P, Q, 1, pad,
+                1, static_cast<long long>(S) * C, C, static_cast<long long>(R) * S * C, split, 0u};
+  st = launch_conv_igemm(p, s);
+  if (st != NITI_OK) return st;
+  return launch_post_i32(dw, nout, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, absmax, s);
+}
+
+extern "C" size_t niti_gemm_i8_workspace(int trans_a, int trans_b, int m, int n, int k) {
+  if (m <= 0 || n <= 0 || k <= 0) return 0;
+  const size_t kp = static_cast<size_t>(round16(k));
+  size_t bytes = 0;
+  if (trans_a || k % 16 != 0) bytes += round256(static_cast<size_t>(m) * kp);
+  if (!trans_b || k % 16 != 0) bytes += round256(static_cast<size_t>(n) * kp);
+  return bytes;
+}
+
+extern "C" int niti_gemm_i8(int trans_a, int trans_b, const int8_t* a, const int8_t* b, int32_t* c, int m, int n, int k,
+                            unsigned flags, uint32_t* absmax, void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  if (m <= 0 || n <= 0 || k <= 0) return fail(NITI_ERR_INVALID_ARG, "gemm: non-positive extent (m=%d n=%d k=%d)", m, n, k);
+  if (a == nullptr || b == nullptr || c == nullptr) return fail(NITI_ERR_INVALID_ARG, "gemm: null pointer");
+  if (!aligned16(c)) return fail(NITI_ERR_INVALID_ARG, "gemm: output must be 16-byte aligned");
+  const size_t need = niti_gemm_i8_workspace(trans_a, trans_b, m, n, k);
+  if (need > 0 && (workspace == nullptr || workspace_bytes < need || !aligned16(workspace)))
+    return fail(NITI_ERR_WORKSPACE, "gemm: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int kp = round16(k);
+  int8_t* ws = static_cast<int8_t*>(workspace);
+  const int8_t* a_use = a;  // [m][kp]
+  const int8_t* b_use = b;  // [n][kp]
+  int st;
+  if (trans_a) {
+    st = launch_transpose_outer_inner_i8(a, ws, k, 1, m, kp, s);  // [k][m] -> [m][kp]
+    if (st != NITI_OK) return st;
+    a_use = ws;
+    ws += round256(static_cast<size_t>(m) * kp);
+  } else if (kp != k) {
+    hipLaunchKernelGGL(pad_rows_i8_kernel, dim3(1024), dim3(256), 0, s, a, ws, static_cast<int64_t>(m), k, kp);
+    if ((st = check_launch("pad_rows")) != NITI_OK) return st;
+    a_use = ws;
+    ws += round256(static_cast<size_t>(m) * kp);
+  }
+  if (!trans_b) {
+    st = launch_transpose_outer_inner_i8(b, ws, k, 1, n, kp, s);  // [k][n] -> [n][kp]
+    if (st != NITI_OK) return st;
+    b_use = ws;
+  } else if (kp != k) {
+    hipLaunchKernelGGL(pad_rows_i8_kernel, dim3(1024), dim3(256), 0, s, b, ws, static_cast<int64_t>(n), k, kp);
+    if ((st = check_launch("pad_rows")) != NITI_OK) return st;
+    b_use = ws;
+  }
+  if (!aligned16(a_use) || !aligned16(b_use)) return fail(NITI_ERR_INVALID_ARG, "gemm: operands must be 16-byte aligned");
+  // a 1x1 convolution over an m x 1 x 1 "image" with kp channels and n filters
+  ConvProblem p{a_use, b_use, c, absmax, m, 1, 1, kp, n, 1, 1, 1, 0, n, n, n, 1, 1, flags};
+  return launch_conv_igemm(p, s);
+}

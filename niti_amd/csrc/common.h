@@ -1,0 +1,101 @@
+// Shared declarations of the gfx950 library: status plumbing, vector types, small device helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "niti_gfx950.h"
+
+namespace niti {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v2i __attribute__((ext_vector_type(2)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+// Records a message for niti_last_error() and returns `status`.
+int fail(int status, const char* fmt, ...);
+void clear_error();
+
+inline int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) return fail(NITI_ERR_LAUNCH, "%s: %s", what, hipGetErrorString(e));
+  return NITI_OK;
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+__device__ inline bool aligned16_dev(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+// ceil(log2(r)) as integer arithmetic (0 for r <= 1)
+__host__ __device__ inline int bitwidth_exact(uint32_t r) {
+  if (r <= 1) return 0;
+  uint32_t v = r - 1;
+#if defined(__HIP_DEVICE_COMPILE__)
+  return 32 - __clz(v);
+#else
+  return 32 - __builtin_clz(v);
+#endif
+}
+
+// int(ceil(log2f((float)r))) under a correctly rounded log2f.  (float)r = 2^e * (1 + j*2^-23);
+// the sum e + log2(1 + j*2^-23) rounds back to e exactly when j is at most jmax(e): half an ulp
+// of e, expressed in mantissa steps (0, 0, 1, 2, 5 for e in [1,2), [2,4), [4,8), [8,16), [16,32)).
+__host__ __device__ inline int bitwidth_float32(uint32_t r) {
+  if (r == 0) return 0;
+  float f = static_cast<float>(r);  // round to nearest even
+  union { float f; uint32_t u; } cvt;
+  cvt.f = f;
+  const int e = static_cast<int>((cvt.u >> 23) & 0xFF) - 127;
+  const uint32_t j = cvt.u & 0x7FFFFFu;
+  if (j == 0) return e;
+  if (e <= 0) return e + 1;
+  int t = 0;
+  for (int v = e; v > 1; v >>= 1) ++t;
+  const uint32_t jmax = t >= 4 ? 5u : (t == 3 ? 2u : (t == 2 ? 1u : 0u));
+  return j <= jmax ? e : e + 1;
+}
+
+__host__ __device__ inline int bitwidth_of(uint32_t r, int bw_mode) {
+  return bw_mode == NITI_BW_F32 ? bitwidth_float32(r) : bitwidth_exact(r);
+}
+
+// int32 -> fp32 (round to nearest even) -> int32 with saturation: the reference's CUTLASS
+// LinearCombinationClamp<int32, 4, int32, float> epilogue with alpha = 1, beta = 0.
+__device__ inline int f32_roundtrip(int v) {
+  const float f = static_cast<float>(v);
+  if (f >= 2147483648.0f) return 2147483647;
+  return static_cast<int>(f);  // f is integral and >= -2^31 here
+}
+
+__device__ inline uint32_t uabs(int v) { return v < 0 ? 0u - static_cast<uint32_t>(v) : static_cast<uint32_t>(v); }
+
+__device__ inline uint32_t wave_max_u32(uint32_t v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    uint32_t o = __shfl_xor(v, off, 64);
+    v = o > v ? o : v;
+  }
+  return v;
+}
+
+// ---- launchers implemented in the .hip files ----
+struct ConvProblem {
+  const int8_t* x;   // [N,H,W,C]
+  const int8_t* w;   // [K,R,S,C]
+  int32_t* y;        // element (n,p,q,k) lives at n*ysN + p*ysP + q*ysQ + k*ysK
+  uint32_t* absmax;  // may be null
+  int N, H, W, C, K, R, S, stride, pad;
+  long long ysN, ysP, ysQ, ysK;
+  int split_k;       // 1: plain stores; >1: k-range split, int32 atomic adds into zeroed y
+  unsigned flags;
+};
+int launch_conv_igemm(const ConvProblem& p, hipStream_t stream);
+
+int launch_fill_u32(uint32_t* dst, int64_t n, uint32_t value, hipStream_t stream);
+// dst[c][r][s][k] = w[k][R-1-r][S-1-s][c]
+int launch_filter_flip_transpose(const int8_t* w, int8_t* dst, int K, int R, int S, int C, hipStream_t stream);
+// src [A][B][C] int8 -> dst [C][B][Apad], zero filled for a >= A
+int launch_transpose_outer_inner_i8(const int8_t* src, int8_t* dst, int A, int B, int C, int Apad, hipStream_t stream);
+// in place: v = roundtrip(v) if requested; absmax folded if non-null
+int launch_post_i32(int32_t* v, int64_t n, bool roundtrip, uint32_t* absmax, hipStream_t stream);
+
+}  // namespace niti

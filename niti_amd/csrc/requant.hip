@@ -1,0 +1,281 @@
+// Integer requantisation kernels: per-tensor max |x|, shift-round-clip back to int8 (nearest,
+// stochastic with supplied random integers, pseudo-stochastic), the fused gradient rounding +
+// weight update, ReLU forward/backward.  All are single-pass HBM-bandwidth kernels that move
+// 16 int32 (64 bytes in, 16 bytes out) per thread per step; the shift is derived on the
+// device from the max the producer kernel left in memory.
+#include "common.h"
+
+namespace niti {
+namespace {
+
+__device__ inline int clip127(long long v) { return static_cast<int>(v > 127 ? 127 : (v < -127 ? -127 : v)); }
+
+// quotient and magnitude of the remainder of x / 2^s: floor division or truncation
+__device__ inline void split_pow2(long long x, int s, bool trunc, long long& q, long long& rem) {
+  if (!trunc || x >= 0) {
+    q = x >> s;
+    rem = x - (q << s);
+  } else {
+    const long long m = -x;
+    q = -(m >> s);
+    rem = m & ((1LL << s) - 1);
+  }
+}
+
+template <int kMethod>
+__device__ inline int round_one(int x, int s, bool trunc, int u) {
+  if (kMethod == NITI_ROUND_NEAREST) {
+    const long long half = 1LL << (s - 1);
+    if (!trunc) return clip127((static_cast<long long>(x) + half) >> s);
+    const long long m = x < 0 ? -static_cast<long long>(x) : static_cast<long long>(x);
+    const long long q = (m + half) >> s;
+    return clip127(x < 0 ? -q : q);
+  }
+  long long q, rem;
+  split_pow2(x, s, trunc, q, rem);
+  const int sg = (x > 0) - (x < 0);
+  if (kMethod == NITI_ROUND_STOCHASTIC) return clip127(q + (rem > static_cast<long long>(u) ? sg : 0));
+  const int h = s >> 1;
+  const long long hi = rem >> h;
+  long long lo = rem & ((1LL << h) - 1);
+  if (s & 1) lo <<= 1;
+  return clip127(q + (hi > lo ? sg : 0));
+}
+
+__global__ __launch_bounds__(256) void absmax_i32_kernel(const int32_t* __restrict__ x, int64_t n, uint32_t* absmax) {
+  const int64_t nv = n >> 2;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  uint32_t lmax = 0;
+  const v4i* xv = reinterpret_cast<const v4i*>(x);
+  for (int64_t i = t0; i < nv; i += stride) {
+    const v4i v = xv[i];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const uint32_t u = uabs(v[e]);
+      lmax = u > lmax ? u : lmax;
+    }
+  }
+  for (int64_t i = (nv << 2) + t0; i < n; i += stride) {
+    const uint32_t u = uabs(x[i]);
+    lmax = u > lmax ? u : lmax;
+  }
+  lmax = wave_max_u32(lmax);
+  if ((threadIdx.x & 63) == 0 && lmax != 0) atomicMax(absmax, lmax);
+}
+
+struct RequantArgs {
+  const int32_t* x;
+  int8_t* y;        // requant: output.  grad update: optional rounded gradient
+  int8_t* w;        // grad update only
+  const int32_t* rand;
+  const uint32_t* absmax;
+  int32_t* shift_out;
+  int64_t n;
+  int target_bits, trunc, bw_mode;
+  unsigned flags;
+};
+
+// kUpdate == false: y = requant(x).  kUpdate == true: g = requant(x); w = clip(w - g); y (optional) = g
+template <int kMethod, bool kUpdate>
+__global__ __launch_bounds__(256) void requant_kernel(const RequantArgs a) {
+  const int shift = bitwidth_of(*a.absmax, a.bw_mode) - a.target_bits;
+  if (a.shift_out != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *a.shift_out = shift > 0 ? shift : 0;
+  const bool trunc = a.trunc != 0;
+  const bool relu = (a.flags & NITI_RQ_RELU) != 0;
+  auto one = [&](int x, int u) -> int {
+    int r;
+    if (shift >= 1) r = round_one<kMethod>(x, shift, trunc, u);
+    else r = static_cast<int>(static_cast<int8_t>(static_cast<uint32_t>(x) & 0xFFu));
+    if (relu && r < 0) r = 0;
+    return r;
+  };
+  const int64_t nv = a.n >> 4;  // groups of 16 elements
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const v4i* xv = reinterpret_cast<const v4i*>(a.x);
+  const v4i* uv = reinterpret_cast<const v4i*>(a.rand);
+  for (int64_t i = t0; i < nv; i += stride) {
+    v4i out;
+    v4i wv = {0, 0, 0, 0};
+    if (kUpdate) wv = reinterpret_cast<const v4i*>(a.w)[i];
+    v4i neww;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      const v4i v = xv[i * 4 + d];
+      v4i u = {0, 0, 0, 0};
+      if (kMethod == NITI_ROUND_STOCHASTIC && shift >= 1) u = uv[i * 4 + d];
+      uint32_t packed = 0, packedw = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int r = one(v[e], u[e]);
+        packed |= (static_cast<uint32_t>(r) & 0xFFu) << (8 * e);
+        if (kUpdate) {
+          const int wold = static_cast<int>(static_cast<int8_t>((static_cast<uint32_t>(wv[d]) >> (8 * e)) & 0xFFu));
+          packedw |= (static_cast<uint32_t>(clip127(wold - r)) & 0xFFu) << (8 * e);
+        }
+      }
+      out[d] = static_cast<int>(packed);
+      neww[d] = static_cast<int>(packedw);
+    }
+    if (kUpdate) {
+      reinterpret_cast<v4i*>(a.w)[i] = neww;
+      if (a.y != nullptr) reinterpret_cast<v4i*>(a.y)[i] = out;
+    } else {
+      reinterpret_cast<v4i*>(a.y)[i] = out;
+    }
+  }
+  for (int64_t i = (nv << 4) + t0; i < a.n; i += stride) {
+    int u = 0;
+    if (kMethod == NITI_ROUND_STOCHASTIC && shift >= 1) u = a.rand[i];
+    const int r = one(a.x[i], u);
+    if (kUpdate) {
+      a.w[i] = static_cast<int8_t>(clip127(static_cast<int>(a.w[i]) - r));
+      if (a.y != nullptr) a.y[i] = static_cast<int8_t>(r);
+    } else {
+      a.y[i] = static_cast<int8_t>(r);
+    }
+  }
+}
+
+__global__ __launch_bounds__(256) void weight_update_kernel(int8_t* w, const int8_t* __restrict__ g, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride)
+    w[i] = static_cast<int8_t>(clip127(static_cast<int>(w[i]) - static_cast<int>(g[i])));
+}
+
+// kBwd == false: y = max(x, 0).  kBwd == true: y = x(act) > 0 ? dy : 0
+template <bool kBwd>
+__global__ __launch_bounds__(256) void relu_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ dy,
+                                                   int8_t* __restrict__ y, int64_t n) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const bool vec = aligned16_dev(x) && aligned16_dev(y) && (!kBwd || aligned16_dev(dy));
+  const int64_t nv = vec ? (n >> 4) : 0;
+  for (int64_t i = t0; i < nv; i += stride) {
+    const v4i xv = reinterpret_cast<const v4i*>(x)[i];
+    v4i dv = {0, 0, 0, 0};
+    if (kBwd) dv = reinterpret_cast<const v4i*>(dy)[i];
+    v4i o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {
+      uint32_t p = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int xe = static_cast<int8_t>((static_cast<uint32_t>(xv[d]) >> (8 * e)) & 0xFFu);
+        const uint32_t src = kBwd ? ((static_cast<uint32_t>(dv[d]) >> (8 * e)) & 0xFFu) : (static_cast<uint32_t>(xe) & 0xFFu);
+        p |= (xe > 0 ? src : 0u) << (8 * e);
+      }
+      o[d] = static_cast<int>(p);
+    }
+    reinterpret_cast<v4i*>(y)[i] = o;
+  }
+  for (int64_t i = (nv << 4) + t0; i < n; i += stride) y[i] = x[i] > 0 ? (kBwd ? dy[i] : x[i]) : static_cast<int8_t>(0);
+}
+
+inline int grid_for(int64_t work_items, int block, int cap = 4096) {
+  int64_t g = (work_items + block - 1) / block;
+  if (g < 1) g = 1;
+  return static_cast<int>(g > cap ? cap : g);
+}
+
+template <bool kUpdate>
+int launch_requant(const RequantArgs& a, int method, hipStream_t stream) {
+  const dim3 grid(grid_for((a.n + 15) / 16, 256)), block(256);
+  switch (method) {
+    case NITI_ROUND_NEAREST:
+      hipLaunchKernelGGL((requant_kernel<NITI_ROUND_NEAREST, kUpdate>), grid, block, 0, stream, a);
+      break;
+    case NITI_ROUND_STOCHASTIC:
+      hipLaunchKernelGGL((requant_kernel<NITI_ROUND_STOCHASTIC, kUpdate>), grid, block, 0, stream, a);
+      break;
+    case NITI_ROUND_PSEUDO_STOCHASTIC:
+      hipLaunchKernelGGL((requant_kernel<NITI_ROUND_PSEUDO_STOCHASTIC, kUpdate>), grid, block, 0, stream, a);
+      break;
+    default:
+      return fail(NITI_ERR_INVALID_ARG, "requant: unknown rounding method %d", method);
+  }
+  return check_launch("requant");
+}
+
+int check_requant_common(const char* who, const void* x, int64_t n, const uint32_t* absmax, int target_bits, int method,
+                         int div_mode, int bw_mode, const int32_t* rand) {
+  if (n < 0) return fail(NITI_ERR_INVALID_ARG, "%s: n=%lld", who, static_cast<long long>(n));
+  if (n == 0) return NITI_OK;
+  if (x == nullptr || absmax == nullptr) return fail(NITI_ERR_INVALID_ARG, "%s: null pointer", who);
+  if (!aligned16(x)) return fail(NITI_ERR_INVALID_ARG, "%s: input must be 16-byte aligned", who);
+  if (target_bits < 1 || target_bits > 7) return fail(NITI_ERR_INVALID_ARG, "%s: target_bits=%d outside 1..7", who, target_bits);
+  if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "%s: div_mode=%d", who, div_mode);
+  if (bw_mode != NITI_BW_INT && bw_mode != NITI_BW_F32) return fail(NITI_ERR_INVALID_ARG, "%s: bw_mode=%d", who, bw_mode);
+  if (method == NITI_ROUND_STOCHASTIC && (rand == nullptr || !aligned16(rand)))
+    return fail(NITI_ERR_INVALID_ARG, "%s: stochastic rounding needs a 16-byte aligned rand tensor", who);
+  return NITI_OK;
+}
+
+}  // namespace
+}  // namespace niti
+
+using namespace niti;
+
+extern "C" int niti_absmax_i32(const int32_t* x, int64_t n, uint32_t* absmax, void* stream) {
+  clear_error();
+  if (n < 0) return fail(NITI_ERR_INVALID_ARG, "absmax: n=%lld", static_cast<long long>(n));
+  if (n == 0) return NITI_OK;
+  if (x == nullptr || absmax == nullptr) return fail(NITI_ERR_INVALID_ARG, "absmax: null pointer");
+  if (!aligned16(x)) return fail(NITI_ERR_INVALID_ARG, "absmax: input must be 16-byte aligned");
+  hipLaunchKernelGGL(absmax_i32_kernel, dim3(grid_for((n + 3) / 4, 256, 2048)), dim3(256), 0,
+                     static_cast<hipStream_t>(stream), x, n, absmax);
+  return check_launch("absmax_i32");
+}
+
+extern "C" int niti_requant_i32_i8(const int32_t* x, int8_t* y, int64_t n, const uint32_t* absmax, int target_bits,
+                                   int method, int div_mode, int bw_mode, const int32_t* rand, unsigned flags,
+                                   int32_t* shift_out, void* stream) {
+  clear_error();
+  int st = check_requant_common("requant", x, n, absmax, target_bits, method, div_mode, bw_mode, rand);
+  if (st != NITI_OK || n == 0) return st;
+  if (y == nullptr || !aligned16(y)) return fail(NITI_ERR_INVALID_ARG, "requant: output must be non-null and 16-byte aligned");
+  RequantArgs a{x, y, nullptr, rand, absmax, shift_out, n, target_bits, div_mode == NITI_DIV_TRUNC, bw_mode, flags};
+  return launch_requant<false>(a, method, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int niti_grad_update_i8(const int32_t* g, int8_t* w, int64_t n, const uint32_t* absmax, int mu, int method,
+                                   int div_mode, int bw_mode, const int32_t* rand, int8_t* g8_out, int32_t* shift_out,
+                                   void* stream) {
+  clear_error();
+  int st = check_requant_common("grad_update", g, n, absmax, mu, method, div_mode, bw_mode, rand);
+  if (st != NITI_OK || n == 0) return st;
+  if (w == nullptr || !aligned16(w)) return fail(NITI_ERR_INVALID_ARG, "grad_update: weights must be non-null and 16-byte aligned");
+  if (g8_out != nullptr && !aligned16(g8_out)) return fail(NITI_ERR_INVALID_ARG, "grad_update: g8_out must be 16-byte aligned");
+  RequantArgs a{g, g8_out, w, rand, absmax, shift_out, n, mu, div_mode == NITI_DIV_TRUNC, bw_mode, 0u};
+  return launch_requant<true>(a, method, static_cast<hipStream_t>(stream));
+}
+
+extern "C" int niti_weight_update_i8(int8_t* w, const int8_t* g, int64_t n, void* stream) {
+  clear_error();
+  if (n < 0) return fail(NITI_ERR_INVALID_ARG, "weight_update: n=%lld", static_cast<long long>(n));
+  if (n == 0) return NITI_OK;
+  if (w == nullptr || g == nullptr) return fail(NITI_ERR_INVALID_ARG, "weight_update: null pointer");
+  hipLaunchKernelGGL(weight_update_kernel, dim3(grid_for(n, 256)), dim3(256), 0, static_cast<hipStream_t>(stream), w, g, n);
+  return check_launch("weight_update");
+}
+
+extern "C" int niti_relu_i8_fwd(const int8_t* x, int8_t* y, int64_t n, void* stream) {
+  clear_error();
+  if (n < 0) return fail(NITI_ERR_INVALID_ARG, "relu: n=%lld", static_cast<long long>(n));
+  if (n == 0) return NITI_OK;
+  if (x == nullptr || y == nullptr) return fail(NITI_ERR_INVALID_ARG, "relu: null pointer");
+  hipLaunchKernelGGL(relu_kernel<false>, dim3(grid_for((n + 15) / 16, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     x, static_cast<const int8_t*>(nullptr), y, n);
+  return check_launch("relu_fwd");
+}
+
+extern "C" int niti_relu_i8_bwd(const int8_t* act, const int8_t* dy, int8_t* dx, int64_t n, void* stream) {
+  clear_error();
+  if (n < 0) return fail(NITI_ERR_INVALID_ARG, "relu_bwd: n=%lld", static_cast<long long>(n));
+  if (n == 0) return NITI_OK;
+  if (act == nullptr || dy == nullptr || dx == nullptr) return fail(NITI_ERR_INVALID_ARG, "relu_bwd: null pointer");
+  hipLaunchKernelGGL(relu_kernel<true>, dim3(grid_for((n + 15) / 16, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     act, dy, dx, n);
+  return check_launch("relu_bwd");
+}

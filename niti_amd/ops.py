@@ -1,0 +1,204 @@
+"""Tensor-level front end of the C ABI: takes torch device tensors, allocates outputs and
+workspaces with the torch allocator, launches on torch's current stream.  Nothing here
+computes: every function is one (or a few) calls into libniti_gfx950.so."""
+from __future__ import annotations
+
+from typing import Optional, Tuple
+
+import torch
+
+from . import _lib as L
+
+
+def _stream(t: torch.Tensor):
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _chk_dev(*ts: torch.Tensor) -> None:
+    for t in ts:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise RuntimeError("niti_amd: tensor must live on the GPU")
+        if not t.is_contiguous():
+            raise RuntimeError("niti_amd: tensor must be contiguous")
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else t.data_ptr()
+
+
+def new_scalar_u32(device) -> torch.Tensor:
+    """Zeroed device scalar the kernels fold max|x| into (stored as int32 bits of a uint32)."""
+    return torch.zeros(1, dtype=torch.int32, device=device)
+
+
+def _flags(f32_epilogue: bool) -> int:
+    return L.EPI_F32_ROUNDTRIP if f32_epilogue else 0
+
+
+def conv2d_fprop(x, w, stride=1, padding=1, f32_epilogue=False, absmax: Optional[torch.Tensor] = None):
+    """x [N,H,W,C] int8, w [K,R,S,C] int8 -> [N,P,Q,K] int32."""
+    _chk_dev(x, w, absmax)
+    if x.dtype != torch.int8 or w.dtype != torch.int8:
+        raise RuntimeError("conv2d_fprop: int8 tensors expected")
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    if C2 != C:
+        raise RuntimeError("conv2d_fprop: channel mismatch %d vs %d" % (C, C2))
+    P = (H + 2 * padding - R) // stride + 1
+    Q = (W + 2 * padding - S) // stride + 1
+    y = torch.empty((N, max(P, 0), max(Q, 0), K), dtype=torch.int32, device=x.device)
+    st = L.lib().niti_conv2d_i8_fprop(_ptr(x), _ptr(w), _ptr(y), N, H, W, C, K, R, S, stride, padding,
+                                      _flags(f32_epilogue), _ptr(absmax), _stream(x))
+    L.check(st, "niti_conv2d_i8_fprop")
+    return y
+
+
+def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None):
+    """err [N,P,Q,K] int8, w [K,R,S,C] int8 -> dx [N,H,W,C] int32 (stride 1)."""
+    _chk_dev(err, w, absmax)
+    N, P, Q, K = err.shape
+    K2, R, S, C = w.shape
+    if K2 != K:
+        raise RuntimeError("conv2d_dgrad: channel mismatch")
+    H = P - 2 * padding + R - 1
+    W = Q - 2 * padding + S - 1
+    dx = torch.empty((N, H, W, C), dtype=torch.int32, device=err.device)
+    nbytes = L.lib().niti_conv2d_i8_dgrad_workspace(C, K, R, S)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=err.device)
+    st = L.lib().niti_conv2d_i8_dgrad(_ptr(err), _ptr(w), _ptr(dx), N, H, W, C, K, R, S, stride, padding,
+                                      _flags(f32_epilogue), _ptr(absmax), _ptr(ws), nbytes, _stream(err))
+    L.check(st, "niti_conv2d_i8_dgrad")
+    return dx
+
+
+def conv2d_wgrad(act, err, R, S, stride=1, padding=1, f32_epilogue=False, absmax=None):
+    """act [N,H,W,C] int8, err [N,P,Q,K] int8 -> dw [K,R,S,C] int32 (stride 1)."""
+    _chk_dev(act, err, absmax)
+    N, H, W, C = act.shape
+    K = err.shape[3]
+    dw = torch.empty((K, R, S, C), dtype=torch.int32, device=act.device)
+    nbytes = L.lib().niti_conv2d_i8_wgrad_workspace(N, H, W, C, K, R, S, padding)
+    ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=act.device)
+    st = L.lib().niti_conv2d_i8_wgrad(_ptr(act), _ptr(err), _ptr(dw), N, H, W, C, K, R, S, stride, padding,
+                                      _flags(f32_epilogue), _ptr(absmax), _ptr(ws), nbytes, _stream(act))
+    L.check(st, "niti_conv2d_i8_wgrad")
+    return dw
+
+
+def gemm(a, b, trans_a=False, trans_b=False, absmax=None, out=None):
+    """c[m,n] = op(a) @ op(b), int8 x int8 -> int32.  trans_a: a stored [k,m]; trans_b: b stored [n,k]."""
+    _chk_dev(a, b, absmax, out)
+    if a.dtype != torch.int8 or b.dtype != torch.int8:
+        raise RuntimeError("gemm: int8 tensors expected")
+    m, k = (a.shape[1], a.shape[0]) if trans_a else (a.shape[0], a.shape[1])
+    n, k2 = (b.shape[0], b.shape[1]) if trans_b else (b.shape[1], b.shape[0])
+    if k != k2:
+        raise RuntimeError("gemm: inner extents differ (%d vs %d)" % (k, k2))
+    c = out if out is not None else torch.empty((m, n), dtype=torch.int32, device=a.device)
+    nbytes = L.lib().niti_gemm_i8_workspace(int(trans_a), int(trans_b), m, n, k)
+    ws = torch.empty(nbytes, dtype=torch.int8, device=a.device) if nbytes else None
+    st = L.lib().niti_gemm_i8(int(trans_a), int(trans_b), _ptr(a), _ptr(b), _ptr(c), m, n, k, 0, _ptr(absmax),
+                              _ptr(ws), nbytes, _stream(a))
+    L.check(st, "niti_gemm_i8")
+    return c
+
+
+def absmax_i32(x, absmax=None):
+    _chk_dev(x, absmax)
+    if absmax is None:
+        absmax = new_scalar_u32(x.device)
+    st = L.lib().niti_absmax_i32(_ptr(x), x.numel(), _ptr(absmax), _stream(x))
+    L.check(st, "niti_absmax_i32")
+    return absmax
+
+
+def requant(x, absmax, target_bits=7, method="round", div_mode="floor", bw_mode="int", rand=None, relu=False,
+            shift_out=None):
+    """int32 -> int8 (act_calc / err_calc / grad_calc).  Returns (int8 tensor, device int32 shift)."""
+    _chk_dev(x, absmax, rand, shift_out)
+    if x.dtype != torch.int32:
+        raise RuntimeError("requant: int32 input expected")
+    if rand is not None and (rand.dtype != torch.int32 or rand.numel() != x.numel()):
+        raise RuntimeError("requant: rand must be int32 with one entry per element")
+    y = torch.empty(x.shape, dtype=torch.int8, device=x.device)
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=x.device)
+    st = L.lib().niti_requant_i32_i8(_ptr(x), _ptr(y), x.numel(), _ptr(absmax), target_bits, L.ROUND[method],
+                                     L.DIV[div_mode], L.BW[bw_mode], _ptr(rand), L.RQ_RELU if relu else 0,
+                                     _ptr(shift_out), _stream(x))
+    L.check(st, "niti_requant_i32_i8")
+    return y, shift_out
+
+
+def grad_update(g, w, absmax, mu, method="psto", div_mode="floor", bw_mode="int", rand=None, want_grad=False,
+                shift_out=None):
+    """Fused grad_calc + weight update, in place on w.  Returns (int8 grad or None, device shift)."""
+    _chk_dev(g, w, absmax, rand, shift_out)
+    if g.dtype != torch.int32 or w.dtype != torch.int8 or g.numel() != w.numel():
+        raise RuntimeError("grad_update: int32 grad and int8 weight of equal size expected")
+    g8 = torch.empty(w.shape, dtype=torch.int8, device=w.device) if want_grad else None
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=w.device)
+    st = L.lib().niti_grad_update_i8(_ptr(g), _ptr(w), g.numel(), _ptr(absmax), mu, L.ROUND[method], L.DIV[div_mode],
+                                     L.BW[bw_mode], _ptr(rand), _ptr(g8), _ptr(shift_out), _stream(g))
+    L.check(st, "niti_grad_update_i8")
+    return g8, shift_out
+
+
+def weight_update(w, g):
+    _chk_dev(w, g)
+    st = L.lib().niti_weight_update_i8(_ptr(w), _ptr(g), w.numel(), _stream(w))
+    L.check(st, "niti_weight_update_i8")
+    return w
+
+
+def relu_fwd(x):
+    _chk_dev(x)
+    y = torch.empty_like(x)
+    L.check(L.lib().niti_relu_i8_fwd(_ptr(x), _ptr(y), x.numel(), _stream(x)), "niti_relu_i8_fwd")
+    return y
+
+
+def relu_bwd(act, dy):
+    _chk_dev(act, dy)
+    dx = torch.empty_like(dy)
+    L.check(L.lib().niti_relu_i8_bwd(_ptr(act), _ptr(dy), _ptr(dx), dy.numel(), _stream(dy)), "niti_relu_i8_bwd")
+    return dx
+
+
+def maxpool_fwd(x, kernel_size=2, stride=2, padding=0):
+    _chk_dev(x)
+    if x.dtype != torch.int8:
+        raise RuntimeError("maxpool_fwd: int8 tensor expected")
+    N, H, W, C = x.shape
+    P = (H + 2 * padding - kernel_size) // stride + 1
+    Q = (W + 2 * padding - kernel_size) // stride + 1
+    y = torch.empty((N, max(P, 0), max(Q, 0), C), dtype=torch.int8, device=x.device)
+    st = L.lib().niti_maxpool_i8_fwd(_ptr(x), _ptr(y), N, H, W, C, kernel_size, stride, padding, _stream(x))
+    L.check(st, "niti_maxpool_i8_fwd")
+    return y
+
+
+def maxpool_bwd(y, dy, x, kernel_size=2, stride=2, padding=0, ties="first"):
+    _chk_dev(y, dy, x)
+    N, H, W, C = x.shape
+    dx = torch.empty_like(x)
+    st = L.lib().niti_maxpool_i8_bwd(_ptr(y), _ptr(dy), _ptr(x), _ptr(dx), N, H, W, C, kernel_size, stride, padding,
+                                     L.TIES[ties], _stream(x))
+    L.check(st, "niti_maxpool_i8_bwd")
+    return dx
+
+
+def group_conv_f32(x, w, stride, padding, dilation, groups):
+    _chk_dev(x, w)
+    N, H, W, C = x.shape
+    K, R, S, Cg = w.shape
+    P = (H + 2 * padding - dilation * (R - 1) - 1) // stride + 1
+    Q = (W + 2 * padding - dilation * (S - 1) - 1) // stride + 1
+    y = torch.empty((N, max(P, 0), max(Q, 0), K), dtype=torch.float32, device=x.device)
+    st = L.lib().niti_group_conv_i8_f32(_ptr(x), _ptr(w), _ptr(y), N, H, W, C, K, R, S, Cg, stride, padding, dilation,
+                                        groups, _stream(x))
+    L.check(st, "niti_group_conv_i8_f32")
+    return y

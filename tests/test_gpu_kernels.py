@@ -1,0 +1,272 @@
+"""GPU parity of every C-ABI entry point against the CPU oracle on seeded inputs (bit-exact)."""
+import sys
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print("[case]", *a, flush=True)
+    sys.stdout.flush()
+
+
+@pytest.fixture(scope="module")
+def dev():
+    assert torch.cuda.is_available(), "GPU tests need a GPU"
+    return torch.device("cuda:0")
+
+
+def ri8(g, *shape, lo=-127, hi=127):
+    return torch.randint(lo, hi + 1, shape, generator=g, dtype=torch.int8)
+
+
+CONV_CASES = [  # N,H,W,C,K,R,S,stride,pad
+    (1, 4, 4, 16, 16, 3, 3, 1, 1),
+    (2, 8, 8, 16, 32, 3, 3, 1, 1),
+    (3, 7, 9, 32, 40, 3, 3, 1, 1),       # ragged M and K
+    (2, 8, 8, 64, 128, 3, 3, 1, 1),
+    (2, 9, 9, 48, 130, 3, 3, 2, 1),      # stride 2, K not a multiple of 4... of 128
+    (2, 8, 8, 16, 10, 5, 5, 1, 2),       # K = 10: scalar store tail
+    (4, 16, 16, 128, 128, 3, 3, 1, 1),
+    (1, 6, 6, 80, 24, 1, 1, 1, 0),
+    (2, 6, 6, 16, 8, 3, 3, 1, 0),        # no padding
+    (8, 32, 32, 128, 128, 3, 3, 1, 1),
+    (2, 40, 40, 16, 16, 36, 36, 1, 1),   # filter wider than 32 (the reference's sp_conv case)
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv_fprop(dev, case):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    N, H, W, C, K, R, S, st, pad = case
+    _say("conv_fprop", case)
+    g = torch.Generator().manual_seed(100 + N + C + K)
+    x, w = ri8(g, N, H, W, C), ri8(g, K, R, S, C)
+    ref = po.conv2d_fprop_i32(x, w, st, pad)
+    am = ops.new_scalar_u32(dev)
+    y = ops.conv2d_fprop(x.to(dev), w.to(dev), st, pad, absmax=am)
+    torch.cuda.synchronize()
+    assert torch.equal(y.cpu(), ref)
+    assert int(am.cpu()) == po.absmax(ref)
+    y2 = ops.conv2d_fprop(x.to(dev), w.to(dev), st, pad, f32_epilogue=True)
+    assert torch.equal(y2.cpu(), po.f32_roundtrip(ref))
+
+
+def test_conv_fprop_f32_epilogue_rounds_large_sums(dev):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    _say("conv_fprop f32 epilogue, |acc| > 2^24")
+    # all +-127 operands and a long reduction: |acc| reaches 127*127*9*256 = 37.2M > 2^24
+    x = torch.full((1, 6, 6, 256), 127, dtype=torch.int8)
+    x[0, 2, 2, 0] = 126                      # odd sums so the round trip is visible
+    w = torch.full((16, 3, 3, 256), 127, dtype=torch.int8)
+    w[1] = -127
+    w[2, 0, 0, 5] = 1
+    ref = po.conv2d_fprop_i32(x, w)
+    assert int(ref.abs().max()) > 2 ** 24
+    rt = po.f32_roundtrip(ref)
+    assert not torch.equal(rt, ref)
+    y = ops.conv2d_fprop(x.to(dev), w.to(dev), 1, 1, f32_epilogue=True)
+    assert torch.equal(y.cpu(), rt)
+    y = ops.conv2d_fprop(x.to(dev), w.to(dev), 1, 1, f32_epilogue=False)
+    assert torch.equal(y.cpu(), ref)
+
+
+DGRAD_CASES = [(2, 8, 8, 16, 16, 3, 1), (2, 8, 8, 32, 48, 3, 1), (3, 7, 9, 40, 32, 3, 1), (2, 16, 16, 128, 128, 3, 1),
+               (2, 8, 8, 16, 32, 5, 2), (2, 8, 8, 24, 16, 3, 0), (2, 6, 6, 3, 16, 3, 1)]
+
+
+@pytest.mark.parametrize("case", DGRAD_CASES)
+def test_conv_dgrad(dev, case):
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, H, W, C, K, R, pad = case
+    _say("conv_dgrad", case)
+    g = torch.Generator().manual_seed(200 + C + K)
+    P, Q = H + 2 * pad - R + 1, W + 2 * pad - R + 1
+    e, w = ri8(g, N, P, Q, K), ri8(g, K, R, R, C)
+    ref = co.conv_dgrad(e, w, H, W, 1, pad)
+    if 2 * pad == R - 1:
+        assert torch.equal(ref, po.conv2d_dgrad_i32(e, w, 1, pad, f32_epilogue=False))
+    am = ops.new_scalar_u32(dev)
+    dx = ops.conv2d_dgrad(e.to(dev), w.to(dev), 1, pad, absmax=am)
+    assert torch.equal(dx.cpu(), ref)
+    assert int(am.cpu()) == po.absmax(ref)
+
+
+WGRAD_CASES = [(2, 8, 8, 16, 16, 3, 1), (16, 8, 8, 32, 48, 3, 1), (5, 7, 9, 40, 24, 3, 1), (32, 16, 16, 64, 128, 3, 1),
+               (4, 8, 8, 3, 16, 3, 1), (6, 8, 8, 16, 10, 5, 2), (3, 6, 6, 8, 8, 3, 0), (128, 8, 8, 16, 16, 3, 1)]
+
+
+@pytest.mark.parametrize("case", WGRAD_CASES)
+def test_conv_wgrad(dev, case):
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, H, W, C, K, R, pad = case
+    _say("conv_wgrad", case)
+    g = torch.Generator().manual_seed(300 + C + K)
+    P, Q = H + 2 * pad - R + 1, W + 2 * pad - R + 1
+    a, e = ri8(g, N, H, W, C), ri8(g, N, P, Q, K)
+    ref = co.conv_wgrad(a, e, R, R, 1, pad)
+    if 2 * pad == R - 1:
+        assert torch.equal(ref, po.conv2d_wgrad_i32(a, e, 1, pad, f32_epilogue=False))
+    am = ops.new_scalar_u32(dev)
+    dw = ops.conv2d_wgrad(a.to(dev), e.to(dev), R, R, 1, pad, absmax=am)
+    assert torch.equal(dw.cpu(), ref)
+    assert int(am.cpu()) == po.absmax(ref)
+
+
+GEMM_CASES = [(16, 16, 16), (128, 128, 64), (100, 10, 512), (7, 5, 3), (130, 70, 100), (128, 1024, 1024), (33, 12, 8192)]
+
+
+@pytest.mark.parametrize("mnk", GEMM_CASES)
+@pytest.mark.parametrize("ta,tb", [(False, True), (False, False), (True, False), (True, True)])
+def test_gemm(dev, mnk, ta, tb):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    m, n, k = mnk
+    _say("gemm", mnk, ta, tb)
+    g = torch.Generator().manual_seed(400 + m + n + k)
+    A, B = ri8(g, m, k), ri8(g, k, n)
+    ref = po.int8mm(A, B)
+    a = (A.t().contiguous() if ta else A).to(dev)
+    b = (B.t().contiguous() if tb else B).to(dev)
+    am = ops.new_scalar_u32(dev)
+    c = ops.gemm(a, b, ta, tb, absmax=am)
+    assert torch.equal(c.cpu(), ref)
+    assert int(am.cpu()) == po.absmax(ref)
+
+
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+@pytest.mark.parametrize("method", ["round", "psto", "sto"])
+def test_requant(dev, method, div_mode):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    g = torch.Generator().manual_seed(500)
+    for n, hi in [(1, 5), (15, 128), (16, 129), (4099, 300), (70001, 40000), (1 << 18, 3000000), (1000, 2 ** 31 - 1)]:
+        for tgt in (7, 5, 3):
+            _say("requant", method, div_mode, n, hi, tgt)
+            x = torch.randint(-hi, hi + 1, (n,), generator=g, dtype=torch.int64).to(torch.int32)
+            x[0] = hi
+            s = max(po.RangeEstimate(x) - tgt, 0)
+            u = torch.randint(0, 2 ** max(s, 1), (n,), generator=g, dtype=torch.int32)
+            if tgt == 7:
+                ref, e = po.act_calc(x, 0, method, div_mode, u)
+            else:
+                ref, e = po.grad_calc(x, tgt, method, div_mode, u)
+            xd = x.to(dev)
+            am = ops.absmax_i32(xd)
+            assert int(am.cpu()) == po.absmax(x)
+            y, sh = ops.requant(xd, am, tgt, method, div_mode, rand=u.to(dev) if method == "sto" else None)
+            assert torch.equal(y.cpu(), ref)
+            assert int(sh.cpu()) == e == s
+            yr, _ = ops.requant(xd, am, tgt, method, div_mode, rand=u.to(dev) if method == "sto" else None, relu=True)
+            assert torch.equal(yr.cpu(), ref.clamp(min=0))
+
+
+def test_requant_special_cases(dev, kat):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    _say("requant special cases")
+    for vals, want_shift in (([0, 0, 0, 0, 0], 0), ([128, -128, 127, 5, -3], 0), ([129, -129, 1, -1, 0], 1)):
+        x = torch.tensor(vals, dtype=torch.int32)
+        ref, e = po.act_calc(x, 0)
+        am = ops.absmax_i32(x.to(dev))
+        y, sh = ops.requant(x.to(dev), am, 7)
+        assert y.cpu().tolist() == ref.tolist() and int(sh.cpu()) == want_shift
+    # known-answer table through the kernel: fix the shift by planting the range in absmax
+    X = torch.tensor(kat["X"], dtype=torch.int32)
+    for mode in ("floor", "trunc"):
+        am = torch.tensor([2 ** 14], dtype=torch.int32, device=dev)   # bitwidth 14 -> shift 7
+        y, sh = ops.requant(X.to(dev), am, 7, "round", mode)
+        assert y.cpu().tolist() == kat[f"round_s7_{mode}"] and int(sh.cpu()) == 7
+        y, _ = ops.requant(X.to(dev), am, 7, "psto", mode)
+        assert y.cpu().tolist() == kat[f"psto_s7_{mode}"]
+    # bit-width evaluated the reference's float way inside the thin band above 2^22
+    x = torch.tensor([2 ** 22 + 2, -5, 77], dtype=torch.int32)
+    am = ops.absmax_i32(x.to(dev))
+    _, s_int = ops.requant(x.to(dev), am, 7, bw_mode="int")
+    _, s_f32 = ops.requant(x.to(dev), am, 7, bw_mode="f32")
+    assert int(s_int.cpu()) == 23 - 7 and int(s_f32.cpu()) == 22 - 7 == po.bitwidth_f32(2 ** 22 + 2) - 7
+
+
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+def test_grad_update_and_weight_update(dev, div_mode):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    g = torch.Generator().manual_seed(600)
+    for n in (7, 1152, 128 * 9 * 128 + 3):
+        for mu in (5, 4, 3):
+            for method in ("psto", "round"):
+                _say("grad_update", div_mode, n, mu, method)
+                gi = torch.randint(-900000, 900001, (n,), generator=g, dtype=torch.int32)
+                w = ri8(g, n)
+                g8, s = po.grad_calc(gi, mu, method, div_mode)
+                wref = po.weight_update(w, g8)
+                wd = w.to(dev)
+                am = ops.absmax_i32(gi.to(dev))
+                g8d, sh = ops.grad_update(gi.to(dev), wd, am, mu, method, div_mode, want_grad=True)
+                assert torch.equal(g8d.cpu(), g8) and torch.equal(wd.cpu(), wref) and int(sh.cpu()) == s
+                w2 = w.to(dev)
+                ops.weight_update(w2, g8.to(dev))
+                assert torch.equal(w2.cpu(), wref)
+
+
+def test_relu(dev):
+    from niti_amd import ops
+    g = torch.Generator().manual_seed(700)
+    for n in (5, 64, 100003):
+        _say("relu", n)
+        x, dy = ri8(g, n, lo=-128), ri8(g, n)
+        assert torch.equal(ops.relu_fwd(x.to(dev)).cpu(), x.clamp(min=0))
+        assert torch.equal(ops.relu_bwd(x.to(dev), dy.to(dev)).cpu(), torch.where(x > 0, dy, torch.zeros_like(dy)))
+
+
+POOL_CASES = [(2, 8, 8, 16, 2, 2, 0), (1, 6, 6, 5, 2, 2, 0), (2, 7, 7, 32, 3, 2, 1), (1, 5, 5, 3, 2, 1, 0),
+              (1, 9, 9, 16, 3, 3, 0), (8, 32, 32, 128, 2, 2, 0), (3, 7, 7, 16, 2, 2, 0)]
+
+
+@pytest.mark.parametrize("case", POOL_CASES)
+def test_maxpool(dev, case):
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    N, H, W, C, ks, st, pad = case
+    g = torch.Generator().manual_seed(800 + C)
+    for lo, hi in ((-128, 127), (-2, 2), (0, 1)):
+        _say("maxpool", case, lo, hi)
+        x = ri8(g, N, H, W, C, lo=lo, hi=hi)
+        yref = co.maxpool_fwd(x, ks, st, pad)
+        y = ops.maxpool_fwd(x.to(dev), ks, st, pad)
+        assert torch.equal(y.cpu(), yref)
+        dy = ri8(g, *yref.shape, lo=-30, hi=30)
+        for ties in ("first", "all"):
+            ref = co.maxpool_bwd(yref, dy, x, ks, st, pad, ties)
+            dx = ops.maxpool_bwd(y, dy.to(dev), x.to(dev), ks, st, pad, ties)
+            assert torch.equal(dx.cpu(), ref), ties
+
+
+def test_group_conv_first_layer_wgrad(dev):
+    """The reference's first-layer weight gradient (ti_torch.py:194-233) routed through the
+    group_conv stand-in gives the true weight gradient as float32."""
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    _say("group_conv")
+    g = torch.Generator().manual_seed(900)
+    N, H, W, C, K = 4, 8, 8, 3, 16
+    act, err = ri8(g, N, H, W, C), ri8(g, N, H, W, K)
+    # operand preparation exactly as conv2d_weight_int8 does it
+    go = err.permute(0, 3, 1, 2).contiguous().repeat(1, C, 1, 1)
+    go = go.contiguous().reshape(N * C * K, 1, H, W).permute(0, 2, 3, 1).contiguous()
+    inp = act.permute(0, 3, 1, 2).contiguous().reshape(1, N * C, H, W).permute(0, 2, 3, 1).contiguous()
+    out = ops.group_conv_f32(inp.to(dev), go.to(dev), 1, 1, 1, C * N).cpu()
+    gw = out.permute(0, 3, 1, 2)
+    gw = gw.view(N, gw.shape[1] // N, gw.shape[2], gw.shape[3]).sum(dim=0)
+    gw = gw.view(C, K, gw.shape[1], gw.shape[2]).transpose(0, 1).narrow(2, 0, 3).narrow(3, 0, 3)
+    gw = gw.permute(0, 2, 3, 1).contiguous()
+    assert gw.dtype == torch.float32
+    assert torch.equal(gw, po.conv2d_weight_int8(act, (K, 3, 3, C), err, 1, 1))
