@@ -72,8 +72,8 @@ int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y, int N, in
  * Data gradient, replaces the reference's fprop-on-flipped-weights rewrite
  * (TiConv2d.backward, ti_torch.py:403-405):
  *   dx[n,h,w,c] = sum_{r,s,k} err[n, h+pad-r, w+pad-s, k] * w[k,r,s,c]
- * err: [N,P,Q,K] int8, w: [K,R,S,C] int8, dx: [N,H,W,C] int32.  Like the reference it is
- * defined for stride 1 with 2*pad == R-1 == S-1 only; needs K % 16 == 0.
+ * err: [N,P,Q,K] int8, w: [K,R,S,C] int8, dx: [N,H,W,C] int32.  Stride 1 and R == S only (the
+ * reference's rewrite additionally needs 2*pad == R-1; here any pad <= R-1); needs K % 16 == 0.
  * Workspace: niti_conv2d_i8_dgrad_workspace() bytes (re-laid filter).
  */
 size_t niti_conv2d_i8_dgrad_workspace(int C, int K, int R, int S);
@@ -115,13 +115,20 @@ int niti_absmax_i32(const int32_t* x, int64_t n, uint32_t* absmax, void* stream)
  *   shift = bitwidth(*absmax) - target_bits
  *   shift >= 1: y = clip(round_method(x, shift), +-127)   else: y = low byte of x (128 wraps)
  *   *shift_out = max(shift, 0)                            (shift_out may be NULL)
+ *   *exp_out   = max(shift, 0) + *exp_a + *exp_b          (each of the three may be NULL)
+ * The last line is the exponent bookkeeping the reference does on the host: exp_in + shift
+ * with exp_in = act_in_exp + weight_exp (ti_torch.py:111,396), err_exp + weight_exp + shift
+ * (ti_torch.py:261,407), err_exp + grad_shift + act_in_exp (ti_torch.py:20).
  * target_bits = 7 for activations and errors, GRAD_BITWIDTH (5/4/3) for gradients.
- * rand: one int32 per element in [0, 2^shift), NITI_ROUND_STOCHASTIC only (stands in for the
- * reference's device torch.randint, ti_torch.py:41).
+ * rand: one int32 per element, NITI_ROUND_STOCHASTIC only (stands in for the reference's device
+ * torch.randint(0, 2^shift), ti_torch.py:41); only the low `shift` bits are used, so values
+ * already in [0, 2^shift) are taken as they are and wider uniform bits may be supplied when the
+ * host does not know the shift.
  */
 int niti_requant_i32_i8(const int32_t* x, int8_t* y, int64_t n, const uint32_t* absmax, int target_bits,
                         int method, int div_mode, int bw_mode, const int32_t* rand, unsigned flags,
-                        int32_t* shift_out, void* stream);
+                        int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                        void* stream);
 
 /*
  * UpdateWeight.weight_update (ti_torch.py:16-21) fused with grad_calc:
@@ -130,7 +137,7 @@ int niti_requant_i32_i8(const int32_t* x, int8_t* y, int64_t n, const uint32_t* 
  */
 int niti_grad_update_i8(const int32_t* g, int8_t* w, int64_t n, const uint32_t* absmax, int mu, int method,
                         int div_mode, int bw_mode, const int32_t* rand, int8_t* g8_out, int32_t* shift_out,
-                        void* stream);
+                        const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
 
 /* w = clip(int16(w) - int16(g), +-127)  (ti_torch.py:21) */
 int niti_weight_update_i8(int8_t* w, const int8_t* g, int64_t n, void* stream);

@@ -35,8 +35,8 @@ SIGNATURES = {
     "niti_gemm_i8_workspace": (_sz, [_i] * 5),
     "niti_gemm_i8": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _i, _u, _vp, _vp, _sz, _vp]),
     "niti_absmax_i32": (_i, [_vp, _i64, _vp, _vp]),
-    "niti_requant_i32_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _u, _vp, _vp]),
-    "niti_grad_update_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "niti_requant_i32_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _u, _vp, _vp, _vp, _vp, _vp]),
+    "niti_grad_update_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "niti_weight_update_i8": (_i, [_vp, _vp, _i64, _vp]),
     "niti_relu_i8_fwd": (_i, [_vp, _vp, _i64, _vp]),
     "niti_relu_i8_bwd": (_i, [_vp, _vp, _vp, _i64, _vp]),

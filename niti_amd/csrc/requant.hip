@@ -71,6 +71,9 @@ struct RequantArgs {
   const int32_t* rand;
   const uint32_t* absmax;
   int32_t* shift_out;
+  const int32_t* exp_a;
+  const int32_t* exp_b;
+  int32_t* exp_out;
   int64_t n;
   int target_bits, trunc, bw_mode;
   unsigned flags;
@@ -80,7 +83,16 @@ struct RequantArgs {
 template <int kMethod, bool kUpdate>
 __global__ __launch_bounds__(256) void requant_kernel(const RequantArgs a) {
   const int shift = bitwidth_of(*a.absmax, a.bw_mode) - a.target_bits;
-  if (a.shift_out != nullptr && blockIdx.x == 0 && threadIdx.x == 0) *a.shift_out = shift > 0 ? shift : 0;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    const int sh = shift > 0 ? shift : 0;
+    if (a.shift_out != nullptr) *a.shift_out = sh;
+    if (a.exp_out != nullptr)
+      *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+  }
+  // random integers are reduced to their low `shift` bits: values already in [0, 2^shift) pass
+  // unchanged, wider uniform bits become uniform in [0, 2^shift) without the host knowing shift
+  const int rm = shift >= 1 ? static_cast<int>((1u << (shift > 31 ? 31 : shift)) - 1u) : 0;
+  const v4i rmask = {rm, rm, rm, rm};
   const bool trunc = a.trunc != 0;
   const bool relu = (a.flags & NITI_RQ_RELU) != 0;
   auto one = [&](int x, int u) -> int {
@@ -104,7 +116,7 @@ __global__ __launch_bounds__(256) void requant_kernel(const RequantArgs a) {
     for (int d = 0; d < 4; ++d) {
       const v4i v = xv[i * 4 + d];
       v4i u = {0, 0, 0, 0};
-      if (kMethod == NITI_ROUND_STOCHASTIC && shift >= 1) u = uv[i * 4 + d];
+      if (kMethod == NITI_ROUND_STOCHASTIC && shift >= 1) u = uv[i * 4 + d] & rmask;
       uint32_t packed = 0, packedw = 0;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -127,7 +139,7 @@ __global__ __launch_bounds__(256) void requant_kernel(const RequantArgs a) {
   }
   for (int64_t i = (nv << 4) + t0; i < a.n; i += stride) {
     int u = 0;
-    if (kMethod == NITI_ROUND_STOCHASTIC && shift >= 1) u = a.rand[i];
+    if (kMethod == NITI_ROUND_STOCHASTIC && shift >= 1) u = a.rand[i] & rmask[0];
     const int r = one(a.x[i], u);
     if (kUpdate) {
       a.w[i] = static_cast<int8_t>(clip127(static_cast<int>(a.w[i]) - r));
@@ -230,24 +242,25 @@ extern "C" int niti_absmax_i32(const int32_t* x, int64_t n, uint32_t* absmax, vo
 
 extern "C" int niti_requant_i32_i8(const int32_t* x, int8_t* y, int64_t n, const uint32_t* absmax, int target_bits,
                                    int method, int div_mode, int bw_mode, const int32_t* rand, unsigned flags,
-                                   int32_t* shift_out, void* stream) {
+                                   int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                   void* stream) {
   clear_error();
   int st = check_requant_common("requant", x, n, absmax, target_bits, method, div_mode, bw_mode, rand);
   if (st != NITI_OK || n == 0) return st;
   if (y == nullptr || !aligned16(y)) return fail(NITI_ERR_INVALID_ARG, "requant: output must be non-null and 16-byte aligned");
-  RequantArgs a{x, y, nullptr, rand, absmax, shift_out, n, target_bits, div_mode == NITI_DIV_TRUNC, bw_mode, flags};
+  RequantArgs a{x, y, nullptr, rand, absmax, shift_out, exp_a, exp_b, exp_out, n, target_bits, div_mode == NITI_DIV_TRUNC, bw_mode, flags};
   return launch_requant<false>(a, method, static_cast<hipStream_t>(stream));
 }
 
 extern "C" int niti_grad_update_i8(const int32_t* g, int8_t* w, int64_t n, const uint32_t* absmax, int mu, int method,
                                    int div_mode, int bw_mode, const int32_t* rand, int8_t* g8_out, int32_t* shift_out,
-                                   void* stream) {
+                                   const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream) {
   clear_error();
   int st = check_requant_common("grad_update", g, n, absmax, mu, method, div_mode, bw_mode, rand);
   if (st != NITI_OK || n == 0) return st;
   if (w == nullptr || !aligned16(w)) return fail(NITI_ERR_INVALID_ARG, "grad_update: weights must be non-null and 16-byte aligned");
   if (g8_out != nullptr && !aligned16(g8_out)) return fail(NITI_ERR_INVALID_ARG, "grad_update: g8_out must be 16-byte aligned");
-  RequantArgs a{g, g8_out, w, rand, absmax, shift_out, n, mu, div_mode == NITI_DIV_TRUNC, bw_mode, 0u};
+  RequantArgs a{g, g8_out, w, rand, absmax, shift_out, exp_a, exp_b, exp_out, n, mu, div_mode == NITI_DIV_TRUNC, bw_mode, 0u};
   return launch_requant<true>(a, method, static_cast<hipStream_t>(stream));
 }
 

@@ -115,9 +115,10 @@ def absmax_i32(x, absmax=None):
 
 
 def requant(x, absmax, target_bits=7, method="round", div_mode="floor", bw_mode="int", rand=None, relu=False,
-            shift_out=None):
-    """int32 -> int8 (act_calc / err_calc / grad_calc).  Returns (int8 tensor, device int32 shift)."""
-    _chk_dev(x, absmax, rand, shift_out)
+            shift_out=None, exp_a=None, exp_b=None, exp_out=None):
+    """int32 -> int8 (act_calc / err_calc / grad_calc).  Returns (int8 tensor, device int32 shift).
+    exp_out (device int32), when given, receives shift + exp_a + exp_b."""
+    _chk_dev(x, absmax, rand, shift_out, exp_a, exp_b, exp_out)
     if x.dtype != torch.int32:
         raise RuntimeError("requant: int32 input expected")
     if rand is not None and (rand.dtype != torch.int32 or rand.numel() != x.numel()):
@@ -127,22 +128,23 @@ def requant(x, absmax, target_bits=7, method="round", div_mode="floor", bw_mode=
         shift_out = torch.empty(1, dtype=torch.int32, device=x.device)
     st = L.lib().niti_requant_i32_i8(_ptr(x), _ptr(y), x.numel(), _ptr(absmax), target_bits, L.ROUND[method],
                                      L.DIV[div_mode], L.BW[bw_mode], _ptr(rand), L.RQ_RELU if relu else 0,
-                                     _ptr(shift_out), _stream(x))
+                                     _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _stream(x))
     L.check(st, "niti_requant_i32_i8")
     return y, shift_out
 
 
 def grad_update(g, w, absmax, mu, method="psto", div_mode="floor", bw_mode="int", rand=None, want_grad=False,
-                shift_out=None):
+                shift_out=None, exp_a=None, exp_b=None, exp_out=None):
     """Fused grad_calc + weight update, in place on w.  Returns (int8 grad or None, device shift)."""
-    _chk_dev(g, w, absmax, rand, shift_out)
+    _chk_dev(g, w, absmax, rand, shift_out, exp_a, exp_b, exp_out)
     if g.dtype != torch.int32 or w.dtype != torch.int8 or g.numel() != w.numel():
         raise RuntimeError("grad_update: int32 grad and int8 weight of equal size expected")
     g8 = torch.empty(w.shape, dtype=torch.int8, device=w.device) if want_grad else None
     if shift_out is None:
         shift_out = torch.empty(1, dtype=torch.int32, device=w.device)
     st = L.lib().niti_grad_update_i8(_ptr(g), _ptr(w), g.numel(), _ptr(absmax), mu, L.ROUND[method], L.DIV[div_mode],
-                                     L.BW[bw_mode], _ptr(rand), _ptr(g8), _ptr(shift_out), _stream(g))
+                                     L.BW[bw_mode], _ptr(rand), _ptr(g8), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b),
+                                     _ptr(exp_out), _stream(g))
     L.check(st, "niti_grad_update_i8")
     return g8, shift_out
 

@@ -1,0 +1,72 @@
+"""Network container with the reference's ``ti_net.TiNet`` interface (ti_net.py:8-48)."""
+import collections
+
+import torch
+from torch.nn.modules import Module
+
+from . import ti_torch
+from .ti_loss import TiLoss
+
+
+class TiNet(Module):
+    def __init__(self):
+        super().__init__()
+        self.loss = TiLoss()
+
+    def fuse(self):
+        """Fold each TiReLU that directly follows a TiConv2d into that layer's requantisation."""
+        layers = list(self.forward_layers)
+        for a, b in zip(layers, layers[1:]):
+            if isinstance(a, ti_torch.TiConv2d) and isinstance(b, ti_torch.TiReLU):
+                a.fuse_relu = True
+                b.fused = True
+        return self
+
+    def forward(self, x):
+        """ti_net.py:17-23: float NCHW batch -> (int8 logits, exponent)."""
+        x_data, x_exp = ti_torch.TiFloatToInt8(x)
+        x_data = x_data.permute(0, 2, 3, 1).contiguous()
+        return self.forward_int8(x_data, x_exp)
+
+    def forward_int8(self, x_data, x_exp=0):
+        """Same as forward() for a batch that already is int8 NHWC with exponent ``x_exp``."""
+        self.out, self.out_exp = self.forward_layers((x_data, x_exp))
+        return self.out, self.out_exp
+
+    @property
+    def out_bits(self):
+        """ti_net.py:22 (computed on demand: it needs a device->host copy)."""
+        return ti_torch.RangeEstimate(self.out)
+
+    def backward(self, target, loss_rand=None):
+        """ti_net.py:25-32."""
+        x = self.loss(self.out, self.out_exp, target, loss_rand)
+        return self.backward_from(x)
+
+    def backward_from(self, x):
+        """Back-propagate a given (int8 error, exponent) pair through the layers in reverse."""
+        for layer in reversed(self.forward_layers):
+            if isinstance(layer, torch.nn.Sequential):
+                for block in reversed(layer):
+                    x = block.backward(x)
+            else:
+                x = layer.backward(x)
+        return x
+
+    def state_dict(self):
+        """ti_net.py:34-41: ``layers.<idx>.weight`` (int8) and ``layers.<idx>.weight_exp`` (0-d float)."""
+        state_dict = collections.OrderedDict()
+        for idx, l in enumerate(self.forward_layers):
+            if hasattr(l, "weight"):
+                prefix = "layers." + str(idx) + "."
+                state_dict[prefix + "weight"] = l.weight
+                state_dict[prefix + "weight_exp"] = l.weight_exp
+        return state_dict
+
+    def load_state_dict(self, state_dict):
+        """ti_net.py:43-48."""
+        for idx, l in enumerate(self.forward_layers):
+            if hasattr(l, "weight"):
+                prefix = "layers." + str(idx) + "."
+                l.weight = state_dict[prefix + "weight"].to(ti_torch.GPU).contiguous()
+                l.weight_exp = state_dict[prefix + "weight_exp"]

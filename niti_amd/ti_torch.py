@@ -1,0 +1,441 @@
+"""Integer layer library with the reference's ``ti_torch`` API (class and function names, tuple
+conventions ``(int8 tensor, exponent)``, module-level switches) on top of libniti_gfx950.so.
+
+Differences in mechanism, not in results:
+  * every requantisation is one device kernel that reads the tensor range the producing
+    conv/GEMM kernel left in device memory; shifts and exponents stay on the device as 1-element
+    int32 tensors, so a training step contains no host synchronisation (the reference
+    synchronises twice per requantisation, ti_torch.py:369-377);
+  * dgrad and wgrad are C-ABI entry points instead of flip/transpose/contiguous copies around the
+    forward convolution (ti_torch.py:404-405, 430-432);
+  * the weight gradient is rounded and applied to the weights in one pass (ti_torch.py:16-21).
+
+Switches (module globals, like the reference's ti_torch.py:457-464 plus the two that main.py
+injects): BITWIDTH, ACT_ROUND_METHOD, ERROR_ROUND_METHOD, GRAD_ROUND_METHOD, WEIGHT_INIT_METHOD,
+GPU, GRAD_BITWIDTH, TRAINING.  Added here: DIV_MODE ("floor" = meaning of ``//`` on torch >= 1.13,
+"trunc" = torch <= 1.12), BW_MODE ("int" exact ceil(log2) / "f32" the reference's float
+evaluation), F32_EPILOGUE (reproduce the CUTLASS int32->fp32->int32 epilogue), POOL_TIES.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+import torch.nn.functional as F
+from torch.nn.modules import Module
+
+from . import ops
+
+GPU = "cuda"
+BITWIDTH = 7
+GRAD_BITWIDTH = 5      # main.py:72-77 sets 5 -> 4 -> 3 over the epochs
+TRAINING = True        # main.py:146-149
+DIV_MODE = "floor"
+BW_MODE = "int"
+F32_EPILOGUE = True
+POOL_TIES = "first"
+
+
+# ------------------------------------------------------------------------------------------
+# small helpers
+# ------------------------------------------------------------------------------------------
+def _exp_tensor(e, device) -> torch.Tensor:
+    """Exponent as a 1-element int32 device tensor (accepts int, float, 0-d or 1-element tensors)."""
+    if isinstance(e, torch.Tensor):
+        return e.reshape(1).to(device=device, dtype=torch.int32)
+    return torch.tensor([int(e)], dtype=torch.int32, device=device)
+
+
+def _planted_absmax(shift: int, target_bits: int, device) -> torch.Tensor:
+    """A range whose bit-width is exactly target_bits + shift (so a kernel applies that shift)."""
+    bits = target_bits + int(shift)
+    if not 1 <= int(shift) or bits > 31:
+        raise ValueError("shift %d out of range" % shift)
+    return torch.tensor([2 ** (bits - 1) + 1], dtype=torch.int64, device=device).to(torch.int32)
+
+
+def _standalone(x: torch.Tensor, shift: int, method: str, rand=None) -> torch.Tensor:
+    x32 = x.to(torch.int32).contiguous()
+    am = _planted_absmax(shift, BITWIDTH, x32.device)
+    y, _ = ops.requant(x32, am, BITWIDTH, method, DIV_MODE, "int", rand)
+    return y
+
+
+def RoundShift(input, shift):
+    """ti_torch.py:23-31."""
+    return _standalone(input, shift, "round")
+
+
+def StoShift(input, shift, rand=None):
+    """ti_torch.py:33-46; ``rand`` (int32, one per element, in [0, 2**shift)) replaces the device
+    ``torch.randint`` when given."""
+    if rand is None:
+        rand = torch.randint(0, 2 ** shift, input.shape, dtype=torch.int32, device=input.device)
+    return _standalone(input, shift, "sto", rand.to(torch.int32).contiguous())
+
+
+def PstoShift(input, shift):
+    """ti_torch.py:48-69."""
+    return _standalone(input, shift, "psto")
+
+
+ACT_ROUND_METHOD = RoundShift
+ERROR_ROUND_METHOD = RoundShift
+GRAD_ROUND_METHOD = PstoShift
+
+
+def _method_name(fn) -> str:
+    if fn is RoundShift:
+        return "round"
+    if fn is StoShift:
+        return "sto"
+    if fn is PstoShift:
+        return "psto"
+    raise ValueError("rounding method must be RoundShift, StoShift or PstoShift")
+
+
+def _rand_bits_like(x: torch.Tensor) -> torch.Tensor:
+    """31 uniform random bits per element; the kernel keeps the low `shift` ones."""
+    return torch.randint(0, 2 ** 31 - 1, x.shape, dtype=torch.int32, device=x.device)
+
+
+def int8_clip(input, clip_val=127):
+    """ti_torch.py:71-72."""
+    return torch.clamp(input, -clip_val, clip_val).type(torch.int8)
+
+
+def Int8Tensor(val):
+    return torch.tensor(val, dtype=torch.int8).to(GPU)
+
+
+def Int8zeros(size):
+    return torch.zeros(size=size, dtype=torch.int8, device=GPU)
+
+
+def roundoff4(size):
+    return (size + 3) // 4 * 4
+
+
+# ------------------------------------------------------------------------------------------
+# range estimate and requantisation (ti_torch.py:103-147, 366-377)
+# ------------------------------------------------------------------------------------------
+def TensorBitwidth(val):
+    """ti_torch.py:366-367 (host value; synchronises)."""
+    from . import _lib
+    return int(_lib.lib().niti_bitwidth(int(val), _lib.BW[BW_MODE]))
+
+
+def RangeEstimate(input):
+    """ti_torch.py:369-377.  Returns a Python int like the reference, which costs a device->host
+    copy; the layers below never call it."""
+    am = ops.absmax_i32(input.to(torch.int32).contiguous())
+    return TensorBitwidth(int(am.item()) & 0xFFFFFFFF)
+
+
+def _requant(acc, target_bits, fn, absmax=None, rand=None, relu=False, exp_a=None, exp_b=None, want_exp=False):
+    acc = acc.contiguous()
+    if acc.dtype != torch.int32:
+        acc = acc.to(torch.int32)        # first-layer gradients arrive as integer-valued float32
+    if absmax is None:
+        absmax = ops.absmax_i32(acc)
+    method = _method_name(fn)
+    if method == "sto" and rand is None:
+        rand = _rand_bits_like(acc)
+    exp_out = torch.empty(1, dtype=torch.int32, device=acc.device) if want_exp else None
+    y, shift = ops.requant(acc, absmax, target_bits, method, DIV_MODE, BW_MODE, rand, relu,
+                           exp_a=exp_a, exp_b=exp_b, exp_out=exp_out)
+    return y, shift, exp_out
+
+
+def act_calc(int32_acc, exp_in, absmax=None, rand=None):
+    """ti_torch.py:103-117.  Returns (int8 tensor, exp_out) with exp_out a 1-element int32 device
+    tensor equal to exp_in + shift."""
+    e = _exp_tensor(exp_in, int32_acc.device)
+    y, _, exp_out = _requant(int32_acc, BITWIDTH, ACT_ROUND_METHOD, absmax, rand, exp_a=e, want_exp=True)
+    return y, exp_out
+
+
+def err_calc(int32_acc, absmax=None, rand=None):
+    """ti_torch.py:119-133.  Returns (int8 tensor, shift) with shift a 1-element int32 device tensor."""
+    y, shift, _ = _requant(int32_acc, BITWIDTH, ERROR_ROUND_METHOD, absmax, rand)
+    return y, shift
+
+
+def grad_calc(int32_acc, mu, absmax=None, rand=None):
+    """ti_torch.py:135-147."""
+    y, shift, _ = _requant(int32_acc, mu, GRAD_ROUND_METHOD, absmax, rand)
+    return y, shift
+
+
+# ------------------------------------------------------------------------------------------
+# op wrappers (ti_torch.py:152-233)
+# ------------------------------------------------------------------------------------------
+def int8mm(lhs, rhs):
+    """ti_torch.py:152-176: [m,k] x [k,n] -> contiguous int32 [m,n] (any m, n, k)."""
+    return ops.gemm(lhs.contiguous(), rhs.contiguous())
+
+
+def _pad_channels16(t):
+    c = t.size(3)
+    return t if c % 16 == 0 else F.pad(t, (0, 16 - c % 16), "constant", 0)
+
+
+def conv2d_int8(input, weight, stride=1, padding=1, absmax=None):
+    """ti_torch.py:178-192: NHWC int8 x KRSC int8 -> NPQK int32."""
+    return ops.conv2d_fprop(_pad_channels16(input).contiguous(), _pad_channels16(weight).contiguous(), stride, padding,
+                            f32_epilogue=F32_EPILOGUE, absmax=absmax)
+
+
+def conv2d_weight_int8(input, weight_size, grad_output, stride=1, padding=0, dilation=1):
+    """ti_torch.py:194-233: first-layer weight gradient, returned like the reference as an
+    integer-valued float32 KRSC tensor."""
+    if stride != 1 or dilation != 1:
+        raise RuntimeError("conv2d_weight_int8: only stride 1, dilation 1 (as guarded in the reference, ti_torch.py:413)")
+    dw = ops.conv2d_wgrad(input.contiguous(), grad_output.contiguous(), weight_size[1], weight_size[2], stride, padding)
+    return dw.float()
+
+
+# ------------------------------------------------------------------------------------------
+# quantisers / initialisers (ti_torch.py:77-99, 334-364)
+# ------------------------------------------------------------------------------------------
+def weight_quant(input):
+    """ti_torch.py:334-339.  Returns (int8 weights on the GPU, exponent as a 0-d float tensor)."""
+    input_range = torch.max(torch.abs(input))
+    input_bitwidth = torch.ceil(torch.log2(input_range))
+    act_exp = input_bitwidth - 7
+    round_val = torch.round(input / input_range * (2 ** 7 - 1)).type(torch.int8).to(GPU)
+    return round_val, act_exp
+
+
+def UniformWeights(size):
+    """ti_torch.py:77-85 (Xavier-uniform drawn in KCRS, stored KRSC)."""
+    if len(size) == 4:
+        temp = torch.zeros(size).permute(0, 3, 1, 2).contiguous()
+        torch.nn.init.xavier_uniform_(temp)
+        return weight_quant(temp.permute(0, 2, 3, 1).contiguous())
+    temp = torch.zeros(size)
+    torch.nn.init.xavier_uniform_(temp)
+    return weight_quant(temp)
+
+
+def NormalWeight(size):
+    """ti_torch.py:87-95."""
+    if len(size) == 4:
+        temp = torch.zeros(size).permute(0, 3, 1, 2).contiguous()
+        torch.nn.init.xavier_normal_(temp)
+        return weight_quant(temp.permute(0, 2, 3, 1).contiguous())
+    temp = torch.zeros(size)
+    torch.nn.init.xavier_normal_(temp)
+    return weight_quant(temp)
+
+
+WEIGHT_INIT_METHOD = UniformWeights
+
+
+def TiFloatToInt8(input):
+    """ti_torch.py:341-356: float tensor -> (int8 tensor on the GPU, exponent).  The exponent is
+    returned as a 0-d float tensor like the reference; no host synchronisation."""
+    input = input.to(GPU)
+    input_range = torch.max(torch.abs(input))
+    input_bitwidth = torch.ceil(torch.log2(input_range))
+    act_exp = input_bitwidth - BITWIDTH
+    norm_val = input * (2 ** (BITWIDTH - input_bitwidth))
+    round_val = torch.round(norm_val)
+    clamp_val = torch.clamp(round_val, -128, 127).type(torch.int8)
+    return clamp_val, act_exp
+
+
+def TiInt8ToFloat(input):
+    """ti_torch.py:358-364."""
+    act_in, exp_in = input
+    if not isinstance(exp_in, torch.Tensor):
+        exp_in = torch.tensor(float(exp_in), device=act_in.device)
+    return act_in.float() * (2 ** (exp_in.float().reshape(())))
+
+
+# ------------------------------------------------------------------------------------------
+# layers
+# ------------------------------------------------------------------------------------------
+class UpdateWeight(Module):
+    """ti_torch.py:11-21: vanilla integer SGD shared by TiConv2d and TiLinear.  grad_calc and the
+    saturating subtraction run as one kernel; ``self.grad`` (the rounded int8 gradient) is kept only
+    when ``keep_grad`` is set."""
+    keep_grad = False
+
+    def _init_weight(self, size):
+        w, e = WEIGHT_INIT_METHOD(size)
+        self.weight = w.to(GPU).contiguous()
+        self.weight_exp = e if isinstance(e, torch.Tensor) else torch.tensor(float(e))
+
+    def _wexp(self):
+        return _exp_tensor(self.weight_exp, self.weight.device)
+
+    def weight_update(self, absmax=None, rand=None):
+        g = self.grad_int32acc
+        if g.dtype != torch.int32:
+            g = g.to(torch.int32)
+        g = g.contiguous()
+        if absmax is None:
+            absmax = ops.absmax_i32(g)
+        method = _method_name(GRAD_ROUND_METHOD)
+        if method == "sto" and rand is None:
+            rand = _rand_bits_like(g)
+        self.grad_exp = torch.empty(1, dtype=torch.int32, device=g.device)
+        if not self.weight.is_contiguous():
+            self.weight = self.weight.contiguous()
+        self.grad, self.grad_shift = ops.grad_update(
+            g, self.weight, absmax, GRAD_BITWIDTH, method, DIV_MODE, BW_MODE, rand, want_grad=self.keep_grad,
+            exp_a=_exp_tensor(self.err_exp, g.device), exp_b=_exp_tensor(self.act_in_exp, g.device), exp_out=self.grad_exp)
+
+
+class TiConv2d(UpdateWeight):
+    """ti_torch.py:379-437: int8 convolution layer, NHWC activations, KRSC weights.
+    ``fuse_relu`` folds the following TiReLU's forward into the activation requantisation."""
+
+    def __init__(self, in_channels, out_channels, kernel_size=3, stride=1, padding=1, first_layer=False):
+        super().__init__()
+        self._init_weight(torch.Size([out_channels, kernel_size, kernel_size, in_channels]))
+        self.first_layer = first_layer
+        self.stride = stride
+        self.padding = padding
+        self.fuse_relu = False
+
+    def forward(self, input, rand=None):
+        self.act, self.act_in_exp = input
+        dev = self.act.device
+        am = ops.new_scalar_u32(dev)
+        acc = conv2d_int8(self.act, self.weight, self.stride, self.padding, absmax=am)
+        act_out, _, exp_out = _requant(acc, BITWIDTH, ACT_ROUND_METHOD, am, rand, relu=self.fuse_relu,
+                                       exp_a=_exp_tensor(self.act_in_exp, dev), exp_b=self._wexp(), want_exp=True)
+        return act_out, exp_out
+
+    def backward(self, input, rand=None, grad_rand=None):
+        err_in, err_exp = input
+        err_in = err_in.contiguous()
+        dev = err_in.device
+        self.err_exp_in = _exp_tensor(err_exp, dev)
+        self.err_exp = self.err_exp_in
+        if not self.first_layer:
+            # data gradient with the weights as they were in the forward pass
+            am = ops.new_scalar_u32(dev)
+            dx = ops.conv2d_dgrad(err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
+            err_out, _, new_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
+                                           exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
+            self.err_exp = new_exp
+        amg = ops.new_scalar_u32(dev)
+        K, R, S, _ = self.weight.shape
+        self.grad_int32acc = ops.conv2d_wgrad(self.act.contiguous(), err_in, R, S, self.stride, self.padding,
+                                              f32_epilogue=F32_EPILOGUE and not self.first_layer, absmax=amg)
+        self.weight_update(amg, grad_rand)
+        if not self.first_layer:
+            return err_out, self.err_exp
+
+
+class TiLinear(UpdateWeight):
+    """ti_torch.py:235-266: int8 fully connected layer, weight [out_features, in_features]."""
+
+    def __init__(self, in_features, out_features, last_layer=False):
+        super().__init__()
+        self._init_weight(torch.Size([out_features, in_features]))
+        self.last_layer = last_layer
+
+    def forward(self, input, rand=None):
+        self.act_in = input
+        act_in, exp_in = input
+        act_in = act_in.contiguous()
+        dev = act_in.device
+        am = ops.new_scalar_u32(dev)
+        acc = ops.gemm(act_in, self.weight, trans_b=True, absmax=am)            # act @ W^T, W read as stored
+        act_out, _, exp_out = _requant(acc, BITWIDTH, ACT_ROUND_METHOD, am, rand,
+                                       exp_a=_exp_tensor(exp_in, dev), exp_b=self._wexp(), want_exp=True)
+        return act_out, exp_out
+
+    def backward(self, input, rand=None, grad_rand=None):
+        err_in, err_exp = input
+        err_in = err_in.contiguous()
+        dev = err_in.device
+        act, self.act_in_exp = self.act_in
+        self.err_exp_in = _exp_tensor(err_exp, dev)
+        am = ops.new_scalar_u32(dev)
+        dx = ops.gemm(err_in, self.weight, absmax=am)                             # err @ W
+        err_out, _, self.err_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
+                                            exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
+        amg = ops.new_scalar_u32(dev)
+        self.grad_int32acc = ops.gemm(err_in, act.contiguous(), trans_a=True, absmax=amg)   # err^T @ act
+        self.weight_update(amg, grad_rand)
+        return err_out, self.err_exp
+
+
+class TiReLU(Module):
+    """ti_torch.py:268-290.  With ``fused`` set the preceding TiConv2d already clamped at zero and
+    forward only records its input (the clamped tensor: ``act > 0`` is the same test on it)."""
+
+    def __init__(self):
+        super().__init__()
+        self.fused = False
+
+    def forward(self, input):
+        self.act_in = input
+        act_in, exp_in = input
+        if self.fused:
+            return input
+        return ops.relu_fwd(act_in.contiguous()), exp_in
+
+    def backward(self, input):
+        err_in, err_exp = input
+        act, _ = self.act_in
+        return ops.relu_bwd(act.contiguous(), err_in.contiguous()), err_exp
+
+
+class TiMaxpool2d(Module):
+    """ti_torch.py:292-316."""
+
+    def __init__(self, kernel_size, stride, padding=0):
+        super().__init__()
+        self.kernel_size = kernel_size
+        self.stride = stride
+        self.padding = padding
+
+    def forward(self, input):
+        self.act_in, exp_in = input
+        self.act_in = self.act_in.contiguous()
+        self.act_out = ops.maxpool_fwd(self.act_in, self.kernel_size, self.stride, self.padding)
+        return self.act_out, exp_in
+
+    def backward(self, input):
+        err_in, err_exp = input
+        err_out = ops.maxpool_bwd(self.act_out, err_in.contiguous(), self.act_in, self.kernel_size, self.stride,
+                                  self.padding, POOL_TIES)
+        return err_out, err_exp
+
+
+class TiFlat(Module):
+    """ti_torch.py:318-332."""
+
+    def forward(self, input):
+        self.act_in = input
+        act_in, exp_in = input
+        return act_in.view(-1, act_in.nelement() // act_in.size(0)), exp_in
+
+    def backward(self, input):
+        err_in, err_exp = input
+        act, _ = self.act_in
+        return err_in.view_as(act), err_exp
+
+
+class TiDropout(Module):
+    """ti_torch.py:439-455: one keep/drop decision per feature (not per sample), exponent + 1.
+    ``mask`` (int8 0/1 per feature) can be supplied for reproducible runs."""
+
+    def forward(self, input, mask=None):
+        if TRAINING:
+            act_in, exp_in = input
+            if mask is None:
+                mask = torch.randint(low=0, high=2, size=(act_in.size(1),), dtype=torch.int8, device=act_in.device)
+            self.drop_mask = mask.to(act_in.device)
+            return act_in * self.drop_mask, _exp_tensor(exp_in, act_in.device) + 1
+        return input
+
+    def backward(self, input):
+        err_in, err_exp = input
+        return err_in * self.drop_mask, err_exp

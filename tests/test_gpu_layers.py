@@ -1,0 +1,224 @@
+"""Layer- and step-level GPU parity: niti_amd.ti_torch / ti_net / ti_vgg against the CPU oracle
+model on the same seeded int8 weights, inputs, labels and injected random draws.  Every int8
+tensor, every exponent and every updated weight must match exactly."""
+import sys
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _say(*a):
+    print("[case]", *a, flush=True)
+
+
+def ri8(g, *shape, lo=-127, hi=127):
+    return torch.randint(lo, hi + 1, shape, generator=g, dtype=torch.int8)
+
+
+def laplace_i8(g, shape, b=16.0):
+    u = torch.rand(shape, generator=g, dtype=torch.float64) - 0.5
+    v = -b * torch.sign(u) * torch.log1p(-2 * u.abs())
+    return torch.clamp(torch.round(v), -127, 127).to(torch.int8)
+
+
+@pytest.fixture()
+def tt():
+    from niti_amd import ti_torch
+    saved = {k: getattr(ti_torch, k) for k in ("ACT_ROUND_METHOD", "ERROR_ROUND_METHOD", "GRAD_ROUND_METHOD",
+                                               "GRAD_BITWIDTH", "DIV_MODE", "BW_MODE", "F32_EPILOGUE", "POOL_TIES", "TRAINING")}
+    yield ti_torch
+    for k, v in saved.items():
+        setattr(ti_torch, k, v)
+
+
+def _ei(e):
+    return int(e.item()) if isinstance(e, torch.Tensor) else int(e)
+
+
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+@pytest.mark.parametrize("first", [False, True])
+def test_conv_layer_fwd_bwd(tt, div_mode, first):
+    from oracle import niti_model_oracle as mo
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(1000 + first)
+    N, H, C, K = 8, 16, (3 if first else 32), 64
+    _say("conv layer", div_mode, first)
+    tt.DIV_MODE = div_mode
+    w, x = ri8(g, K, 3, 3, C), ri8(g, N, H, H, C)
+    err = laplace_i8(g, (N, H, H, K))
+    cfg = mo.Cfg(div_mode=div_mode)
+    o = mo.OConv2d(w, -9, first_layer=first)
+    yo, eo = o.forward((x, -3), cfg)
+    ro = o.backward((err, -5), cfg)
+    layer = tt.TiConv2d(C, K, first_layer=first)
+    layer.weight = w.to(dev)
+    layer.weight_exp = torch.tensor(-9.0)
+    layer.keep_grad = True
+    y, e = layer.forward((x.to(dev), -3))
+    assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+    r = layer.backward((err.to(dev), -5))
+    assert torch.equal(layer.grad.cpu(), o.grad) and _ei(layer.grad_shift) == o.grad_shift
+    assert torch.equal(layer.weight.cpu(), o.weight)
+    assert _ei(layer.grad_exp) == o.grad_exp
+    if first:
+        assert r is None and ro is None
+    else:
+        assert torch.equal(r[0].cpu(), ro[0]) and _ei(r[1]) == ro[1]
+
+
+@pytest.mark.parametrize("methods", [("round", "round", "psto"), ("sto", "sto", "sto"), ("psto", "psto", "round")])
+def test_linear_layer_fwd_bwd(tt, methods):
+    from oracle import niti_model_oracle as mo
+    from oracle import niti_oracle as po
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(1100)
+    m, kin, nout = 32, 512, 48
+    _say("linear layer", methods)
+    fn = {"round": tt.RoundShift, "sto": tt.StoShift, "psto": tt.PstoShift}
+    tt.ACT_ROUND_METHOD, tt.ERROR_ROUND_METHOD, tt.GRAD_ROUND_METHOD = (fn[x] for x in methods)
+    w, x, err = ri8(g, nout, kin), ri8(g, m, kin), ri8(g, m, nout)
+    # random integers for the three stochastic roundings, drawn for the shifts the oracle will see
+    acc_f, acc_b, acc_g = po.int8mm(x, w.t().contiguous()), po.int8mm(err, w), po.int8mm(err.t().contiguous(), x)
+    def draw(acc, tgt):
+        s = max(po.RangeEstimate(acc) - tgt, 1)
+        return torch.randint(0, 2 ** s, acc.shape, generator=g, dtype=torch.int32)
+    rf, rb, rg = draw(acc_f, 7), draw(acc_b, 7), draw(acc_g, 5)
+    cfg = mo.Cfg(*methods)
+    o = mo.OLinear(w, -8)
+    yo, eo = o.forward((x, 1), cfg, rf)
+    ro = o.backward((err, -2), cfg, rb, rg)
+    layer = tt.TiLinear(kin, nout)
+    layer.weight, layer.weight_exp, layer.keep_grad = w.to(dev), torch.tensor(-8.0), True
+    y, e = layer.forward((x.to(dev), 1), rf.to(dev))
+    assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+    r = layer.backward((err.to(dev), -2), rb.to(dev), rg.to(dev))
+    assert torch.equal(r[0].cpu(), ro[0]) and _ei(r[1]) == ro[1]
+    assert torch.equal(layer.grad.cpu(), o.grad)
+    assert torch.equal(layer.weight.cpu(), o.weight) and _ei(layer.grad_exp) == o.grad_exp
+
+
+def test_standalone_shift_functions(tt, kat):
+    dev = torch.device("cuda:0")
+    _say("standalone RoundShift/PstoShift/StoShift")
+    X = torch.tensor(kat["X"], dtype=torch.int32, device=dev)
+    for mode in ("floor", "trunc"):
+        tt.DIV_MODE = mode
+        assert tt.RoundShift(X, 7).cpu().tolist() == kat[f"round_s7_{mode}"]
+        assert tt.PstoShift(X, 7).cpu().tolist() == kat[f"psto_s7_{mode}"]
+        r20 = torch.arange(-20, 21, dtype=torch.int32, device=dev)
+        assert tt.StoShift(r20, 4, torch.full_like(r20, 7)).cpu().tolist() == kat[f"sto_s4_u7_m20_20_{mode}"]
+        assert tt.PstoShift(r20, 4).cpu().tolist() == kat[f"psto_s4_m20_20_{mode}"]
+    y = tt.StoShift(X, 3)          # device random draw: only the range is checkable
+    assert int(y.min()) >= -127 and int(y.max()) <= 127
+
+
+def _build_pair(tt, cfg_list, widths_in, N, seed, dropout, image=32):
+    """Same int8 weights in the GPU model and in the oracle model."""
+    from niti_amd import ti_vgg
+    from oracle import niti_model_oracle as mo
+    g = torch.Generator().manual_seed(seed)
+    dev = torch.device("cuda:0")
+    ti_vgg.cifar_cfg["test"] = cfg_list
+    net = ti_vgg.TiVGG_cifar("test", fuse=True, dropout=dropout)
+    weights, exps = [], []
+    for l in net.forward_layers:
+        if hasattr(l, "weight"):
+            w = ri8(g, *l.weight.shape)
+            e = -int(torch.randint(6, 12, (1,), generator=g))
+            l.weight, l.weight_exp = w.to(dev), torch.tensor(float(e))
+            weights.append(w)
+            exps.append(e)
+    fc_in = weights[-1].shape[1]
+    mask = torch.randint(0, 2, (fc_in,), generator=g, dtype=torch.int8) if dropout else None
+    onet = mo.build_vgg(cfg_list, weights, exps, mo.Cfg(), mask)
+    x = ri8(g, N, image, image, 3)
+    target = torch.randint(0, 10, (N,), generator=g)
+    loss_rand = torch.randint(0, 16, (N, 10), generator=g, dtype=torch.int32)
+    return net, onet, x, target, loss_rand, mask
+
+
+@pytest.mark.parametrize("name,cfg_list,N", [
+    ("vgg7-narrow", [16, 16, 'M', 32, 32, 'M', 512, 512, 'M'], 8),
+    ("vgg7-full", [128, 128, 'M', 256, 256, 'M', 512, 512, 'M'], 16),
+])
+def test_training_step(tt, name, cfg_list, N):
+    """One complete integer training step (forward, loss gradient, backward, weight update)."""
+    from niti_amd import ti_torch
+    dev = torch.device("cuda:0")
+    _say("training step", name, N)
+    net, onet, x, target, loss_rand, mask = _build_pair(tt, cfg_list, None, N, 2000, dropout=True)
+    # forward
+    yo, eo = onet.forward_int8(x, 0)
+    drop = [l for l in net.forward_layers if isinstance(l, ti_torch.TiDropout)][0]
+    orig_fwd = drop.forward
+    drop.forward = lambda inp: orig_fwd(inp, mask.to(dev))
+    y, e = net.forward_int8(x.to(dev), 0)
+    assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+    # backward from the oracle's loss gradient (the float loss itself is compared separately)
+    onet.backward(target, loss_rand)
+    net.backward_from((onet.loss_err.to(dev), 0))
+    gl = [l for l in net.forward_layers if hasattr(l, "weight")]
+    ol = [l for l in onet.layers if hasattr(l, "weight")]
+    assert len(gl) == len(ol)
+    for i, (a, b) in enumerate(zip(gl, ol)):
+        assert torch.equal(a.weight.cpu(), b.weight), "updated weight of layer %d" % i
+        assert _ei(a.grad_exp) == b.grad_exp, "grad exponent of layer %d" % i
+        if i > 0:
+            assert _ei(a.err_exp) == b.err_exp, "error exponent of layer %d" % i
+    # a second step on the updated weights keeps matching
+    yo, eo = onet.forward_int8(x, 0)
+    y, e = net.forward_int8(x.to(dev), 0)
+    assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+
+
+def test_ti_loss_matches_oracle_on_typical_logits(tt):
+    """TiLoss runs float32 ops on the device; on these inputs the result equals the CPU evaluation."""
+    from niti_amd.ti_loss import TiLoss
+    from oracle import niti_oracle as po
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(3000)
+    for e in (-9, -7, -6, -3, 0):
+        _say("ti_loss", e)
+        out = ri8(g, 64, 10)
+        tgt = torch.randint(0, 10, (64,), generator=g)
+        u = torch.randint(0, 16, (64, 10), generator=g, dtype=torch.int32)
+        ref, _ = po.ti_loss(out, e, tgt, u)
+        got, ge = TiLoss()(out.to(dev), e, tgt.to(dev), u.to(dev))
+        assert ge == 0
+        diff = (got.cpu().to(torch.int16) - ref.to(torch.int16)).abs()
+        # float32 pow may differ in the last ulp between host and device: allow one int8 step
+        assert int(diff.max()) <= 1
+        assert float((diff != 0).float().mean()) < 0.01
+
+
+def test_shims_match_reference_conventions():
+    """The four stand-in extension modules: names, return dtypes / shapes / strides, error behaviour."""
+    import niti_amd.shims as shims
+    from oracle import niti_oracle as po
+    dev = torch.device("cuda:0")
+    _say("shims")
+    shims.install()
+    import cutlassconv_cuda, int8conv_cuda, int8mm_cuda, int8pool_cuda
+    g = torch.Generator().manual_seed(4000)
+    x, w = ri8(g, 2, 8, 8, 16), ri8(g, 24, 3, 3, 16)
+    y = cutlassconv_cuda.sp_conv_optimized(x.to(dev), w.to(dev), 1, 1)
+    assert y.dtype == torch.int32 and y.is_contiguous() and tuple(y.shape) == (2, 8, 8, 24)
+    assert torch.equal(y.cpu(), po.conv2d_int8(x, w))
+    assert torch.equal(cutlassconv_cuda.sp_conv(x.to(dev), w.to(dev), 2, 1).cpu(), po.conv2d_int8(x, w, 2, 1))
+    with pytest.raises(RuntimeError):
+        cutlassconv_cuda.sp_conv(x, w.to(dev), 1, 1)                       # CPU tensor
+    with pytest.raises(RuntimeError):
+        cutlassconv_cuda.sp_conv(x.to(dev).permute(0, 2, 1, 3), w.to(dev), 1, 1)   # not contiguous
+    a, b = ri8(g, 12, 32), ri8(g, 32, 20)
+    c = int8mm_cuda.int8_mm(a.to(dev), b.to(dev))
+    assert c.dtype == torch.int32 and tuple(c.shape) == (12, 20) and not c.is_contiguous() and c.stride() == (1, 12)
+    assert torch.equal(c.contiguous().cpu(), po.int8mm(a, b))
+    p = int8pool_cuda.int8_pool(x.to(dev), 2, 2, 0)
+    assert torch.equal(p.cpu(), po.maxpool_fwd(x))
+    dy = ri8(g, 2, 4, 4, 16, lo=-20, hi=20)
+    dx = int8pool_cuda.int8_pool_backward(p.half(), dy.to(dev).half(), x.to(dev).half(), 2, 2, 0)
+    assert dx.dtype == torch.float16
+    assert torch.equal(dx.type(torch.int8).cpu(), po.maxpool_bwd(po.maxpool_fwd(x), dy, x))
+    assert hasattr(int8conv_cuda, "group_conv") and hasattr(cutlassconv_cuda, "weight_grad")
