@@ -34,6 +34,8 @@ enum {
 #define NITI_EPI_F32_ROUNDTRIP 1u /* pass every int32 result through fp32 and back, as the
                                      reference's CUTLASS epilogue does
                                      (pytorch/cutlass-extension/cutlassconv_kernel.cu:78-85) */
+#define NITI_DGRAD_FILTER_PREPARED 2u /* niti_conv2d_i8_dgrad: `w` already is the re-laid filter
+                                         written by niti_filter_dgrad_layout_i8; no workspace */
 /* requant flags */
 #define NITI_RQ_RELU 1u /* clamp the int8 result at 0 (TiReLU.forward, ti_torch.py:272-279) */
 
@@ -77,6 +79,9 @@ int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y, int N, in
  * Workspace: niti_conv2d_i8_dgrad_workspace() bytes (re-laid filter).
  */
 size_t niti_conv2d_i8_dgrad_workspace(int C, int K, int R, int S);
+/* dst[c][r][s][k] = w[k][R-1-r][S-1-s][c]: the filter as the data gradient streams it
+ * (the reference materialises the same tensor with flip/transpose/contiguous, ti_torch.py:404) */
+int niti_filter_dgrad_layout_i8(const int8_t* w, int8_t* dst, int K, int R, int S, int C, void* stream);
 int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N, int H, int W, int C, int K, int R,
                          int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
                          size_t workspace_bytes, void* stream);

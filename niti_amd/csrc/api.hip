@@ -106,18 +106,30 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
     return fail(NITI_ERR_UNSUPPORTED, "conv_dgrad: needs stride 1, square filter, pad <= R-1 (stride=%d R=%d S=%d pad=%d)", stride, R, S, pad);
   if (K % 16 != 0) return fail(NITI_ERR_UNSUPPORTED, "conv_dgrad: K=%d must be a multiple of 16", K);
   if (!aligned16(err) || !aligned16(dx)) return fail(NITI_ERR_INVALID_ARG, "conv_dgrad: pointers must be 16-byte aligned");
-  const size_t need = niti_conv2d_i8_dgrad_workspace(C, K, R, S);
-  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
-    return fail(NITI_ERR_WORKSPACE, "conv_dgrad: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
   hipStream_t s = static_cast<hipStream_t>(stream);
-  int8_t* wt = static_cast<int8_t*>(workspace);
-  st = launch_filter_flip_transpose(w, wt, K, R, S, C, s);
-  if (st != NITI_OK) return st;
+  const int8_t* wt = w;
+  if (!(flags & NITI_DGRAD_FILTER_PREPARED)) {
+    const size_t need = niti_conv2d_i8_dgrad_workspace(C, K, R, S);
+    if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+      return fail(NITI_ERR_WORKSPACE, "conv_dgrad: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
+    st = launch_filter_flip_transpose(w, static_cast<int8_t*>(workspace), K, R, S, C, s);
+    if (st != NITI_OK) return st;
+    wt = static_cast<const int8_t*>(workspace);
+  } else if (!aligned16(w)) {
+    return fail(NITI_ERR_INVALID_ARG, "conv_dgrad: prepared filter must be 16-byte aligned");
+  }
   const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
   // fprop over the error map: "input" [N,P,Q,K], "filter" [C,R,S,K], padding R-1-pad -> [N,H,W,C]
   ConvProblem p{err, wt, dx, absmax, N, P, Q, K, C, R, S, 1, R - 1 - pad,
                 static_cast<long long>(H) * W * C, static_cast<long long>(W) * C, C, 1, 1, flags};
   return launch_conv_igemm(p, s);
+}
+
+extern "C" int niti_filter_dgrad_layout_i8(const int8_t* w, int8_t* dst, int K, int R, int S, int C, void* stream) {
+  clear_error();
+  if (w == nullptr || dst == nullptr || K <= 0 || R <= 0 || S <= 0 || C <= 0)
+    return fail(NITI_ERR_INVALID_ARG, "filter_dgrad_layout: bad arguments");
+  return launch_filter_flip_transpose(w, dst, K, R, S, C, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad) {

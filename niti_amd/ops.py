@@ -55,9 +55,19 @@ def conv2d_fprop(x, w, stride=1, padding=1, f32_epilogue=False, absmax: Optional
     return y
 
 
-def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None):
-    """err [N,P,Q,K] int8, w [K,R,S,C] int8 -> dx [N,H,W,C] int32 (stride 1)."""
-    _chk_dev(err, w, absmax)
+def filter_dgrad_layout(w):
+    """w [K,R,S,C] int8 -> [C,R,S,K] int8 with flipped taps (the data gradient's filter operand)."""
+    _chk_dev(w)
+    K, R, S, C = w.shape
+    dst = torch.empty((C, R, S, K), dtype=torch.int8, device=w.device)
+    L.check(L.lib().niti_filter_dgrad_layout_i8(_ptr(w), _ptr(dst), K, R, S, C, _stream(w)), "niti_filter_dgrad_layout_i8")
+    return dst
+
+
+def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None, prepared_filter=None):
+    """err [N,P,Q,K] int8, w [K,R,S,C] int8 -> dx [N,H,W,C] int32 (stride 1).  ``prepared_filter``:
+    the output of filter_dgrad_layout(w), to skip the re-layout inside the call."""
+    _chk_dev(err, w, absmax, prepared_filter)
     N, P, Q, K = err.shape
     K2, R, S, C = w.shape
     if K2 != K:
@@ -65,10 +75,15 @@ def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None):
     H = P - 2 * padding + R - 1
     W = Q - 2 * padding + S - 1
     dx = torch.empty((N, H, W, C), dtype=torch.int32, device=err.device)
-    nbytes = L.lib().niti_conv2d_i8_dgrad_workspace(C, K, R, S)
-    ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=err.device)
-    st = L.lib().niti_conv2d_i8_dgrad(_ptr(err), _ptr(w), _ptr(dx), N, H, W, C, K, R, S, stride, padding,
-                                      _flags(f32_epilogue), _ptr(absmax), _ptr(ws), nbytes, _stream(err))
+    flags = _flags(f32_epilogue)
+    if prepared_filter is not None:
+        st = L.lib().niti_conv2d_i8_dgrad(_ptr(err), _ptr(prepared_filter), _ptr(dx), N, H, W, C, K, R, S, stride, padding,
+                                          flags | L.DGRAD_FILTER_PREPARED, _ptr(absmax), None, 0, _stream(err))
+    else:
+        nbytes = L.lib().niti_conv2d_i8_dgrad_workspace(C, K, R, S)
+        ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=err.device)
+        st = L.lib().niti_conv2d_i8_dgrad(_ptr(err), _ptr(w), _ptr(dx), N, H, W, C, K, R, S, stride, padding,
+                                          flags, _ptr(absmax), _ptr(ws), nbytes, _stream(err))
     L.check(st, "niti_conv2d_i8_dgrad")
     return dx
 
