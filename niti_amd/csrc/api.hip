@@ -136,6 +136,7 @@ extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || pad < 0) return 0;
   const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
   if (P <= 0 || Q <= 0) return 0;
+  if (wgrad3x3_supported(N, H, W, C, K, R, S, 1, pad)) return round256(wgrad3x3_workspace(N, H, C, K));
   const size_t np = static_cast<size_t>(round16(N));
   return round256(static_cast<size_t>(C) * H * W * np) + round256(static_cast<size_t>(K) * P * Q * np);
 }
@@ -152,6 +153,11 @@ extern "C" int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_
   if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
     return fail(NITI_ERR_WORKSPACE, "conv_wgrad: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
   hipStream_t s = static_cast<hipStream_t>(stream);
+  if (wgrad3x3_supported(N, H, W, C, K, R, S, stride, pad)) {
+    if (!aligned16(act) || !aligned16(err) || !aligned16(dw))
+      return fail(NITI_ERR_INVALID_ARG, "conv_wgrad: pointers must be 16-byte aligned");
+    return launch_wgrad3x3(act, err, dw, N, H, C, K, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, absmax, workspace, s);
+  }
   const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
   const int np = round16(N);
   int8_t* act_t = static_cast<int8_t*>(workspace);                                 // [C][H*W][np]

@@ -77,6 +77,18 @@ __device__ inline uint32_t wave_max_u32(uint32_t v) {
   return v;
 }
 
+// Folds a wavefront's max |value| into *dst.  Same-address atomics serialise in the memory
+// system (about 10 ns each), so a wavefront first looks at the value already there and only
+// issues the atomic when it would raise it; the stored value only ever grows, so a stale read
+// can at worst cause a redundant atomic.
+__device__ inline void fold_absmax(uint32_t* dst, uint32_t lane_max) {
+  const uint32_t m = wave_max_u32(lane_max);
+  if ((threadIdx.x & 63) == 0 && m != 0) {
+    const uint32_t seen = __hip_atomic_load(dst, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (m > seen) atomicMax(dst, m);
+  }
+}
+
 // ---- launchers implemented in the .hip files ----
 struct ConvProblem {
   const int8_t* x;   // [N,H,W,C]
@@ -97,5 +109,11 @@ int launch_filter_flip_transpose(const int8_t* w, int8_t* dst, int K, int R, int
 int launch_transpose_outer_inner_i8(const int8_t* src, int8_t* dst, int A, int B, int C, int Apad, hipStream_t stream);
 // in place: v = roundtrip(v) if requested; absmax folded if non-null
 int launch_post_i32(int32_t* v, int64_t n, bool roundtrip, uint32_t* absmax, hipStream_t stream);
+
+// native 3x3 / stride 1 / pad 1 weight gradient (wgrad3x3.hip)
+bool wgrad3x3_supported(int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
+size_t wgrad3x3_workspace(int N, int H, int C, int K);
+int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, int H, int C, int K, bool roundtrip,
+                    uint32_t* absmax, void* workspace, hipStream_t stream);
 
 }  // namespace niti

@@ -12,7 +12,10 @@
 // leaves every lane holding 4 consecutive output channels of one pixel per register quad:
 // the int32 result goes out as 16-byte stores.  LDS rows are padded to 80 bytes so that the
 // 16 lanes served together by a ds_read_b128 hit 16 distinct bank groups.
+#include <stdlib.h>
+
 #include "common.h"
+#include "conv_args.h"
 
 namespace niti {
 namespace {
@@ -21,19 +24,6 @@ constexpr int BM = 128;  // pixels per workgroup
 constexpr int BN = 128;  // output channels per workgroup
 constexpr int BK = 64;   // reduction bytes per main-loop step
 constexpr int LD = 80;   // padded LDS row pitch in bytes
-
-struct ConvArgs {
-  const int8_t* x;
-  const int8_t* w;
-  int32_t* y;
-  uint32_t* absmax;
-  int N, H, W, C, K, R, S, P, Q, stride, pad;
-  int M, Kg;
-  int kiters, kiters_per_split;
-  long long ysN, ysP, ysQ, ysK;
-  int dense_out;  // y is plain [M][K]: vector stores allowed
-  unsigned flags;
-};
 
 template <bool kSplitK>
 __global__ __launch_bounds__(256, 2) void conv_igemm_i8_kernel(const ConvArgs a) {
@@ -202,13 +192,20 @@ __global__ __launch_bounds__(256, 2) void conv_igemm_i8_kernel(const ConvArgs a)
       }
     }
   }
-  if (!kSplitK && a.absmax != nullptr) {
-    lmax = wave_max_u32(lmax);
-    if (lane == 0 && lmax != 0) atomicMax(a.absmax, lmax);
-  }
+  if (!kSplitK && a.absmax != nullptr) fold_absmax(a.absmax, lmax);
 }
 
 }  // namespace
+
+static int tile_override_from_env() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("NITI_CONV_TILE");
+    v = e ? atoi(e) : 0;
+    if (v < 0 || v > 4) v = 0;
+  }
+  return v;
+}
 
 int launch_conv_igemm(const ConvProblem& p, hipStream_t stream) {
   ConvArgs a;
@@ -230,13 +227,17 @@ int launch_conv_igemm(const ConvProblem& p, hipStream_t stream) {
   a.dense_out = (p.ysK == 1 && p.ysQ == p.K && p.ysP == static_cast<long long>(a.Q) * p.K &&
                  p.ysN == static_cast<long long>(a.P) * a.Q * p.K && p.K % 4 == 0) ? 1 : 0;
   a.flags = p.flags;
+  a.x_bytes = static_cast<long long>(p.N) * p.H * p.W * p.C;
+  a.w_bytes = static_cast<long long>(p.K) * a.Kg;
+  a.tile_override = tile_override_from_env();
   int split = p.split_k < 1 ? 1 : p.split_k;
   if (split > a.kiters) split = a.kiters;
   a.kiters_per_split = (a.kiters + split - 1) / split;
   split = (a.kiters + a.kiters_per_split - 1) / a.kiters_per_split;
+  if (conv_mfma_supported(a)) return launch_conv_mfma(a, split, stream);
   dim3 grid((a.M + BM - 1) / BM, (p.K + BN - 1) / BN, split);
   if (grid.y > 65535u || grid.z > 65535u) return fail(NITI_ERR_UNSUPPORTED, "conv: K=%d too large", p.K);
-  if (p.split_k > 1)
+  if (split > 1)
     hipLaunchKernelGGL(conv_igemm_i8_kernel<true>, grid, dim3(256), 0, stream, a);
   else
     hipLaunchKernelGGL(conv_igemm_i8_kernel<false>, grid, dim3(256), 0, stream, a);

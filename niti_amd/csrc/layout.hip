@@ -61,10 +61,7 @@ __global__ void post_i32_kernel(int32_t* v, int64_t n, int roundtrip, uint32_t* 
     const uint32_t u = uabs(t);
     lmax = u > lmax ? u : lmax;
   }
-  if (absmax != nullptr) {
-    lmax = wave_max_u32(lmax);
-    if ((threadIdx.x & 63) == 0 && lmax != 0) atomicMax(absmax, lmax);
-  }
+  if (absmax != nullptr) fold_absmax(absmax, lmax);
 }
 
 inline int grid_for(int64_t n, int block, int cap = 8192) {

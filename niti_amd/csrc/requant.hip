@@ -60,8 +60,7 @@ __global__ __launch_bounds__(256) void absmax_i32_kernel(const int32_t* __restri
     const uint32_t u = uabs(x[i]);
     lmax = u > lmax ? u : lmax;
   }
-  lmax = wave_max_u32(lmax);
-  if ((threadIdx.x & 63) == 0 && lmax != 0) atomicMax(absmax, lmax);
+  fold_absmax(absmax, lmax);
 }
 
 struct RequantArgs {

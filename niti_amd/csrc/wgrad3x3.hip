@@ -1,0 +1,342 @@
+// Native int8 weight gradient of a 3x3, stride-1, pad-1 convolution on the gfx950 matrix cores:
+//   dw[k,r,s,c] = sum_{n,p,q} err[n,p,q,k] * act[n,p+r-1,q+s-1,c]
+//
+// GEMM view: rows = output channels k, columns = (tap, input channel c), reduction over the
+// output pixels.  Both operands are stored with channels contiguous and the reduction index
+// (pixels) strided, the opposite of what an MFMA operand needs (16 reduction bytes per lane).
+// The kernel therefore stages tiles in their natural [pixel][channel] layout with
+// buffer_load ... lds and builds the fragments with ds_read_b64_tr_b8, the gfx950 transposing
+// LDS read: within 16 lanes, lane j supplies the address of an 8-byte row and lane i receives
+// byte (i % 8) of the rows supplied by lanes 2m + i/8 (m = 0..7).  Pointing lanes 2m and 2m+1 at
+// the two 8-channel halves of pixel m gives every lane 8 consecutive pixels of channel i.
+//
+// Work split: a workgroup (8 wavefronts, 4 x 2) owns 128 output channels x 64 input channels x 9
+// taps of accumulators (one 32 x 32 tile per tap and wavefront: 144 registers per lane, two
+// wavefronts per SIMD) and walks over "bands" of 128 consecutive output pixels
+// (whole rows of an image, or whole small images).  Per band it stages the 128 x 128 error tile
+// and the activation rows with their halo once, and serves all nine taps from that one halo
+// tile, so activations are read from L2 once instead of nine times.  The pixel range is split
+// over gridDim.z workgroups; each writes its partial sums to a workspace slice and a second
+// kernel adds the slices (integer addition: any split gives the same result).
+#include "common.h"
+
+namespace niti {
+namespace {
+
+#define NITI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+typedef int v2i_t __attribute__((ext_vector_type(2)));
+constexpr int kOob = -1;
+
+template <int N>
+__device__ inline void wg_wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (((N >> 4) & 3) << 14) | 0x0F70);
+}
+__device__ inline void wg_sync() {
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
+struct WgradArgs {
+  const int8_t* act;  // [N,H,W,C], H == W == Q
+  const int8_t* err;  // [N,Q,Q,K]
+  int32_t* partial;   // [splits][slice_stride], slice z holds K*9*C partial sums
+  long long slice_stride;
+  int N, C, K;
+  int bands, bands_per_split;
+  long long act_bytes, err_bytes;
+};
+
+// Q: image width = height; BR: output rows of one image per band; NI: images per band; BR*NI*Q == 128
+template <int Q, int BR, int NI>
+struct Geom {
+  static constexpr int RP = (Q + 2 + 15) / 16 * 16;  // halo row pitch in pixel slots (multiple of 16)
+  static constexpr int HR = BR + 2;                   // halo rows per image
+  static constexpr int ACT_INSTR = NI * HR * (RP / 16);
+  static constexpr int ACT_BYTES = NI * HR * RP * 64;
+  static constexpr int ERR_BYTES = 128 * 128;
+  static constexpr int STAGE_BYTES = ERR_BYTES + ACT_BYTES;
+  static constexpr int ACT_LOADS = (ACT_INSTR + 7) / 8;  // per wavefront
+  static constexpr int NL = 2 + ACT_LOADS;               // loads per wavefront per stage
+  static constexpr int BANDS_PER_IMAGE = Q / BR;         // valid when NI == 1
+  static_assert(BR * NI * Q == 128, "a band is 128 output pixels");
+};
+
+template <int Q, int BR, int NI, int STAGES>
+__global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
+  using G = Geom<Q, BR, NI>;
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];  // STAGES stages + 1 KB dump slot
+  int8_t* const dump = smem + STAGES * G::STAGE_BYTES;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int k0 = blockIdx.x * 128;
+  const int c0 = blockIdx.y * 64;
+  const int band_begin = blockIdx.z * a.bands_per_split;
+  const int band_end = min(band_begin + a.bands_per_split, a.bands);
+  const int nb = band_end - band_begin;
+
+  const __amdgpu_buffer_rsrc_t ract = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.act), 0, a.act_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rerr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.err), 0, a.err_bytes, 0x00020000);
+
+  // ---- staging.  Error tile: 16 instructions of 8 pixels x 128 bytes; lane -> (pixel lane/8, piece lane%8)
+  int err_off[2];  // byte offset of this lane's 16 bytes relative to the band's first pixel, or kOob
+#pragma unroll
+  for (int i = 0; i < 2; ++i) {
+    const int pix = (wave + 8 * i) * 8 + (lane >> 3);
+    const int piece = (lane & 7) ^ ((pix >> 1) & 7);
+    const int ch = k0 + piece * 16;
+    err_off[i] = ch < a.K ? pix * a.K + ch : kOob;
+  }
+  // Activation halo tile: NI images x HR rows x RP pixel slots x 64 bytes; an instruction fills 16 slots
+  int act_off[G::ACT_LOADS];   // byte offset relative to the band's first image row p0 = 0, or kOob
+  int act_hrow[G::ACT_LOADS];  // halo row (to test against the image border per band)
+  int act_dst[G::ACT_LOADS];   // LDS byte offset of the instruction's 1 KB inside the stage, or -1 -> dump
+#pragma unroll
+  for (int i = 0; i < G::ACT_LOADS; ++i) {
+    const int idx = wave + 8 * i;
+    int off = kOob, hrow = 0, dst = -1;
+    if (idx < G::ACT_INSTR) {
+      const int ni = idx / (G::HR * (G::RP / 16));
+      const int rem = idx - ni * (G::HR * (G::RP / 16));
+      const int h = rem / (G::RP / 16);
+      const int wg = rem - h * (G::RP / 16);
+      const int w = wg * 16 + (lane >> 2);
+      const int piece = (lane & 3) ^ ((w >> 2) & 3);
+      const int ch = c0 + piece * 16;
+      const int iw = w - 1;
+      hrow = h;
+      dst = G::ERR_BYTES + ((ni * G::HR + h) * G::RP + wg * 16) * 64;
+      if (iw >= 0 && iw < Q && ch < a.C) off = ((ni * Q + (h - 1)) * Q + iw) * a.C + ch;  // relative to image n0, row p0
+      else off = kOob;
+      if (w >= Q + 2) off = kOob;
+    }
+    act_off[i] = off;
+    act_hrow[i] = hrow;
+    act_dst[i] = dst;
+  }
+
+  auto issue = [&](int band, int st) {
+    int8_t* base = smem + st * G::STAGE_BYTES;
+    const int pixbase = band * 128;  // first output pixel of the band in [N*Q*Q]
+    // image / first row of the band
+    const int n0 = pixbase / (Q * Q);
+    const int p0 = (pixbase - n0 * (Q * Q)) / Q;
+    const int eb = pixbase * a.K;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int off = err_off[i] == kOob ? kOob : eb + err_off[i];
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rerr, NITI_LDS(base + (wave + 8 * i) * 1024), 16, off, 0, 0, 0);
+    }
+    const int ab = (n0 * Q + p0) * Q * a.C;
+#pragma unroll
+    for (int i = 0; i < G::ACT_LOADS; ++i) {
+      const int ih = p0 + act_hrow[i] - 1;
+      const bool ok = act_off[i] != kOob && ih >= 0 && ih < Q;
+      const int off = ok ? ab + act_off[i] : kOob;
+      int8_t* dst = act_dst[i] >= 0 ? base + act_dst[i] : dump;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ract, NITI_LDS(dst), 16, off, 0, 0, 0);
+    }
+  };
+
+  // ---- fragment addressing (transposing LDS reads)
+  const int j = lane & 15;         // lane inside its group of 16
+  const int gg = (lane >> 4) & 1;  // which 16 channels of the 32-row MFMA operand
+  const int lk = lane >> 5;        // which 16 of the 32 pixels of a reduction step
+  const int wk = wave & 3;         // 32-output-channel quarter of the tile
+  const int wc = wave >> 2;        // 32-input-channel half of the tile
+  int a_base[2];     // [o]: error tile byte offset of this lane's 8-byte row, reduction step 0
+  int b_base[2][3];  // [o][s]: halo tile byte offset, reduction step 0, filter row 0
+#pragma unroll
+  for (int o = 0; o < 2; ++o) {
+    const int lpix = 16 * lk + 8 * o + (j >> 1);  // pixel inside the 32-pixel step
+    {
+      const int cb = wk * 32 + gg * 16 + 8 * (j & 1);
+      a_base[o] = lpix * 128 + ((((cb >> 4) ^ ((lpix >> 1) & 7)) << 4) | (cb & 15));
+    }
+    const int lrow = lpix / Q, pw = lpix % Q;
+    const int cb = wc * 32 + gg * 16 + 8 * (j & 1);
+#pragma unroll
+    for (int s = 0; s < 3; ++s) {
+      const int w = pw + s;
+      b_base[o][s] = G::ERR_BYTES + (lrow * G::RP + w) * 64 + ((((cb >> 4) ^ ((w >> 2) & 3)) << 4) | (cb & 15));
+    }
+  }
+
+  v16i acc[9];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[t][e] = 0;
+
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s)
+    if (s < nb) issue(band_begin + s, s);
+
+  for (int it = 0; it < nb; ++it) {
+    if (it + STAGES - 2 < nb) wg_wait_vmcnt<(STAGES - 2) * G::NL>();
+    else wg_wait_vmcnt<0>();
+    wg_sync();
+    if (it + STAGES - 1 < nb) issue(band_begin + it + STAGES - 1, (it + STAGES - 1) % STAGES);
+    const int8_t* sbase = smem + (it % STAGES) * G::STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int prow = ks * 32 / Q;                         // first output row of this reduction step inside the band
+      const int hrow0 = (prow / BR) * G::HR + (prow % BR);  // its halo row for filter row 0
+      const v2i_t alo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[0] + ks * 4096));
+      const v2i_t ahi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[1] + ks * 4096));
+      const v4i af = v4i{alo[0], alo[1], ahi[0], ahi[1]};
+      v4i bf[9];
+#pragma unroll
+      for (int r = 0; r < 3; ++r)
+#pragma unroll
+        for (int s = 0; s < 3; ++s) {
+          const int roff = (hrow0 + r) * G::RP * 64;
+          const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+              (__attribute__((address_space(3))) v2i_t*)(sbase + b_base[0][s] + roff));
+          const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+              (__attribute__((address_space(3))) v2i_t*)(sbase + b_base[1][s] + roff));
+          bf[r * 3 + s] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        }
+#pragma unroll
+      for (int t = 0; t < 9; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf[t], acc[t], 0, 0, 0);
+    }
+  }
+
+  // ---- partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+wc*32+(lane&31)]
+  int32_t* out = a.partial + static_cast<long long>(blockIdx.z) * a.slice_stride;
+  const int c = c0 + wc * 32 + (lane & 31);
+  if (c < a.C) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int k = k0 + wk * 32 + g * 8 + lk * 4 + e;
+        if (k >= a.K) continue;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) out[(static_cast<long long>(k) * 9 + t) * a.C + c] = acc[t][4 * g + e];
+      }
+  }
+}
+
+// dw[e] = sum_z partial[z][e]; optional fp32 round trip; max |dw| folded into *absmax.
+// A workgroup owns 64 int4 columns; its 4 wavefronts each add every 4th slice, then combine in LDS.
+__global__ __launch_bounds__(256) void wgrad_reduce_kernel(const int32_t* __restrict__ partial, int32_t* __restrict__ dw,
+                                                           int64_t nelem, int64_t n, int splits, int roundtrip,
+                                                           uint32_t* absmax) {
+  __shared__ v4i part[3][64];
+  const int64_t nv = nelem >> 2;  // n below is the slice stride
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t col = static_cast<int64_t>(blockIdx.x) * 64 + lane;
+  v4i s = {0, 0, 0, 0};
+  if (col < nv) {
+    int z = wave;
+    for (; z + 12 < splits; z += 16) {
+      const v4i v0 = reinterpret_cast<const v4i*>(partial + (z + 0) * n)[col];
+      const v4i v1 = reinterpret_cast<const v4i*>(partial + (z + 4) * n)[col];
+      const v4i v2 = reinterpret_cast<const v4i*>(partial + (z + 8) * n)[col];
+      const v4i v3 = reinterpret_cast<const v4i*>(partial + (z + 12) * n)[col];
+      s += (v0 + v1) + (v2 + v3);
+    }
+    for (; z < splits; z += 4) s += reinterpret_cast<const v4i*>(partial + z * n)[col];
+  }
+  if (wave > 0) part[wave - 1][lane] = s;
+  __syncthreads();
+  uint32_t lmax = 0;
+  if (wave == 0 && col < nv) {
+    s += part[0][lane] + part[1][lane] + part[2][lane];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (roundtrip) s[e] = f32_roundtrip(s[e]);
+      const uint32_t u = uabs(s[e]);
+      lmax = u > lmax ? u : lmax;
+    }
+    reinterpret_cast<v4i*>(dw)[col] = s;
+  }
+  if (absmax != nullptr && wave == 0) fold_absmax(absmax, lmax);
+}
+
+// Slices are spaced so that the same element of consecutive slices falls into different memory
+// channels (a stride that is a multiple of 64 KB would put them all into one).
+long long slice_stride_for(int C, int K) {
+  const long long n = static_cast<long long>(K) * 9 * C;
+  return (n + 1023) / 1024 * 1024 + 1088;
+}
+
+int pick_splits(int N, int Q, int C, int K) {
+  const int bands = N * Q * Q / 128;
+  const int tiles = ((K + 127) / 128) * ((C + 63) / 64);
+  int splits = (256 + tiles - 1) / tiles;  // one workgroup per compute unit
+  if (splits > bands) splits = bands;
+  if (splits < 1) splits = 1;
+  const int per = (bands + splits - 1) / splits;
+  return (bands + per - 1) / per;
+}
+
+template <int Q, int BR, int NI>
+int launch_geom(const WgradArgs& a, int splits, hipStream_t stream) {
+  using G = Geom<Q, BR, NI>;
+  constexpr int STAGES = 3;
+  constexpr size_t lds = static_cast<size_t>(STAGES) * G::STAGE_BYTES + 1024;
+  static_assert(lds <= 160 * 1024, "stages must fit in LDS");
+  auto k = wgrad3x3_kernel<Q, BR, NI, STAGES>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return fail(NITI_ERR_LAUNCH, "wgrad: cannot reserve %zu bytes of LDS", lds);
+    attr_set = true;
+  }
+  dim3 grid((a.K + 127) / 128, (a.C + 63) / 64, splits);
+  hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, a);
+  return check_launch("wgrad3x3");
+}
+
+}  // namespace
+
+bool wgrad3x3_supported(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
+  if (R != 3 || S != 3 || stride != 1 || pad != 1 || H != W) return false;
+  if (H != 8 && H != 16 && H != 32) return false;
+  if (C % 16 != 0 || K % 16 != 0) return false;
+  const long long pix = static_cast<long long>(N) * H * W;
+  if (pix % 128 != 0) return false;  // bands of 128 pixels: whole rows / whole images
+  if (H == 8 && N % 2 != 0) return false;
+  if (pix * C >= 0x7fffffffLL || pix * K >= 0x7fffffffLL) return false;
+  return true;
+}
+
+size_t wgrad3x3_workspace(int N, int H, int C, int K) {
+  return static_cast<size_t>(pick_splits(N, H, C, K)) * slice_stride_for(C, K) * sizeof(int32_t);
+}
+
+int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, int H, int C, int K, bool roundtrip,
+                    uint32_t* absmax, void* workspace, hipStream_t stream) {
+  WgradArgs a;
+  a.act = act;
+  a.err = err;
+  a.partial = static_cast<int32_t*>(workspace);
+  a.slice_stride = slice_stride_for(C, K);
+  a.N = N;
+  a.C = C;
+  a.K = K;
+  a.bands = N * H * H / 128;
+  const int splits = pick_splits(N, H, C, K);
+  a.bands_per_split = (a.bands + splits - 1) / splits;
+  a.act_bytes = static_cast<long long>(N) * H * H * C;
+  a.err_bytes = static_cast<long long>(N) * H * H * K;
+  int st;
+  if (H == 32) st = launch_geom<32, 4, 1>(a, splits, stream);
+  else if (H == 16) st = launch_geom<16, 8, 1>(a, splits, stream);
+  else st = launch_geom<8, 8, 2>(a, splits, stream);
+  if (st != NITI_OK) return st;
+  const int64_t n = static_cast<int64_t>(K) * 9 * C;
+  int64_t g = (n / 4 + 63) / 64;
+  if (g < 1) g = 1;
+  hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0, stream, a.partial, dw, n,
+                     static_cast<int64_t>(a.slice_stride), splits, roundtrip ? 1 : 0, absmax);
+  return check_launch("wgrad_reduce");
+}
+
+}  // namespace niti

@@ -304,7 +304,9 @@ class TiConv2d(UpdateWeight):
         self.act, self.act_in_exp = input
         dev = self.act.device
         am = ops.new_scalar_u32(dev)
-        acc = conv2d_int8(self.act, self.weight, self.stride, self.padding, absmax=am)
+        self.act16 = _pad_channels16(self.act).contiguous()      # channel-padded copy, reused by the weight gradient
+        acc = ops.conv2d_fprop(self.act16, _pad_channels16(self.weight).contiguous(), self.stride, self.padding,
+                               f32_epilogue=F32_EPILOGUE, absmax=am)
         act_out, _, exp_out = _requant(acc, BITWIDTH, ACT_ROUND_METHOD, am, rand, relu=self.fuse_relu,
                                        exp_a=_exp_tensor(self.act_in_exp, dev), exp_b=self._wexp(), want_exp=True)
         return act_out, exp_out
@@ -323,9 +325,11 @@ class TiConv2d(UpdateWeight):
                                            exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
             self.err_exp = new_exp
         amg = ops.new_scalar_u32(dev)
-        K, R, S, _ = self.weight.shape
-        self.grad_int32acc = ops.conv2d_wgrad(self.act.contiguous(), err_in, R, S, self.stride, self.padding,
-                                              f32_epilogue=F32_EPILOGUE and not self.first_layer, absmax=amg)
+        K, R, S, C = self.weight.shape
+        dw = ops.conv2d_wgrad(self.act16, err_in, R, S, self.stride, self.padding,
+                              f32_epilogue=F32_EPILOGUE and not self.first_layer, absmax=amg)
+        # zero-padded input channels give zero gradient columns: drop them (they cannot raise the range)
+        self.grad_int32acc = dw if dw.shape[3] == C else dw[..., :C].contiguous()
         self.weight_update(amg, grad_rand)
         if not self.first_layer:
             return err_out, self.err_exp

@@ -98,7 +98,8 @@ def test_conv_dgrad(dev, case):
     assert int(am.cpu()) == po.absmax(ref)
 
 
-WGRAD_CASES = [(2, 8, 8, 16, 16, 3, 1), (16, 8, 8, 32, 48, 3, 1), (5, 7, 9, 40, 24, 3, 1), (32, 16, 16, 64, 128, 3, 1),
+WGRAD_CASES = [(4, 32, 32, 16, 32, 3, 1), (8, 16, 16, 128, 64, 3, 1), (6, 8, 8, 80, 144, 3, 1), (2, 32, 32, 64, 128, 3, 1),
+               (64, 8, 8, 64, 256, 3, 1), (16, 16, 16, 256, 128, 3, 1), (2, 8, 8, 16, 16, 3, 1), (16, 8, 8, 32, 48, 3, 1), (5, 7, 9, 40, 24, 3, 1), (32, 16, 16, 64, 128, 3, 1),
                (4, 8, 8, 3, 16, 3, 1), (6, 8, 8, 16, 10, 5, 2), (3, 6, 6, 8, 8, 3, 0), (128, 8, 8, 16, 16, 3, 1)]
 
 
