@@ -101,6 +101,33 @@ class ConvTriple:
             ops.grad_update(dw, L["w"], am[2:3], 5, "psto")
 
 
+def make_runner(step_fn, warmup, use_graph=True):
+    """Warm up eagerly, then capture one step into a HIP graph (launch-bound chains of small kernels
+    replay without per-launch host cost).  Returns (callable, "graph" | "eager")."""
+    import torch
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(max(warmup, 3)):
+            step_fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    if not use_graph:
+        return step_fn, "eager"
+    try:
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            step_fn()
+        for _ in range(2):
+            g.replay()
+        torch.cuda.synchronize()
+        return g.replay, "graph"
+    except Exception as e:  # capture refused: keep measuring, say so
+        print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
+        torch.cuda.synchronize()
+        return step_fn, "eager"
+
+
 def cpu_baseline(min_seconds=10.0):
     """The plain-C oracle (OpenMP) over the same six layer triples, on synthetic inputs of the same
     shapes, repeated until at least `min_seconds` of CPU work."""
@@ -149,15 +176,14 @@ def train_step_rate(dev, steps, warmup):
         net.forward_int8(x, 0)
         net.backward(target)
 
-    for _ in range(warmup):
-        one()
+    run, mode = make_runner(one, warmup)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
-        one()
+        run()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
-    return BATCH / dt, dt * 1e3
+    return BATCH / dt, dt * 1e3, mode
 
 
 def main():
@@ -167,6 +193,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train-step", action="store_true")
+    ap.add_argument("--eager", action="store_true", help="time eager launches instead of a captured HIP graph")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -182,17 +209,23 @@ def main():
     torch.cuda.set_device(dev)
 
     wl = ConvTriple(dev)
-    for _ in range(args.warmup):
-        wl.step()
+    run, mode = make_runner(wl.step, args.warmup, not args.eager)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(args.steps):
-        wl.step(record=True)
+        run()
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     tops = wl.ops_per_step / (ms_per_step * 1e-3) / 1e12
 
-    # dominant kernel: the MFMA implicit-GEMM convolution (forward + data-gradient launches)
+    # Dominant kernel: the MFMA implicit-GEMM convolution (forward + data-gradient launches), timed
+    # per launch with HIP events on the launch stream over the same K steps run eagerly.  A device
+    # sleep is queued first so that the host runs ahead of the GPU and the event pairs bracket
+    # kernel execution, not host launch latency.
+    torch.cuda._sleep(int(4e7))
+    for _ in range(args.steps):
+        wl.step(record=True)
+    torch.cuda.synchronize()
     k_ms = sum(e0.elapsed_time(e1) for (e0, e1, _) in wl.events)
     k_ops = sum(o for (_, _, o) in wl.events)
     n_launch = len(wl.events)
@@ -204,7 +237,7 @@ def main():
             traffic = json.load(f).get("conv_igemm_i8_kernel_bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic,
-                "kernel": "conv_igemm_i8_kernel<false>", "launches": n_launch,
+                "kernel": "conv_mfma_kernel<..., false>", "launches": n_launch,
                 "avg_launch_us": round(k_ms * 1e3 / max(n_launch, 1), 2),
                 "ops_per_launch_avg": k_ops / max(n_launch, 1),
                 "note": "int8 multiply-accumulate counted as 2 ops; unit is tera-ops/s"}
@@ -217,12 +250,13 @@ def main():
                                   "wgrad + grad rounding + weight update) over the six VGG-small conv shapes, batch 128, "
                                   "3x3 pad 1, uniform int8 inputs, Laplace int8 errors",
                       "ops_per_step": wl.ops_per_step, "batch": BATCH},
+           "launch_mode": mode,
            "pct_int8_mfma_peak": round(100.0 * tops / INT8_MFMA_PEAK_TOPS, 2),
            "roofline": roofline}
     if not args.no_train_step:
-        ips, ms = train_step_rate(dev, max(args.steps, 5), max(args.warmup, 2))
+        ips, ms, tmode = train_step_rate(dev, max(args.steps, 5), max(args.warmup, 2))
         out["train_step"] = {"workload": "BASELINE configs[3]: VGG-small (6 conv + FC) integer training step, batch 128",
-                             "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3)}
+                             "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": tmode}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))

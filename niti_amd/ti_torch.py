@@ -39,11 +39,23 @@ POOL_TIES = "first"
 # ------------------------------------------------------------------------------------------
 # small helpers
 # ------------------------------------------------------------------------------------------
+_EXP_CONSTANTS = {}
+
+
 def _exp_tensor(e, device) -> torch.Tensor:
-    """Exponent as a 1-element int32 device tensor (accepts int, float, 0-d or 1-element tensors)."""
+    """Exponent as a 1-element int32 device tensor (accepts int, float, 0-d or 1-element tensors).
+    Host values are uploaded once and cached, so steady-state steps issue no host-to-device copies
+    (which also keeps a step capturable into a HIP graph)."""
     if isinstance(e, torch.Tensor):
-        return e.reshape(1).to(device=device, dtype=torch.int32)
-    return torch.tensor([int(e)], dtype=torch.int32, device=device)
+        if e.is_cuda:
+            return e.reshape(1) if e.dtype == torch.int32 else e.reshape(1).to(torch.int32)
+        e = int(e)
+    key = (int(e), str(device))
+    t = _EXP_CONSTANTS.get(key)
+    if t is None:
+        t = torch.tensor([int(e)], dtype=torch.int32, device=device)
+        _EXP_CONSTANTS[key] = t
+    return t
 
 
 def _planted_absmax(shift: int, target_bits: int, device) -> torch.Tensor:
@@ -51,7 +63,12 @@ def _planted_absmax(shift: int, target_bits: int, device) -> torch.Tensor:
     bits = target_bits + int(shift)
     if not 1 <= int(shift) or bits > 31:
         raise ValueError("shift %d out of range" % shift)
-    return torch.tensor([2 ** (bits - 1) + 1], dtype=torch.int64, device=device).to(torch.int32)
+    key = ("absmax", bits, str(device))
+    t = _EXP_CONSTANTS.get(key)
+    if t is None:
+        t = torch.tensor([2 ** (bits - 1) + 1], dtype=torch.int64, device=device).to(torch.int32)
+        _EXP_CONSTANTS[key] = t
+    return t
 
 
 def _standalone(x: torch.Tensor, shift: int, method: str, rand=None) -> torch.Tensor:
@@ -268,7 +285,12 @@ class UpdateWeight(Module):
         self.weight_exp = e if isinstance(e, torch.Tensor) else torch.tensor(float(e))
 
     def _wexp(self):
-        return _exp_tensor(self.weight_exp, self.weight.device)
+        """weight_exp (a host-side 0-d float tensor, as in the reference) as a cached device int32."""
+        cached = getattr(self, "_wexp_cache", None)
+        if cached is None or cached[0] is not self.weight_exp:
+            cached = (self.weight_exp, _exp_tensor(self.weight_exp, self.weight.device))
+            self._wexp_cache = cached
+        return cached[1]
 
     def weight_update(self, absmax=None, rand=None):
         g = self.grad_int32acc
