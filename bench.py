@@ -97,7 +97,9 @@ class ConvTriple:
                     self.events.append((e0, e1, conv_ops(BATCH, hw, c, k)))
                 ops.requant(dx, am[1:2], 7, "round")
             # weight gradient + gradient rounding + weight update
-            dw = ops.conv2d_wgrad(L["x"], L["err"], 3, 3, 1, 1, f32_epilogue=(i > 0), absmax=am[2:3])
+            dw = ops.conv2d_wgrad(L["x16"], L["err"], 3, 3, 1, 1, f32_epilogue=(i > 0), absmax=am[2:3])
+            if c % 16:
+                dw = dw[..., :c].contiguous()     # zero-padded input channels give zero gradient columns
             ops.grad_update(dw, L["w"], am[2:3], 5, "psto")
 
 

@@ -17,6 +17,8 @@ struct ConvArgs {
   int dense_out;     // y is plain [M][K] with K % 4 == 0: 16-byte stores allowed
   unsigned flags;
   long long x_bytes, w_bytes;  // extents of x and w, for the buffer descriptors
+  long long y_bytes;           // extent of a dense y (0 otherwise)
+  int pq_shift, q_shift;       // log2(P*Q), log2(Q) when both are powers of two, else -1
   int tile_override;           // 0: heuristic; 1..4 force a tile configuration (tuning)
 };
 

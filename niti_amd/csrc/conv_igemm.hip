@@ -202,7 +202,7 @@ static int tile_override_from_env() {
   if (v < 0) {
     const char* e = getenv("NITI_CONV_TILE");
     v = e ? atoi(e) : 0;
-    if (v < 0 || v > 4) v = 0;
+    if (v < 0 || v > 6) v = 0;
   }
   return v;
 }
@@ -230,6 +230,15 @@ int launch_conv_igemm(const ConvProblem& p, hipStream_t stream) {
   a.x_bytes = static_cast<long long>(p.N) * p.H * p.W * p.C;
   a.w_bytes = static_cast<long long>(p.K) * a.Kg;
   a.tile_override = tile_override_from_env();
+  a.y_bytes = a.dense_out ? static_cast<long long>(a.M) * p.K * 4 : 0;
+  a.pq_shift = a.q_shift = -1;
+  {
+    const int pq = a.P * a.Q;
+    if ((pq & (pq - 1)) == 0 && (a.Q & (a.Q - 1)) == 0) {
+      a.pq_shift = __builtin_ctz(pq);
+      a.q_shift = __builtin_ctz(a.Q);
+    }
+  }
   int split = p.split_k < 1 ? 1 : p.split_k;
   if (split > a.kiters) split = a.kiters;
   a.kiters_per_split = (a.kiters + split - 1) / split;

@@ -18,6 +18,8 @@
 // tile, so activations are read from L2 once instead of nine times.  The pixel range is split
 // over gridDim.z workgroups; each writes its partial sums to a workspace slice and a second
 // kernel adds the slices (integer addition: any split gives the same result).
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace niti {
@@ -269,7 +271,13 @@ long long slice_stride_for(int C, int K) {
 int pick_splits(int N, int Q, int C, int K) {
   const int bands = N * Q * Q / 128;
   const int tiles = ((K + 127) / 128) * ((C + 63) / 64);
-  int splits = (256 + tiles - 1) / tiles;  // one workgroup per compute unit
+  static int target = -1;
+  if (target < 0) {
+    const char* e = getenv("NITI_WGRAD_BLOCKS");
+    target = e ? atoi(e) : 192;  // fewer, longer workgroups: less partial-sum traffic per MFMA
+    if (target < 1) target = 192;
+  }
+  int splits = (target + tiles - 1) / tiles;
   if (splits > bands) splits = bands;
   if (splits < 1) splits = 1;
   const int per = (bands + splits - 1) / splits;
