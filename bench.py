@@ -196,6 +196,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train-step", action="store_true")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a captured HIP graph")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run three plain 256 MiB device copies (a kernel of known traffic, to scale "
+                         "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -209,6 +212,14 @@ def main():
         return 3
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
+
+    if args.calibrate_copy:
+        src = torch.ones(256 << 20, dtype=torch.int8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(3):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     wl = ConvTriple(dev)
     run, mode = make_runner(wl.step, args.warmup, not args.eager)
@@ -236,7 +247,7 @@ def main():
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("conv_igemm_i8_kernel_bytes_per_launch")
+            traffic = json.load(f).get("bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic,
                 "kernel": "conv_mfma_kernel<..., false>", "launches": n_launch,

@@ -1,0 +1,141 @@
+"""CPU-only checks of the C-ABI library: it loads, exports every symbol the header declares, the
+host-side pieces (bit-width rule, argument validation, workspace sizing) behave, and the Python
+package refuses to run without it.  No kernel is launched here."""
+import ctypes as C
+import os
+import re
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "niti_gfx950.h")
+
+
+@pytest.fixture(scope="module")
+def lib():
+    from niti_amd import _lib
+    if not os.path.exists(_lib.SO_PATH):
+        from niti_amd import build
+        build.build()
+    return _lib.lib()
+
+
+def declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(niti_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_every_declared_symbol_is_exported_and_bound(lib):
+    from niti_amd import _lib
+    names = declared_symbols()
+    assert len(names) >= 20
+    for n in names:
+        assert hasattr(lib, n), "library does not export " + n
+        assert n in _lib.SIGNATURES, "ctypes signature table misses " + n
+    assert sorted(_lib.SIGNATURES) == names, "signature table lists symbols the header does not declare"
+
+
+def test_header_cites_the_reference_interfaces():
+    text = open(HEADER).read()
+    for cite in ("cutlassconv.cpp:57-73", "int8mm.cpp:9-14", "int8pool.cpp:37-57", "int8conv.cpp:35-44",
+                 "ti_torch.py:103-147", "ti_torch.py:16-21", "ti_torch.py:403-405", "ti_torch.py:430-432"):
+        assert cite in text, cite
+
+
+def test_version_and_status_strings(lib):
+    assert lib.niti_version() >= 100
+    assert lib.niti_status_string(0) == b"ok"
+    assert b"invalid" in lib.niti_status_string(1)
+    assert lib.niti_status_string(99) == b"unknown status"
+
+
+def test_bitwidth_rule_matches_the_oracle(lib, kat):
+    from oracle import niti_oracle as po
+    for r, bw in kat["bitwidth_int"].items():
+        assert lib.niti_bitwidth(int(r), 0) == bw
+    for r, bw in kat["bitwidth_f32"].items():
+        assert lib.niti_bitwidth(int(r), 1) == bw
+    for k in range(1, 31):
+        for d in range(-3, 12):
+            r = 2 ** k + d
+            if r < 0:
+                continue
+            assert lib.niti_bitwidth(r, 0) == po.bitwidth_int(r), r
+            assert lib.niti_bitwidth(r, 1) == po.bitwidth_f32(r), r     # torch CPU log2, literal reference form
+
+
+def test_argument_validation_without_a_gpu(lib):
+    from niti_amd import _lib
+    null = None
+    # null pointers / bad extents are rejected before any HIP call
+    st = lib.niti_conv2d_i8_fprop(null, null, null, 1, 8, 8, 16, 16, 3, 3, 1, 1, 0, null, null)
+    assert st == 1 and b"null" in lib.niti_last_error()
+    st = lib.niti_conv2d_i8_fprop(null, null, null, 0, 8, 8, 16, 16, 3, 3, 1, 1, 0, null, null)
+    assert st == 1
+    buf = (C.c_char * 4096)()
+    p = C.addressof(buf) + (-C.addressof(buf)) % 16
+    st = lib.niti_conv2d_i8_fprop(p, p, p, 1, 4, 4, 3, 4, 3, 3, 1, 1, 0, null, null)      # C not a multiple of 16
+    assert st == 2 and b"multiple of 16" in lib.niti_last_error()
+    st = lib.niti_conv2d_i8_fprop(p + 1, p, p, 1, 4, 4, 16, 4, 3, 3, 1, 1, 0, null, null)  # misaligned
+    assert st == 1 and b"aligned" in lib.niti_last_error()
+    st = lib.niti_conv2d_i8_dgrad(p, p, p, 1, 4, 4, 16, 16, 3, 3, 2, 1, 0, null, p, 4096, null)  # stride 2
+    assert st == 2
+    st = lib.niti_conv2d_i8_wgrad(p, p, p, 4, 8, 8, 16, 16, 3, 3, 1, 1, 0, null, null, 0, null)  # no workspace
+    assert st == 3 and b"workspace" in lib.niti_last_error()
+    st = lib.niti_requant_i32_i8(p, p, 16, p, 9, 0, 0, 0, null, 0, null, null, null, null, null)  # target_bits 9
+    assert st == 1
+    st = lib.niti_requant_i32_i8(p, p, 16, p, 7, 1, 0, 0, null, 0, null, null, null, null, null)  # sto without rand
+    assert st == 1 and b"rand" in lib.niti_last_error()
+    st = lib.niti_maxpool_i8_fwd(p, p, 1, 4, 4, 16, 2, 0, 0, null)                               # stride 0
+    assert st == 1
+    st = lib.niti_gemm_i8(0, 1, p, p, p, 0, 4, 4, 0, null, null, 0, null)
+    assert st == 1
+    # empty inputs are fine
+    assert lib.niti_absmax_i32(null, 0, null, null) == 0
+    assert lib.niti_fill_u32(null, 0, 0, null) == 0
+    assert lib.niti_last_error() == b""
+
+
+def test_workspace_sizes(lib):
+    # re-laid filter of the data gradient: one byte per filter element, rounded to 256
+    assert lib.niti_conv2d_i8_dgrad_workspace(128, 256, 3, 3) == 128 * 256 * 9
+    assert lib.niti_conv2d_i8_dgrad_workspace(3, 10, 3, 3) == 512
+    # direct GEMM form needs nothing when k is a multiple of 16
+    assert lib.niti_gemm_i8_workspace(0, 1, 128, 1024, 8192) == 0
+    assert lib.niti_gemm_i8_workspace(0, 1, 128, 10, 100) > 0
+    assert lib.niti_gemm_i8_workspace(0, 0, 128, 1024, 8192) == 1024 * 8192
+    assert lib.niti_gemm_i8_workspace(1, 0, 128, 1024, 8192) == 128 * 8192 + 1024 * 8192
+    # weight gradient: native 3x3 path = partial-sum slices, generic path = two transposed copies
+    n = lib.niti_conv2d_i8_wgrad_workspace(128, 32, 32, 128, 128, 3, 3, 1)
+    assert n >= 128 * 9 * 128 * 4 and n % 256 == 0
+    g = lib.niti_conv2d_i8_wgrad_workspace(5, 7, 9, 40, 24, 3, 3, 1)
+    assert g >= 16 * 7 * 9 * (40 + 24)
+    assert lib.niti_conv2d_i8_wgrad_workspace(0, 7, 9, 40, 24, 3, 3, 1) == 0
+
+
+def test_package_fails_loudly_without_the_library(tmp_path):
+    """The product has no CPU fallback: importing the ops with the shared object missing raises."""
+    code = (
+        "import sys, os\n"
+        "sys.path.insert(0, %r)\n"
+        "from niti_amd import _lib\n"
+        "_lib.SO_PATH = os.path.join(%r, 'missing.so')\n"
+        "try:\n"
+        "    _lib.lib()\n"
+        "except ImportError as e:\n"
+        "    print('ImportError', 'no fallback' in str(e))\n"
+    ) % (ROOT, str(tmp_path))
+    out = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=120)
+    assert "ImportError True" in out.stdout, out.stdout + out.stderr
+
+
+def test_product_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "niti_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert "oracle" not in text, os.path.join(dirpath, f)
