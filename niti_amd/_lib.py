@@ -12,7 +12,7 @@ SO_PATH = os.path.join(_HERE, "libniti_gfx950.so")
 
 OK = 0
 EPI_F32_ROUNDTRIP = 1
-DGRAD_FILTER_PREPARED = 2
+CONV_FILTER_PREPARED = 2
 RQ_RELU = 1
 ROUND = {"round": 0, "sto": 1, "psto": 2}
 DIV = {"floor": 0, "trunc": 1}
@@ -28,10 +28,10 @@ SIGNATURES = {
     "niti_last_error": (C.c_char_p, []),
     "niti_bitwidth": (_i, [C.c_uint32, _i]),
     "niti_fill_u32": (_i, [_vp, _i64, C.c_uint32, _vp]),
-    "niti_conv2d_i8_fprop": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp]),
-    "niti_conv2d_i8_dgrad_workspace": (_sz, [_i] * 4),
+    "niti_conv2d_i8_filter_workspace": (_sz, [_i] * 10),
+    "niti_conv2d_i8_filter_prepare": (_i, [_vp, _vp, _sz] + [_i] * 10 + [_vp]),
+    "niti_conv2d_i8_fprop": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp, _sz, _vp]),
     "niti_conv2d_i8_dgrad": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp, _sz, _vp]),
-    "niti_filter_dgrad_layout_i8": (_i, [_vp, _vp, _i, _i, _i, _i, _vp]),
     "niti_conv2d_i8_wgrad_workspace": (_sz, [_i] * 8),
     "niti_conv2d_i8_wgrad": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp, _sz, _vp]),
     "niti_gemm_i8_workspace": (_sz, [_i] * 5),

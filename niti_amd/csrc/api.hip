@@ -1,6 +1,7 @@
 // extern "C" surface of libniti_gfx950: argument checking, workspace carving and the
 // composition of kernels behind each entry point declared in include/niti_gfx950.h.
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include "common.h"
@@ -77,22 +78,82 @@ static int check_conv_dims(const char* who, int N, int H, int W, int C, int K, i
   return NITI_OK;
 }
 
+static bool halo_off() {
+  static int v = -1;
+  if (v < 0) {
+    const char* e = getenv("NITI_NO_HALO");
+    v = (e && e[0] == '1') ? 1 : 0;
+  }
+  return v == 1;
+}
+
+// which filter copy a convolution of this shape uses: 0 none (w as stored), 1 flipped/transposed
+// [C][R][S][K] (data gradient through the generic kernel), 2 / 3 tap-major blocks of the halo kernel
+// (forward / data gradient)
+static int filter_copy_kind(int N, int H, int W, int C, int K, int R, int S, int stride, int pad, int dgrad) {
+  if (!dgrad) return (!halo_off() && conv3x3_halo_supported(N, H, W, C, K, R, S, stride, pad)) ? 2 : 0;
+  if (stride != 1 || R != S || pad > R - 1) return 1;
+  const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
+  return (!halo_off() && conv3x3_halo_supported(N, P, Q, K, C, R, S, 1, R - 1 - pad)) ? 3 : 1;
+}
+
+extern "C" size_t niti_conv2d_i8_filter_workspace(int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                                                  int dgrad) {
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0) return 0;
+  switch (filter_copy_kind(N, H, W, C, K, R, S, stride, pad, dgrad)) {
+    case 1: return round256(static_cast<size_t>(C) * R * S * K);
+    case 2: return conv3x3_halo_filter_bytes(C, K);
+    case 3: return conv3x3_halo_filter_bytes(K, C);
+    default: return 0;
+  }
+}
+
+extern "C" int niti_conv2d_i8_filter_prepare(const int8_t* w, int8_t* dst, size_t dst_bytes, int N, int H, int W, int C,
+                                             int K, int R, int S, int stride, int pad, int dgrad, void* stream) {
+  clear_error();
+  int st = check_conv_dims("filter_prepare", N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
+  const size_t need = niti_conv2d_i8_filter_workspace(N, H, W, C, K, R, S, stride, pad, dgrad);
+  if (need == 0) return NITI_OK;
+  if (w == nullptr || dst == nullptr || dst_bytes < need || !aligned16(dst))
+    return fail(NITI_ERR_WORKSPACE, "filter_prepare: needs %zu bytes (16-byte aligned), got %zu", need, dst_bytes);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  switch (filter_copy_kind(N, H, W, C, K, R, S, stride, pad, dgrad)) {
+    case 1: return launch_filter_flip_transpose(w, dst, K, R, S, C, s);
+    case 2: return launch_halo_filter_prepare(w, dst, K, C, 0, s);
+    case 3: return launch_halo_filter_prepare(w, dst, C, K, 1, s);
+    default: return NITI_OK;
+  }
+}
+
 extern "C" int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y, int N, int H, int W, int C, int K,
-                                    int R, int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* stream) {
+                                    int R, int S, int stride, int pad, unsigned flags, uint32_t* absmax, void* workspace,
+                                    size_t workspace_bytes, void* stream) {
   clear_error();
   int st = check_conv_dims("conv_fprop", N, H, W, C, K, R, S, stride, pad);
   if (st != NITI_OK) return st;
   if (x == nullptr || w == nullptr || y == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: null pointer");
   if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: pointers must be 16-byte aligned");
+  if (C % 16 != 0) return fail(NITI_ERR_UNSUPPORTED, "conv: C=%d must be a multiple of 16", C);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  const int kind = filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 0);
+  if (kind == 2) {
+    const int8_t* wp = nullptr;
+    if (flags & NITI_CONV_FILTER_PREPARED) {
+      wp = w;
+    } else if (workspace != nullptr && aligned16(workspace) && workspace_bytes >= conv3x3_halo_filter_bytes(C, K)) {
+      st = launch_halo_filter_prepare(w, static_cast<int8_t*>(workspace), K, C, 0, s);
+      if (st != NITI_OK) return st;
+      wp = static_cast<const int8_t*>(workspace);
+    }
+    if (wp != nullptr) return launch_conv3x3_halo(x, wp, y, N, H, C, K, flags, absmax, s);
+  } else if (flags & NITI_CONV_FILTER_PREPARED) {
+    // no copy exists for this shape: filter_prepare wrote nothing, so `w` must be the filter itself
+  }
   const int P = (H + 2 * pad - R) / stride + 1, Q = (W + 2 * pad - S) / stride + 1;
   ConvProblem p{x, w, y, absmax, N, H, W, C, K, R, S, stride, pad,
                 static_cast<long long>(P) * Q * K, static_cast<long long>(Q) * K, K, 1, 1, flags};
-  return launch_conv_igemm(p, static_cast<hipStream_t>(stream));
-}
-
-extern "C" size_t niti_conv2d_i8_dgrad_workspace(int C, int K, int R, int S) {
-  if (C <= 0 || K <= 0 || R <= 0 || S <= 0) return 0;
-  return round256(static_cast<size_t>(C) * R * S * K);
+  return launch_conv_igemm(p, s);
 }
 
 extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N, int H, int W, int C, int K,
@@ -107,12 +168,14 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
   if (K % 16 != 0) return fail(NITI_ERR_UNSUPPORTED, "conv_dgrad: K=%d must be a multiple of 16", K);
   if (!aligned16(err) || !aligned16(dx)) return fail(NITI_ERR_INVALID_ARG, "conv_dgrad: pointers must be 16-byte aligned");
   hipStream_t s = static_cast<hipStream_t>(stream);
+  const int kind = filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 1);
   const int8_t* wt = w;
-  if (!(flags & NITI_DGRAD_FILTER_PREPARED)) {
-    const size_t need = niti_conv2d_i8_dgrad_workspace(C, K, R, S);
+  if (!(flags & NITI_CONV_FILTER_PREPARED)) {
+    const size_t need = niti_conv2d_i8_filter_workspace(N, H, W, C, K, R, S, stride, pad, 1);
     if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
       return fail(NITI_ERR_WORKSPACE, "conv_dgrad: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
-    st = launch_filter_flip_transpose(w, static_cast<int8_t*>(workspace), K, R, S, C, s);
+    st = kind == 3 ? launch_halo_filter_prepare(w, static_cast<int8_t*>(workspace), C, K, 1, s)
+                   : launch_filter_flip_transpose(w, static_cast<int8_t*>(workspace), K, R, S, C, s);
     if (st != NITI_OK) return st;
     wt = static_cast<const int8_t*>(workspace);
   } else if (!aligned16(w)) {
@@ -120,16 +183,10 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
   }
   const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
   // fprop over the error map: "input" [N,P,Q,K], "filter" [C,R,S,K], padding R-1-pad -> [N,H,W,C]
+  if (kind == 3) return launch_conv3x3_halo(err, wt, dx, N, P, K, C, flags, absmax, s);
   ConvProblem p{err, wt, dx, absmax, N, P, Q, K, C, R, S, 1, R - 1 - pad,
                 static_cast<long long>(H) * W * C, static_cast<long long>(W) * C, C, 1, 1, flags};
   return launch_conv_igemm(p, s);
-}
-
-extern "C" int niti_filter_dgrad_layout_i8(const int8_t* w, int8_t* dst, int K, int R, int S, int C, void* stream) {
-  clear_error();
-  if (w == nullptr || dst == nullptr || K <= 0 || R <= 0 || S <= 0 || C <= 0)
-    return fail(NITI_ERR_INVALID_ARG, "filter_dgrad_layout: bad arguments");
-  return launch_filter_flip_transpose(w, dst, K, R, S, C, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad) {

@@ -116,4 +116,11 @@ size_t wgrad3x3_workspace(int N, int H, int C, int K);
 int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, int H, int C, int K, bool roundtrip,
                     uint32_t* absmax, void* workspace, hipStream_t stream);
 
+// 3x3 / stride 1 / pad 1 forward kernel with LDS-resident activation halo (conv3x3_halo.hip)
+bool conv3x3_halo_supported(int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
+size_t conv3x3_halo_filter_bytes(int C, int K);
+int launch_halo_filter_prepare(const int8_t* w, int8_t* dst, int kout, int cin, int mode, hipStream_t stream);
+int launch_conv3x3_halo(const int8_t* x, const int8_t* wp, int32_t* y, int N, int H, int C, int K, unsigned flags,
+                        uint32_t* absmax, hipStream_t stream);
+
 }  // namespace niti

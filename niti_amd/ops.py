@@ -37,9 +37,26 @@ def _flags(f32_epilogue: bool) -> int:
     return L.EPI_F32_ROUNDTRIP if f32_epilogue else 0
 
 
-def conv2d_fprop(x, w, stride=1, padding=1, f32_epilogue=False, absmax: Optional[torch.Tensor] = None):
-    """x [N,H,W,C] int8, w [K,R,S,C] int8 -> [N,P,Q,K] int32."""
-    _chk_dev(x, w, absmax)
+def conv_filter_prepare(w, N, H, W, stride=1, padding=1, dgrad=False):
+    """Kernel-ready copy of the [K,R,S,C] filter for a convolution over an [N,H,W,*] input (forward) or
+    the data gradient of one (dgrad=True).  Returns None when the kernels read the filter as stored."""
+    _chk_dev(w)
+    K, R, S, C = w.shape
+    nbytes = L.lib().niti_conv2d_i8_filter_workspace(N, H, W, C, K, R, S, stride, padding, int(dgrad))
+    if nbytes == 0:
+        return None
+    dst = torch.empty(nbytes, dtype=torch.int8, device=w.device)
+    st = L.lib().niti_conv2d_i8_filter_prepare(_ptr(w), _ptr(dst), nbytes, N, H, W, C, K, R, S, stride, padding,
+                                               int(dgrad), _stream(w))
+    L.check(st, "niti_conv2d_i8_filter_prepare")
+    return dst
+
+
+def conv2d_fprop(x, w, stride=1, padding=1, f32_epilogue=False, absmax: Optional[torch.Tensor] = None,
+                 prepared_filter=None):
+    """x [N,H,W,C] int8, w [K,R,S,C] int8 -> [N,P,Q,K] int32.  ``prepared_filter``: the output of
+    conv_filter_prepare(w, N, H, W, stride, padding), to keep the filter copy out of the call."""
+    _chk_dev(x, w, absmax, prepared_filter)
     if x.dtype != torch.int8 or w.dtype != torch.int8:
         raise RuntimeError("conv2d_fprop: int8 tensors expected")
     N, H, W, C = x.shape
@@ -49,24 +66,22 @@ def conv2d_fprop(x, w, stride=1, padding=1, f32_epilogue=False, absmax: Optional
     P = (H + 2 * padding - R) // stride + 1
     Q = (W + 2 * padding - S) // stride + 1
     y = torch.empty((N, max(P, 0), max(Q, 0), K), dtype=torch.int32, device=x.device)
-    st = L.lib().niti_conv2d_i8_fprop(_ptr(x), _ptr(w), _ptr(y), N, H, W, C, K, R, S, stride, padding,
-                                      _flags(f32_epilogue), _ptr(absmax), _stream(x))
+    flags = _flags(f32_epilogue)
+    if prepared_filter is not None:
+        st = L.lib().niti_conv2d_i8_fprop(_ptr(x), _ptr(prepared_filter), _ptr(y), N, H, W, C, K, R, S, stride, padding,
+                                          flags | L.CONV_FILTER_PREPARED, _ptr(absmax), None, 0, _stream(x))
+    else:
+        nbytes = L.lib().niti_conv2d_i8_filter_workspace(N, H, W, C, K, R, S, stride, padding, 0)
+        ws = torch.empty(nbytes, dtype=torch.int8, device=x.device) if nbytes else None
+        st = L.lib().niti_conv2d_i8_fprop(_ptr(x), _ptr(w), _ptr(y), N, H, W, C, K, R, S, stride, padding, flags,
+                                          _ptr(absmax), _ptr(ws), nbytes, _stream(x))
     L.check(st, "niti_conv2d_i8_fprop")
     return y
 
 
-def filter_dgrad_layout(w):
-    """w [K,R,S,C] int8 -> [C,R,S,K] int8 with flipped taps (the data gradient's filter operand)."""
-    _chk_dev(w)
-    K, R, S, C = w.shape
-    dst = torch.empty((C, R, S, K), dtype=torch.int8, device=w.device)
-    L.check(L.lib().niti_filter_dgrad_layout_i8(_ptr(w), _ptr(dst), K, R, S, C, _stream(w)), "niti_filter_dgrad_layout_i8")
-    return dst
-
-
 def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None, prepared_filter=None):
     """err [N,P,Q,K] int8, w [K,R,S,C] int8 -> dx [N,H,W,C] int32 (stride 1).  ``prepared_filter``:
-    the output of filter_dgrad_layout(w), to skip the re-layout inside the call."""
+    the output of conv_filter_prepare(w, N, H, W, stride, padding, dgrad=True)."""
     _chk_dev(err, w, absmax, prepared_filter)
     N, P, Q, K = err.shape
     K2, R, S, C = w.shape
@@ -78,9 +93,9 @@ def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None, p
     flags = _flags(f32_epilogue)
     if prepared_filter is not None:
         st = L.lib().niti_conv2d_i8_dgrad(_ptr(err), _ptr(prepared_filter), _ptr(dx), N, H, W, C, K, R, S, stride, padding,
-                                          flags | L.DGRAD_FILTER_PREPARED, _ptr(absmax), None, 0, _stream(err))
+                                          flags | L.CONV_FILTER_PREPARED, _ptr(absmax), None, 0, _stream(err))
     else:
-        nbytes = L.lib().niti_conv2d_i8_dgrad_workspace(C, K, R, S)
+        nbytes = L.lib().niti_conv2d_i8_filter_workspace(N, H, W, C, K, R, S, stride, padding, 1)
         ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=err.device)
         st = L.lib().niti_conv2d_i8_dgrad(_ptr(err), _ptr(w), _ptr(dx), N, H, W, C, K, R, S, stride, padding,
                                           flags, _ptr(absmax), _ptr(ws), nbytes, _stream(err))

@@ -71,15 +71,15 @@ def test_argument_validation_without_a_gpu(lib):
     from niti_amd import _lib
     null = None
     # null pointers / bad extents are rejected before any HIP call
-    st = lib.niti_conv2d_i8_fprop(null, null, null, 1, 8, 8, 16, 16, 3, 3, 1, 1, 0, null, null)
+    st = lib.niti_conv2d_i8_fprop(null, null, null, 1, 8, 8, 16, 16, 3, 3, 1, 1, 0, null, null, 0, null)
     assert st == 1 and b"null" in lib.niti_last_error()
-    st = lib.niti_conv2d_i8_fprop(null, null, null, 0, 8, 8, 16, 16, 3, 3, 1, 1, 0, null, null)
+    st = lib.niti_conv2d_i8_fprop(null, null, null, 0, 8, 8, 16, 16, 3, 3, 1, 1, 0, null, null, 0, null)
     assert st == 1
     buf = (C.c_char * 4096)()
     p = C.addressof(buf) + (-C.addressof(buf)) % 16
-    st = lib.niti_conv2d_i8_fprop(p, p, p, 1, 4, 4, 3, 4, 3, 3, 1, 1, 0, null, null)      # C not a multiple of 16
+    st = lib.niti_conv2d_i8_fprop(p, p, p, 1, 4, 4, 3, 4, 3, 3, 1, 1, 0, null, null, 0, null)      # C not a multiple of 16
     assert st == 2 and b"multiple of 16" in lib.niti_last_error()
-    st = lib.niti_conv2d_i8_fprop(p + 1, p, p, 1, 4, 4, 16, 4, 3, 3, 1, 1, 0, null, null)  # misaligned
+    st = lib.niti_conv2d_i8_fprop(p + 1, p, p, 1, 4, 4, 16, 4, 3, 3, 1, 1, 0, null, null, 0, null)  # misaligned
     assert st == 1 and b"aligned" in lib.niti_last_error()
     st = lib.niti_conv2d_i8_dgrad(p, p, p, 1, 4, 4, 16, 16, 3, 3, 2, 1, 0, null, p, 4096, null)  # stride 2
     assert st == 2
@@ -100,9 +100,12 @@ def test_argument_validation_without_a_gpu(lib):
 
 
 def test_workspace_sizes(lib):
-    # re-laid filter of the data gradient: one byte per filter element, rounded to 256
-    assert lib.niti_conv2d_i8_dgrad_workspace(128, 256, 3, 3) == 128 * 256 * 9
-    assert lib.niti_conv2d_i8_dgrad_workspace(3, 10, 3, 3) == 512
+    # filter copies: flipped/transposed filter for a generic data gradient (one byte per element, rounded to
+    # 256), tap-major 128 x 64 blocks for the 3x3 kernels, nothing when the kernel reads the filter as stored
+    assert lib.niti_conv2d_i8_filter_workspace(2, 9, 9, 3, 10, 5, 5, 1, 2, 1) == 768
+    assert lib.niti_conv2d_i8_filter_workspace(2, 9, 9, 16, 16, 5, 5, 1, 2, 0) == 0
+    assert lib.niti_conv2d_i8_filter_workspace(128, 32, 32, 128, 256, 3, 3, 1, 1, 0) == 2 * 2 * 9 * 128 * 64
+    assert lib.niti_conv2d_i8_filter_workspace(128, 32, 32, 128, 256, 3, 3, 1, 1, 1) == 1 * 4 * 9 * 128 * 64
     # direct GEMM form needs nothing when k is a multiple of 16
     assert lib.niti_gemm_i8_workspace(0, 1, 128, 1024, 8192) == 0
     assert lib.niti_gemm_i8_workspace(0, 1, 128, 10, 100) > 0

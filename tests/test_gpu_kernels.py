@@ -34,6 +34,12 @@ CONV_CASES = [  # N,H,W,C,K,R,S,stride,pad
     (2, 6, 6, 16, 8, 3, 3, 1, 0),        # no padding
     (8, 32, 32, 128, 128, 3, 3, 1, 1),
     (2, 40, 40, 16, 16, 36, 36, 1, 1),   # filter wider than 32 (the reference's sp_conv case)
+    (8, 8, 8, 64, 128, 3, 3, 1, 1),      # 3x3 kernel with LDS-resident halo: whole small images per workgroup
+    (4, 8, 8, 80, 24, 3, 3, 1, 1),       # ... ragged channel slice and channel tile
+    (1, 16, 16, 16, 40, 3, 3, 1, 1),
+    (2, 32, 32, 16, 64, 3, 3, 1, 1),
+    (3, 16, 16, 192, 260, 3, 3, 1, 1),   # three channel slices, three channel tiles
+    (12, 8, 8, 512, 128, 3, 3, 1, 1),
 ]
 
 
@@ -75,7 +81,7 @@ def test_conv_fprop_f32_epilogue_rounds_large_sums(dev):
     assert torch.equal(y.cpu(), ref)
 
 
-DGRAD_CASES = [(2, 8, 8, 16, 16, 3, 1), (2, 8, 8, 32, 48, 3, 1), (3, 7, 9, 40, 32, 3, 1), (2, 16, 16, 128, 128, 3, 1),
+DGRAD_CASES = [(4, 8, 8, 96, 48, 3, 1), (1, 32, 32, 32, 16, 3, 1), (2, 16, 16, 256, 128, 3, 1), (2, 8, 8, 16, 16, 3, 1), (2, 8, 8, 32, 48, 3, 1), (3, 7, 9, 40, 32, 3, 1), (2, 16, 16, 128, 128, 3, 1),
                (2, 8, 8, 16, 32, 5, 2), (2, 8, 8, 24, 16, 3, 0), (2, 6, 6, 3, 16, 3, 1)]
 
 
