@@ -63,6 +63,15 @@ class ConvTriple:
             L["x16"] = F.pad(L["x"], (0, 16 - c % 16)).contiguous() if c % 16 else L["x"]
             self.layers.append(L)
         self.absmax = torch.zeros(3 * len(LAYERS), dtype=torch.int32, device=dev)
+        # zeroed words the single-launch conv + requantisation kernels exchange their tile ranges through
+        off = 0
+        for L in self.layers:
+            for key, dgrad in (("sync_f", False), ("sync_d", True)):
+                n = ops.conv_requant_sync_words(BATCH, L["hw"], L["hw"], L["x16"].shape[3] if not dgrad else L["c"], L["k"],
+                                                dgrad=dgrad)
+                L[key] = (off, n)
+                off += n
+        self.sync = torch.zeros(max(off, 1), dtype=torch.int32, device=dev)
         self.exp0 = torch.zeros(1, dtype=torch.int32, device=dev)
         self.ops_per_step = sum(conv_ops(BATCH, hw, c, k) * (2 if i == 0 else 3) for i, (c, k, hw) in enumerate(LAYERS))
         self.main_kernel_ops = []     # algorithmic ops of every launch bracketed by events, in launch order
@@ -72,6 +81,7 @@ class ConvTriple:
         torch, ops = self.torch, self.ops
         import torch.nn.functional as F
         self.absmax.zero_()
+        self.sync.zero_()
         for i, L in enumerate(self.layers):
             c, k, hw = L["c"], L["k"], L["hw"]
             am = self.absmax[3 * i: 3 * i + 3]
@@ -81,22 +91,34 @@ class ConvTriple:
             if record:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
-            acc = ops.conv2d_fprop(L["x16"], w16, 1, 1, f32_epilogue=True, absmax=am[0:1], prepared_filter=wp)
+            so, sn = L["sync_f"]
+            if sn:
+                ops.conv2d_fprop_requant(L["x16"], w16, 1, 1, f32_epilogue=True, sync=self.sync[so:so + sn], exp_a=self.exp0,
+                                         exp_b=self.exp0, exp_out=torch.empty_like(self.exp0), prepared_filter=wp)
+            else:
+                acc = ops.conv2d_fprop(L["x16"], w16, 1, 1, f32_epilogue=True, absmax=am[0:1], prepared_filter=wp)
             if record:
                 e1.record()
                 self.events.append((e0, e1, conv_ops(BATCH, hw, c, k)))
-            ops.requant(acc, am[0:1], 7, "round", exp_a=self.exp0, exp_b=self.exp0, exp_out=torch.empty_like(self.exp0))
+            if not sn:
+                ops.requant(acc, am[0:1], 7, "round", exp_a=self.exp0, exp_b=self.exp0, exp_out=torch.empty_like(self.exp0))
             # data gradient + error requantisation
             if i > 0:
                 wt = ops.conv_filter_prepare(L["w"], BATCH, hw, hw, dgrad=True)
                 if record:
                     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     e0.record()
-                dx = ops.conv2d_dgrad(L["err"], L["w"], 1, 1, f32_epilogue=True, absmax=am[1:2], prepared_filter=wt)
+                so, sn = L["sync_d"]
+                if sn:
+                    ops.conv2d_dgrad_requant(L["err"], L["w"], 1, 1, f32_epilogue=True, sync=self.sync[so:so + sn],
+                                             prepared_filter=wt)
+                else:
+                    dx = ops.conv2d_dgrad(L["err"], L["w"], 1, 1, f32_epilogue=True, absmax=am[1:2], prepared_filter=wt)
                 if record:
                     e1.record()
                     self.events.append((e0, e1, conv_ops(BATCH, hw, c, k)))
-                ops.requant(dx, am[1:2], 7, "round")
+                if not sn:
+                    ops.requant(dx, am[1:2], 7, "round")
             # weight gradient + gradient rounding + weight update
             dw = ops.conv2d_wgrad(L["x16"], L["err"], 3, 3, 1, 1, f32_epilogue=(i > 0), absmax=am[2:3])
             if c % 16:
@@ -251,7 +273,7 @@ def main():
             traffic = json.load(f).get("bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic,
-                "kernel": "conv_mfma_kernel<..., false>", "launches": n_launch,
+                "kernel": "conv3x3_halo_kernel<..., true> (convolution + requantisation)", "launches": n_launch,
                 "avg_launch_us": round(k_ms * 1e3 / max(n_launch, 1), 2),
                 "ops_per_launch_avg": k_ops / max(n_launch, 1),
                 "note": "int8 multiply-accumulate counted as 2 ops; unit is tera-ops/s"}

@@ -100,6 +100,41 @@ int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N,
                          size_t workspace_bytes, void* stream);
 
 /*
+ * Convolution and requantisation in one launch.  Replaces the pairs
+ *   cutlassconv_cuda.sp_conv_optimized + act_calc   (TiConv2d.forward,  ti_torch.py:393-397 with 103-117)
+ *   cutlassconv_cuda.sp_conv_optimized + err_calc   (TiConv2d.backward, ti_torch.py:403-407 with 119-133)
+ * with the same result as niti_conv2d_i8_fprop / _dgrad followed by niti_requant_i32_i8, bit for bit,
+ * but the int32 sums stay in registers: every workgroup publishes the largest magnitude of its tile,
+ * waits for all others, derives the tensor-wide shift and stores int8.
+ *
+ * Covered: 3x3, stride 1, pad 1, square inputs of side 8, 16 or 32, N*H*W % 256 == 0, input channels % 16 == 0,
+ * output channels % 16 == 0, rounding NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC, and a launch whose
+ * workgroups (N*H*W/256 x ceil(out channels/128)) all fit on the device at once.  niti_conv2d_i8_requant_sync_words
+ * returns 0 for shapes outside that (then use the two-pass entry points); the entry points return
+ * NITI_ERR_UNSUPPORTED for them and for a device too small for the launch.
+ *
+ * sync: niti_conv2d_i8_requant_sync_words(...) uint32 words that are ZERO on entry (niti_fill_u32).  On return
+ * word 0 holds max |sum| over the tensor; word 1 is non-zero if the wait for the other workgroups ran into its
+ * time limit (10 s, or NITI_SYNC_TIMEOUT_MS from the environment), in which case the output is invalid - this
+ * can only happen when other work keeps part of the device busy that long.  Launches that share a sync buffer
+ * must not overlap.
+ * flags: NITI_EPI_F32_ROUNDTRIP, NITI_CONV_FILTER_PREPARED (w is a copy made by niti_conv2d_i8_filter_prepare;
+ * otherwise workspace must hold niti_conv2d_i8_filter_workspace bytes).  rq_flags: NITI_RQ_RELU.
+ * shift_out / exp_a / exp_b / exp_out as in niti_requant_i32_i8 (each may be NULL).
+ */
+size_t niti_conv2d_i8_requant_sync_words(int N, int H, int W, int C, int K, int R, int S, int stride, int pad, int dgrad);
+int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, int8_t* y8, int N, int H, int W, int C, int K, int R,
+                                 int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
+                                 int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
+                                 const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int N, int H, int W, int C, int K, int R,
+                                 int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
+                                 int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
+                                 const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
+/*
  * Weight gradient, replaces the reference's fprop-on-transposed-operands rewrite
  * (ti_torch.py:430-432) and, for the first layer, conv2d_weight_int8 -> group_conv
  * (ti_torch.py:194-233):

@@ -189,6 +189,82 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
   return launch_conv_igemm(p, s);
 }
 
+// ---- convolution + requantisation in one launch -------------------------------------------------------
+static int fused_blocks(int N, int H, int W, int C, int K, int R, int S, int stride, int pad, int dgrad) {
+  if (halo_off()) return 0;
+  if (!dgrad) return conv3x3_halo_requant_blocks(N, H, W, C, K, R, S, stride, pad);
+  if (stride != 1 || R != S || pad > R - 1) return 0;
+  const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;
+  return conv3x3_halo_requant_blocks(N, P, Q, K, C, R, S, 1, R - 1 - pad);
+}
+
+extern "C" size_t niti_conv2d_i8_requant_sync_words(int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
+                                                    int dgrad) {
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0) return 0;
+  const int nb = fused_blocks(N, H, W, C, K, R, S, stride, pad, dgrad);
+  return nb > 0 ? conv3x3_halo_sync_words(nb) : 0;
+}
+
+static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_t* w, int8_t* y8, int N, int H, int W, int C,
+                        int K, int R, int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
+                        int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
+                        const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace, size_t workspace_bytes,
+                        void* stream) {
+  clear_error();
+  int st = check_conv_dims(who, N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
+  if (x == nullptr || w == nullptr || y8 == nullptr || sync == nullptr) return fail(NITI_ERR_INVALID_ARG, "%s: null pointer", who);
+  if (!aligned16(x) || !aligned16(w) || !aligned16(y8)) return fail(NITI_ERR_INVALID_ARG, "%s: pointers must be 16-byte aligned", who);
+  if (target_bits < 1 || target_bits > 7) return fail(NITI_ERR_INVALID_ARG, "%s: target_bits=%d outside 1..7", who, target_bits);
+  if (method != NITI_ROUND_NEAREST && method != NITI_ROUND_PSEUDO_STOCHASTIC)
+    return fail(NITI_ERR_UNSUPPORTED, "%s: rounding method %d needs random input; use the two-pass path", who, method);
+  if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "%s: div_mode=%d", who, div_mode);
+  if (bw_mode != NITI_BW_INT && bw_mode != NITI_BW_F32) return fail(NITI_ERR_INVALID_ARG, "%s: bw_mode=%d", who, bw_mode);
+  const int nb = fused_blocks(N, H, W, C, K, R, S, stride, pad, dgrad);
+  if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "%s: shape not covered by the single-launch path; use the two-pass path", who);
+  if (sync_words < conv3x3_halo_sync_words(nb))
+    return fail(NITI_ERR_WORKSPACE, "%s: needs %zu zeroed sync words, got %zu", who, conv3x3_halo_sync_words(nb), sync_words);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // geometry of the forward problem the kernel runs: the data gradient is a forward pass over the error map
+  const int Hk = dgrad ? H + 2 * pad - R + 1 : H;
+  const int Ck = dgrad ? K : C, Kk = dgrad ? C : K;
+  const int8_t* wp = w;
+  if (!(flags & NITI_CONV_FILTER_PREPARED)) {
+    const size_t need = conv3x3_halo_filter_bytes(Ck, Kk);
+    if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+      return fail(NITI_ERR_WORKSPACE, "%s: needs %zu workspace bytes (16-byte aligned), got %zu", who, need, workspace_bytes);
+    st = launch_halo_filter_prepare(w, static_cast<int8_t*>(workspace), Kk, Ck, dgrad ? 1 : 0, s);
+    if (st != NITI_OK) return st;
+    wp = static_cast<const int8_t*>(workspace);
+  }
+  static long long spin_limit = -1;  // 100 MHz ticks; NITI_SYNC_TIMEOUT_MS overrides the 10 s default
+  if (spin_limit < 0) {
+    const char* e = getenv("NITI_SYNC_TIMEOUT_MS");
+    const long long ms = e != nullptr ? atoll(e) : 10000;
+    spin_limit = (ms > 0 ? ms : 1) * 100000LL;
+  }
+  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, spin_limit, shift_out, exp_a, exp_b, exp_out};
+  return launch_conv3x3_halo_requant(x, wp, y8, N, Hk, Ck, Kk, flags, sync, rq, s);
+}
+
+extern "C" int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, int8_t* y8, int N, int H, int W, int C, int K,
+                                            int R, int S, int stride, int pad, unsigned flags, int target_bits, int method,
+                                            int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words,
+                                            int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  return conv_requant("conv_fprop_requant", 0, x, w, y8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method, div_mode,
+                      bw_mode, rq_flags, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
+}
+
+extern "C" int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int N, int H, int W, int C, int K,
+                                            int R, int S, int stride, int pad, unsigned flags, int target_bits, int method,
+                                            int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words,
+                                            int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                            void* workspace, size_t workspace_bytes, void* stream) {
+  return conv_requant("conv_dgrad_requant", 1, err, w, dx8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method, div_mode,
+                      bw_mode, rq_flags, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
+}
+
 extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || pad < 0) return 0;
   const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;

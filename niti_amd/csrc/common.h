@@ -122,5 +122,19 @@ size_t conv3x3_halo_filter_bytes(int C, int K);
 int launch_halo_filter_prepare(const int8_t* w, int8_t* dst, int kout, int cin, int mode, hipStream_t stream);
 int launch_conv3x3_halo(const int8_t* x, const int8_t* wp, int32_t* y, int N, int H, int C, int K, unsigned flags,
                         uint32_t* absmax, hipStream_t stream);
+// requantisation parameters of the convolution that rounds its own sums to int8
+struct RequantSpec {
+  int target_bits, method, trunc, bw_mode;
+  unsigned flags;          // NITI_RQ_*
+  long long spin_limit;    // 100 MHz wall-clock ticks the grid-wide wait may last
+  int32_t* shift_out;
+  const int32_t* exp_a;
+  const int32_t* exp_b;
+  int32_t* exp_out;
+};
+int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
+size_t conv3x3_halo_sync_words(int blocks);
+int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, int N, int H, int C, int K, unsigned flags,
+                                uint32_t* sync, const RequantSpec& rq, hipStream_t stream);
 
 }  // namespace niti

@@ -12,11 +12,20 @@
 // About 23 bytes/clock/CU at MFMA peak.
 //
 // 8 wavefronts (4 pixel groups x 2 channel halves), each 64 pixels x 64 channels = 2x2 tiles of
-// v_mfma_i32_32x32x32_i8.  Halo slices are double buffered, filter stages run through a 3-deep
-// ring of filter rows (three taps each); one s_barrier per filter row, LDS fragment reads
-// software-pipelined one sub-step ahead of the MFMAs.  The same kernel computes the data gradient when given the
-// flipped / transposed filter arrangement (prepare kernel, mode 1).
+// v_mfma_i32_32x32x32_i8.  One halo buffer plus a 4-deep ring of filter taps keeps a workgroup
+// under 80 KB of LDS and 128 VGPRs, so two workgroups share a compute unit: while one waits for its
+// next halo slice, starts up or writes its results, the other one feeds the matrix cores.  The same
+// kernel computes the data gradient when given the flipped / transposed filter arrangement
+// (prepare kernel, mode 1).
+//
+// Requantising variant (kFused): the int32 sums never leave the registers.  Every workgroup publishes
+// the largest magnitude of its tile in a slot of its own, waits until the slots of all workgroups of the
+// launch are filled (they are all resident: the host refuses grids larger than the chip holds at once,
+// and the wait is bounded by a wall-clock limit so that every wavefront exits whatever happens), derives
+// the tensor-wide shift from the maximum over the slots and stores rounded int8.  Compared with the
+// int32 store + separate requantisation pass this removes 8 of the 9 bytes moved per output element.
 #include "common.h"
+#include "requant_math.h"
 
 namespace niti {
 namespace {
@@ -43,7 +52,20 @@ struct HaloArgs {
   int cslices;        // ceil(C / 64)
   long long x_bytes, wp_bytes, y_bytes;
   unsigned flags;
+  // requantising variant only
+  int8_t* y8;         // [N,Q,Q,K] int8
+  uint32_t* sync;     // word 0: max |sum| of the launch (output), word 1: set when the wait gave up,
+                      // words kSyncSlot0..: one slot per workgroup, max + 1; all zero on entry
+  long long y8_bytes;
+  int target_bits, method, trunc, bw_mode;
+  unsigned rq_flags;
+  long long spin_limit;  // wall-clock ticks (100 MHz) the wait may last
+  int32_t* shift_out;
+  const int32_t* exp_a;
+  const int32_t* exp_b;
+  int32_t* exp_out;
 };
+constexpr int kSyncSlot0 = 16;
 
 // Q: image width = height; BR: output rows of one image per workgroup; NI: images per workgroup; BR*NI*Q == 256
 template <int Q, int BR, int NI>
@@ -53,18 +75,18 @@ struct HGeom {
   static constexpr int ACT_INSTR = NI * HR * (RP / 16);
   static constexpr int ACT_BYTES = NI * HR * RP * 64;
   static constexpr int ACT_LOADS = (ACT_INSTR + 7) / 8;  // per wavefront per slice
-  static constexpr int W_BYTES = 3 * 128 * 64;           // one filter stage: the three taps of a filter row
-  static constexpr int WSTAGES = 3;
-  static constexpr int LDS_BYTES = 2 * ACT_BYTES + WSTAGES * W_BYTES + 1024;  // + dump slot
+  static constexpr int W_BYTES = 128 * 64;               // one filter stage: one tap
+  static constexpr int WSTAGES = 4;
+  static constexpr int LDS_BYTES = ACT_BYTES + WSTAGES * W_BYTES + 1024;  // + dump slot
   static_assert(BR * NI * Q == 256, "a workgroup owns 256 output pixels");
 };
 
-template <int Q, int BR, int NI>
-__global__ __launch_bounds__(512, 1) void conv3x3_halo_kernel(const HaloArgs a) {
+template <int Q, int BR, int NI, bool kFused>
+__global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) {
   using G = HGeom<Q, BR, NI>;
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
-  int8_t* const act_buf = smem;                         // 2 x ACT_BYTES
-  int8_t* const w_buf = smem + 2 * G::ACT_BYTES;        // WSTAGES x 8 KB
+  int8_t* const act_buf = smem;                         // ACT_BYTES
+  int8_t* const w_buf = smem + G::ACT_BYTES;            // WSTAGES x 8 KB
   int8_t* const dump = w_buf + G::WSTAGES * G::W_BYTES;
 
   const int tid = threadIdx.x;
@@ -101,8 +123,8 @@ __global__ __launch_bounds__(512, 1) void conv3x3_halo_kernel(const HaloArgs a) 
     act_off[i] = off;
     act_dst[i] = dst;
   }
-  auto issue_act = [&](int cs, int buf) {
-    int8_t* base = act_buf + buf * G::ACT_BYTES;
+  auto issue_act = [&](int cs) {
+    int8_t* base = act_buf;
 #pragma unroll
     for (int i = 0; i < G::ACT_LOADS; ++i) {
       // channel range check: the 16 bytes at slice offset cs*64 + piece*16 must lie inside C
@@ -116,15 +138,12 @@ __global__ __launch_bounds__(512, 1) void conv3x3_halo_kernel(const HaloArgs a) 
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, NITI_LDS(dst), 16, off, 0, 0, 0);
     }
   };
-  // ---- filter staging: stage (cs, r) is one contiguous 24 KB block (three taps); three KB per wavefront
-  const int wstep_base = (kt * a.cslices) * 3 * G::W_BYTES + wave * 1024 + lane * 16;
-  auto issue_w = [&](int step, int st) {  // step = cs * 3 + r
-#pragma unroll
-    for (int s = 0; s < 3; ++s) {
-      int8_t* dst = w_buf + st * G::W_BYTES + s * 8192 + wave * 1024;
-      const int off = wstep_base + step * G::W_BYTES + s * 8192;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
-    }
+  // ---- filter staging: stage (cs, tap) is one contiguous 8 KB block; one KB per wavefront
+  const int wstep_base = (kt * a.cslices) * 9 * G::W_BYTES + wave * 1024 + lane * 16;
+  auto issue_w = [&](int step, int st) {  // step = cs * 9 + tap
+    int8_t* dst = w_buf + st * G::W_BYTES + wave * 1024;
+    const int off = wstep_base + step * G::W_BYTES;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
   };
 
   // ---- fragment addressing
@@ -158,66 +177,62 @@ __global__ __launch_bounds__(512, 1) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  // ---- pipeline.  Per-wavefront load order: act(0), W(0), W(1), then inside stage t: W(t+2) and, at the
-  // first stage of every slice, act(next slice).  All waits are derived from that order.
-  // Every workgroup of a launch streams the same filter; started together they would all pull the same
-  // 24 KB through the same few L2 channels at the same time.  Integer sums do not depend on the order,
-  // so each workgroup starts at its own channel slice and filter row and wraps around.
-  const int nst = a.cslices * 3;
+  // ---- pipeline.  Per-wavefront load order: act(slice 0), W(0), W(1), W(2); inside step t: W(t+3); before
+  // the first step of every later slice: act(slice).  All waits are derived from that order.
+  // Every workgroup of a launch streams the same filter; integer sums do not depend on the order, so each
+  // workgroup starts at its own channel slice and filter row and wraps around, which spreads the
+  // simultaneous requests over the filter copy instead of piling them onto the same lines.
+  const int nst = a.cslices * 9;
   const int cs0 = blockIdx.x % a.cslices;
   const int r0 = (blockIdx.x / a.cslices) % 3;
   auto slice_of = [&](int ci) { const int c = ci + cs0; return c >= a.cslices ? c - a.cslices : c; };
-  auto stage_of = [&](int t) {  // t-th stage in this workgroup's order -> index in the filter copy
-    const int ci = t / 3, ri = t - ci * 3;
+  auto tap_of = [&](int ti) {  // ti-th tap in this workgroup's order
+    const int ri = ti / 3, s = ti - ri * 3;
     const int r = ri + r0 >= 3 ? ri + r0 - 3 : ri + r0;
-    return slice_of(ci) * 3 + r;
+    return r * 3 + s;
   };
-  issue_act(slice_of(0), 0);
+  auto stage_of = [&](int t) { const int ci = t / 9; return slice_of(ci) * 9 + tap_of(t - ci * 9); };
+  issue_act(slice_of(0));
   issue_w(stage_of(0), 0);
   if (1 < nst) issue_w(stage_of(1), 1);
+  if (2 < nst) issue_w(stage_of(2), 2);
   for (int ci = 0; ci < a.cslices; ++ci) {
-    const int8_t* sact = act_buf + (ci & 1) * G::ACT_BYTES;
+    if (ci > 0) {
+      hc_sync();  // every wavefront has finished reading the previous slice
+      issue_act(slice_of(ci));
+    }
 #pragma unroll
-    for (int ri = 0; ri < 3; ++ri) {
-      const int t = ci * 3 + ri;
-      // younger than W(t) and possibly still in flight: W(t+1); act(next slice), issued at ri == 0 after W(t+2)
-      const bool young_w = t + 1 < nst;
-      const bool young_act = ri >= 1 && ci + 1 < a.cslices;
-      if (young_act) {
-        if (young_w) hc_wait_vmcnt<3 + G::ACT_LOADS>();
-        else hc_wait_vmcnt<G::ACT_LOADS>();
-      } else {
-        if (young_w) hc_wait_vmcnt<3>();
-        else hc_wait_vmcnt<0>();
-      }
+    for (int ti = 0; ti < 9; ++ti) {
+      const int t = ci * 9 + ti;
+      // younger than W(t): W(t+1), W(t+2); the halo slice issued just above is the youngest of all
+      const int young = min(2, nst - 1 - t);
+      if (ti == 0 && ci > 0) hc_wait_vmcnt<0>();
+      else if (young == 2) hc_wait_vmcnt<2>();
+      else if (young == 1) hc_wait_vmcnt<1>();
+      else hc_wait_vmcnt<0>();
       hc_sync();
-      if (t + 2 < nst) issue_w(stage_of(t + 2), (t + 2) % G::WSTAGES);
-      if (ri == 0 && ci + 1 < a.cslices) issue_act(slice_of(ci + 1), (ci + 1) & 1);
-      const int r = ri + r0 >= 3 ? ri + r0 - 3 : ri + r0;
+      if (t + 3 < nst) issue_w(stage_of(t + 3), (t + 3) % G::WSTAGES);
+      const int tap = tap_of(ti);
+      const int r = tap / 3, s = tap - r * 3;
       const int8_t* sw = w_buf + (t % G::WSTAGES) * G::W_BYTES;
       const int roff = r * G::RP * 64;
-      // six sub-steps (three taps x two 32-byte reduction halves); fragments of sub-step i+1 are
-      // fetched from LDS before the MFMAs of sub-step i are issued
+      int pa[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) pa[j] = (s == 0 ? p_addr[j][0] : (s == 1 ? p_addr[j][1] : p_addr[j][2])) + roff;
       v4i wf[2][2], pf[2][2];
-      auto fetch = [&](int sub, int slot) {
-        const int s = sub >> 1, kk = sub & 1;
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
-          wf[slot][i] = *reinterpret_cast<const v4i*>(sw + s * 8192 + (w_addr[i] ^ (kk << 5)));
+      for (int kk = 0; kk < 2; ++kk) {
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
-          pf[slot][j] = *reinterpret_cast<const v4i*>(sact + ((p_addr[j][s] ^ (kk << 5)) + roff));
-      };
-      fetch(0, 0);
+        for (int i = 0; i < 2; ++i) wf[kk][i] = *reinterpret_cast<const v4i*>(sw + (w_addr[i] ^ (kk << 5)));
 #pragma unroll
-      for (int sub = 0; sub < 6; ++sub) {
-        if (sub + 1 < 6) fetch(sub + 1, (sub + 1) & 1);
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-          for (int j = 0; j < 2; ++j)
-            acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[sub & 1][i], pf[sub & 1][j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < 2; ++j) pf[kk][j] = *reinterpret_cast<const v4i*>(act_buf + (pa[j] ^ (kk << 5)));
       }
+#pragma unroll
+      for (int kk = 0; kk < 2; ++kk)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[kk][i], pf[kk][j], acc[i][j], 0, 0, 0);
     }
   }
 
@@ -248,32 +263,116 @@ __global__ __launch_bounds__(512, 1) void conv3x3_halo_kernel(const HaloArgs a) 
           lmax = u > lmax ? u : lmax;
         }
   }
-  hc_sync();  // all wavefronts are done with the tiles: reuse LDS as per-wavefront transposition patches
-  constexpr int ROWB = 64 * 4 + 16;
-  int8_t* patch = smem + wave * (32 * ROWB);
-  const int rrow = lane >> 4, rcol = lane & 15;  // 16 lanes x 16 bytes = one 64-channel row
-  const int ch = kt * 128 + wc * 64 + rcol * 4;
   const long long total_pix = static_cast<long long>(a.N) * Q * Q;
+  if constexpr (!kFused) {
+  hc_sync();  // all wavefronts are done with the tiles: reuse LDS as per-wavefront transposition patches
+  constexpr int ROWB = 32 * 4 + 16;  // one 32-channel tile row of int32, padded
+  int8_t* patch = smem + wave * (32 * ROWB);
+  const int rrow = lane >> 3, rcol = lane & 7;  // 8 lanes x 16 bytes = one 32-channel row
   const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
+    const int mrow = pixbase + wp_ * 64 + j * 32 + rrow;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const v4i v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        *reinterpret_cast<v4i*>(patch + lr * ROWB + (g * 8 + lk * 4) * 4) = v;
+      }
+      // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
+      const int ch = kt * 128 + wc * 64 + i * 32 + rcol * 4;
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const v4i v = *reinterpret_cast<const v4i*>(patch + (t * 8 + rrow) * ROWB + rcol * 16);
+        const int m = mrow + t * 8;
+        const int off = (m < total_pix && ch < a.K) ? (m * a.K + ch) * 4 : kOob;
+        __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0);
+      }
+    }
+  }
+  if (a.absmax != nullptr) fold_absmax(a.absmax, lmax);
+  } else {
+  // ---- tensor-wide range: workgroup maximum -> own slot -> wait for all slots -> maximum over the slots
+  uint32_t* const red = reinterpret_cast<uint32_t*>(dump);  // behind the tiles, clear of the patches below
+  const uint32_t wmax = wave_max_u32(lmax);
+  __syncthreads();  // the tiles are dead from here on
+  if (lane == 0) red[wave] = wmax;
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t bmax = lane < 8 ? red[lane] : 0u;
+    bmax = wave_max_u32(bmax);
+    const int nb = gridDim.x * gridDim.y;
+    const int b = blockIdx.y * gridDim.x + blockIdx.x;
+    uint32_t* const slots = a.sync + kSyncSlot0;
+    if (lane == 0) __hip_atomic_store(&slots[b], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const long long t0 = wall_clock64();
+    uint32_t g = 0;
+    for (;;) {
+      bool ok = true;
+      g = 0;
+      for (int i = lane; i < nb; i += 64) {
+        const uint32_t v = __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && v != 0u;
+        g = v > g ? v : g;
+      }
+      if (__all(ok)) break;
+      if (wall_clock64() - t0 > a.spin_limit) {  // not every workgroup showed up: flag it and leave anyway
+        if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(4);
+    }
+    g = wave_max_u32(g);
+    if (lane == 0) red[8] = g != 0u ? g - 1u : 0u;
+  }
+  __syncthreads();
+  const uint32_t gmax = red[8];
+  const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
+  if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
+    const int sh = shift > 0 ? shift : 0;
+    a.sync[0] = gmax;
+    if (a.shift_out != nullptr) *a.shift_out = sh;
+    if (a.exp_out != nullptr)
+      *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+  }
+  // ---- round, pack four channels per dword, transpose through a per-wavefront patch, store 16-byte pieces
+  const bool trunc = a.trunc != 0;
+  const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
+  const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
+  constexpr int PROW = 64 + 16;  // 64 channels of one pixel, padded
+  int8_t* patch = smem + wave * (64 * PROW);
+#pragma unroll
+  for (int j = 0; j < 2; ++j)
 #pragma unroll
     for (int i = 0; i < 2; ++i)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const v4i v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
-        *reinterpret_cast<v4i*>(patch + lr * ROWB + (i * 32 + g * 8 + lk * 4) * 4) = v;
-      }
-    const int mrow = pixbase + wp_ * 64 + j * 32 + rrow;
+        uint32_t packed = 0;
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-      const v4i v = *reinterpret_cast<const v4i*>(patch + (t * 4 + rrow) * ROWB + rcol * 16);
-      const int m = mrow + t * 4;
-      const int off = (m < total_pix && ch < a.K) ? (m * a.K + ch) * 4 : kOob;
-      __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0);
-    }
+        for (int e = 0; e < 4; ++e) {
+          const int x = acc[i][j][4 * g + e];
+          int r;
+          if (shift >= 1) r = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
+          else r = wrap_to_i8(x);
+          if (relu && r < 0) r = 0;
+          packed |= (static_cast<uint32_t>(r) & 0xFFu) << (8 * e);
+        }
+        *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = packed;
+      }
+  // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
+  const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y8, 0, a.y8_bytes, 0x00020000);
+  const int prow = lane >> 2, piece = lane & 3;
+  const int ch = kt * 128 + wc * 64 + piece * 16;
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    const int pl = t * 16 + prow;
+    const v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
+    const int m = pixbase + wp_ * 64 + pl;
+    const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
+    __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0);
   }
-  if (a.absmax != nullptr) fold_absmax(a.absmax, lmax);
+  }
 }
 
 // Filter arrangement for the kernel above.  mode 0 (forward): F(k, tap, c) = w[k][tap][c], w is [K][9][C].
@@ -305,21 +404,33 @@ __global__ __launch_bounds__(256) void halo_filter_prepare_kernel(const int8_t* 
   }
 }
 
-template <int Q, int BR, int NI>
+template <int Q, int BR, int NI, bool kFused>
 int launch_halo(const HaloArgs& a, hipStream_t stream) {
   using G = HGeom<Q, BR, NI>;
   constexpr size_t lds = G::LDS_BYTES;
   static_assert(lds <= 160 * 1024, "tiles must fit in LDS");
-  static_assert(8 * 32 * (64 * 4 + 16) <= lds, "epilogue patches must fit in LDS");
-  auto k = conv3x3_halo_kernel<Q, BR, NI>;
+  static_assert(8 * 32 * (32 * 4 + 16) <= G::ACT_BYTES + G::WSTAGES * G::W_BYTES, "epilogue patches must fit in LDS");
+  static_assert(8 * 64 * (64 + 16) <= G::ACT_BYTES + G::WSTAGES * G::W_BYTES, "int8 patches must stay clear of the reduction words");
+  static_assert(2 * lds <= 160 * 1024, "two workgroups per compute unit");
+  auto k = conv3x3_halo_kernel<Q, BR, NI, kFused>;
   static bool attr_set = false;
+  static int resident = 0;  // workgroups the device holds at once
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return fail(NITI_ERR_LAUNCH, "conv3x3_halo: cannot reserve %zu bytes of LDS", lds);
+    if (kFused) {
+      int dev = 0, cus = 0, per_cu = 0;
+      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+          hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(k), 512, lds) != hipSuccess)
+        return fail(NITI_ERR_LAUNCH, "conv3x3_halo: cannot query occupancy");
+      resident = cus * per_cu;
+    }
     attr_set = true;
   }
   const long long pix = static_cast<long long>(a.N) * Q * Q;
   dim3 grid(static_cast<unsigned>((pix + 255) / 256), (a.K + 127) / 128);
+  if (kFused && static_cast<long long>(grid.x) * grid.y > resident)
+    return fail(NITI_ERR_UNSUPPORTED, "conv3x3_halo: %u workgroups do not fit on the device at once (%d)", grid.x * grid.y, resident);
   hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, a);
   return check_launch("conv3x3_halo");
 }
@@ -349,24 +460,60 @@ int launch_halo_filter_prepare(const int8_t* w, int8_t* dst, int kout, int cin, 
   return check_launch("halo_filter_prepare");
 }
 
-int launch_conv3x3_halo(const int8_t* x, const int8_t* wp, int32_t* y, int N, int H, int C, int K, unsigned flags,
-                        uint32_t* absmax, hipStream_t stream) {
-  HaloArgs a;
+static void fill_common(HaloArgs& a, const int8_t* x, const int8_t* wp, int N, int H, int C, int K, unsigned flags) {
+  a = HaloArgs{};
   a.x = x;
   a.wp = wp;
-  a.y = y;
-  a.absmax = absmax;
   a.N = N;
   a.C = C;
   a.K = K;
   a.cslices = (C + 63) / 64;
   a.x_bytes = static_cast<long long>(N) * H * H * C;
   a.wp_bytes = static_cast<long long>(conv3x3_halo_filter_bytes(C, K));
-  a.y_bytes = static_cast<long long>(N) * H * H * K * 4;
   a.flags = flags;
-  if (H == 32) return launch_halo<32, 8, 1>(a, stream);
-  if (H == 16) return launch_halo<16, 16, 1>(a, stream);
-  return launch_halo<8, 8, 4>(a, stream);
+}
+
+int launch_conv3x3_halo(const int8_t* x, const int8_t* wp, int32_t* y, int N, int H, int C, int K, unsigned flags,
+                        uint32_t* absmax, hipStream_t stream) {
+  HaloArgs a;
+  fill_common(a, x, wp, N, H, C, K, flags);
+  a.y = y;
+  a.absmax = absmax;
+  a.y_bytes = static_cast<long long>(N) * H * H * K * 4;
+  if (H == 32) return launch_halo<32, 8, 1, false>(a, stream);
+  if (H == 16) return launch_halo<16, 16, 1, false>(a, stream);
+  return launch_halo<8, 8, 4, false>(a, stream);
+}
+
+// Workgroups of a launch of the requantising variant (= sync slots), or 0 when the variant cannot run the shape.
+int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
+  if (!conv3x3_halo_supported(N, H, W, C, K, R, S, stride, pad) || K % 16 != 0) return 0;
+  const long long nb = (static_cast<long long>(N) * H * W / 256) * ((K + 127) / 128);
+  return nb <= 2048 ? static_cast<int>(nb) : 0;  // the device check happens at launch; this bounds the workspace
+}
+
+size_t conv3x3_halo_sync_words(int blocks) { return static_cast<size_t>(kSyncSlot0 + (blocks + 15) / 16 * 16); }
+
+int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, int N, int H, int C, int K, unsigned flags,
+                                uint32_t* sync, const RequantSpec& rq, hipStream_t stream) {
+  HaloArgs a;
+  fill_common(a, x, wp, N, H, C, K, flags);
+  a.y8 = y8;
+  a.sync = sync;
+  a.y8_bytes = static_cast<long long>(N) * H * H * K;
+  a.target_bits = rq.target_bits;
+  a.method = rq.method;
+  a.trunc = rq.trunc;
+  a.bw_mode = rq.bw_mode;
+  a.rq_flags = rq.flags;
+  a.spin_limit = rq.spin_limit;
+  a.shift_out = rq.shift_out;
+  a.exp_a = rq.exp_a;
+  a.exp_b = rq.exp_b;
+  a.exp_out = rq.exp_out;
+  if (H == 32) return launch_halo<32, 8, 1, true>(a, stream);
+  if (H == 16) return launch_halo<16, 16, 1, true>(a, stream);
+  return launch_halo<8, 8, 4, true>(a, stream);
 }
 
 }  // namespace niti

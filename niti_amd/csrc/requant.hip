@@ -4,43 +4,10 @@
 // 16 int32 (64 bytes in, 16 bytes out) per thread per step; the shift is derived on the
 // device from the max the producer kernel left in memory.
 #include "common.h"
+#include "requant_math.h"
 
 namespace niti {
 namespace {
-
-__device__ inline int clip127(long long v) { return static_cast<int>(v > 127 ? 127 : (v < -127 ? -127 : v)); }
-
-// quotient and magnitude of the remainder of x / 2^s: floor division or truncation
-__device__ inline void split_pow2(long long x, int s, bool trunc, long long& q, long long& rem) {
-  if (!trunc || x >= 0) {
-    q = x >> s;
-    rem = x - (q << s);
-  } else {
-    const long long m = -x;
-    q = -(m >> s);
-    rem = m & ((1LL << s) - 1);
-  }
-}
-
-template <int kMethod>
-__device__ inline int round_one(int x, int s, bool trunc, int u) {
-  if (kMethod == NITI_ROUND_NEAREST) {
-    const long long half = 1LL << (s - 1);
-    if (!trunc) return clip127((static_cast<long long>(x) + half) >> s);
-    const long long m = x < 0 ? -static_cast<long long>(x) : static_cast<long long>(x);
-    const long long q = (m + half) >> s;
-    return clip127(x < 0 ? -q : q);
-  }
-  long long q, rem;
-  split_pow2(x, s, trunc, q, rem);
-  const int sg = (x > 0) - (x < 0);
-  if (kMethod == NITI_ROUND_STOCHASTIC) return clip127(q + (rem > static_cast<long long>(u) ? sg : 0));
-  const int h = s >> 1;
-  const long long hi = rem >> h;
-  long long lo = rem & ((1LL << h) - 1);
-  if (s & 1) lo <<= 1;
-  return clip127(q + (hi > lo ? sg : 0));
-}
 
 __global__ __launch_bounds__(256) void absmax_i32_kernel(const int32_t* __restrict__ x, int64_t n, uint32_t* absmax) {
   const int64_t nv = n >> 2;
@@ -97,7 +64,7 @@ __global__ __launch_bounds__(256) void requant_kernel(const RequantArgs a) {
   auto one = [&](int x, int u) -> int {
     int r;
     if (shift >= 1) r = round_one<kMethod>(x, shift, trunc, u);
-    else r = static_cast<int>(static_cast<int8_t>(static_cast<uint32_t>(x) & 0xFFu));
+    else r = wrap_to_i8(x);
     if (relu && r < 0) r = 0;
     return r;
   };

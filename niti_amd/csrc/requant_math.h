@@ -1,0 +1,78 @@
+// Per-element shift-round-clip of the integer requantisation, shared by the stand-alone requantisation
+// kernels and the convolution kernel that requantises its own sums.
+#pragma once
+#include "common.h"
+
+namespace niti {
+
+__device__ inline int clip127(long long v) { return static_cast<int>(v > 127 ? 127 : (v < -127 ? -127 : v)); }
+
+// quotient and magnitude of the remainder of x / 2^s: floor division or truncation
+__device__ inline void split_pow2(long long x, int s, bool trunc, long long& q, long long& rem) {
+  if (!trunc || x >= 0) {
+    q = x >> s;
+    rem = x - (q << s);
+  } else {
+    const long long m = -x;
+    q = -(m >> s);
+    rem = m & ((1LL << s) - 1);
+  }
+}
+
+// s >= 1.  u: random integer in [0, 2^s) for NITI_ROUND_STOCHASTIC, ignored otherwise
+template <int kMethod>
+__device__ inline int round_one(int x, int s, bool trunc, int u) {
+  if (kMethod == NITI_ROUND_NEAREST) {
+    const long long half = 1LL << (s - 1);
+    if (!trunc) return clip127((static_cast<long long>(x) + half) >> s);
+    const long long m = x < 0 ? -static_cast<long long>(x) : static_cast<long long>(x);
+    const long long q = (m + half) >> s;
+    return clip127(x < 0 ? -q : q);
+  }
+  long long q, rem;
+  split_pow2(x, s, trunc, q, rem);
+  const int sg = (x > 0) - (x < 0);
+  if (kMethod == NITI_ROUND_STOCHASTIC) return clip127(q + (rem > static_cast<long long>(u) ? sg : 0));
+  const int h = s >> 1;
+  const long long hi = rem >> h;
+  long long lo = rem & ((1LL << h) - 1);
+  if (s & 1) lo <<= 1;
+  return clip127(q + (hi > lo ? sg : 0));
+}
+
+// The same results as round_one for the methods that need no random input, in 32-bit arithmetic
+// (1 <= s <= 31): floor((x + 2^(s-1)) / 2^s) = (x >> s) + bit s-1 of x, and remainders are masks.
+template <int kMethod>
+__host__ __device__ inline int round_one32(int x, int s, bool trunc) {
+  static_assert(kMethod == NITI_ROUND_NEAREST || kMethod == NITI_ROUND_PSEUDO_STOCHASTIC, "no random input here");
+  const bool neg = x < 0;
+  const uint32_t m = neg ? 0u - static_cast<uint32_t>(x) : static_cast<uint32_t>(x);
+  const bool by_magnitude = trunc && neg;
+  int q;
+  uint32_t rem;
+  if (by_magnitude) {
+    q = -static_cast<int>(m >> s);
+    rem = m & ((1u << s) - 1u);
+  } else {
+    q = x >> s;
+    rem = static_cast<uint32_t>(x) & ((1u << s) - 1u);
+  }
+  int r;
+  if (kMethod == NITI_ROUND_NEAREST) {
+    const int up = static_cast<int>((rem >> (s - 1)) & 1u);
+    r = by_magnitude ? q - up : q + up;
+  } else {
+    const int h = s >> 1;
+    const uint32_t hi = rem >> h;
+    uint32_t lo = rem & ((1u << h) - 1u);
+    if (s & 1) lo <<= 1;
+    const int sg = (x > 0) - (x < 0);
+    r = q + (hi > lo ? sg : 0);
+  }
+  return r > 127 ? 127 : (r < -127 ? -127 : r);
+}
+
+// shift < 1: the reference converts int32 to int8 by keeping the low byte
+__device__ inline int wrap_to_i8(int x) { return static_cast<int>(static_cast<int8_t>(static_cast<uint32_t>(x) & 0xFFu)); }
+
+}  // namespace niti

@@ -103,6 +103,75 @@ def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None, p
     return dx
 
 
+def conv_requant_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1, dgrad=False) -> int:
+    """uint32 words of the sync buffer conv2d_fprop_requant / conv2d_dgrad_requant need for a convolution with
+    INPUT [N,H,W,C] and filter [K,R,S,C]; 0 when only the two-pass path (conv2d_* then requant) covers the shape."""
+    return int(L.lib().niti_conv2d_i8_requant_sync_words(N, H, W, C, K, R, S, stride, padding, int(dgrad)))
+
+
+def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epilogue, target_bits, method, div_mode,
+                  bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter):
+    _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter)
+    if x.dtype != torch.int8 or w.dtype != torch.int8:
+        raise RuntimeError("%s: int8 tensors expected" % entry)
+    N, H, W, C, K, R, S = dims
+    words = conv_requant_sync_words(N, H, W, C, K, R, S, stride, padding, dgrad)
+    if words == 0:
+        raise L.NitiError("%s: shape not covered by the single-launch path" % entry)
+    if sync is None:
+        sync = torch.zeros(words, dtype=torch.int32, device=x.device)
+    elif sync.dtype != torch.int32 or sync.numel() < words:
+        raise RuntimeError("%s: sync must be a zeroed int32 tensor of at least %d words" % (entry, words))
+    y = torch.empty(out_shape, dtype=torch.int8, device=x.device)
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=x.device)
+    flags = _flags(f32_epilogue)
+    if prepared_filter is not None:
+        wptr, ws, nbytes, flags = _ptr(prepared_filter), None, 0, flags | L.CONV_FILTER_PREPARED
+    else:
+        nbytes = L.lib().niti_conv2d_i8_filter_workspace(N, H, W, C, K, R, S, stride, padding, int(dgrad))
+        ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=x.device)
+        wptr = _ptr(w)
+    st = getattr(L.lib(), entry)(_ptr(x), wptr, _ptr(y), N, H, W, C, K, R, S, stride, padding, flags, target_bits,
+                                 L.ROUND[method], L.DIV[div_mode], L.BW[bw_mode], L.RQ_RELU if relu else 0, _ptr(sync),
+                                 sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes,
+                                 _stream(x))
+    L.check(st, entry)
+    return y, shift_out, sync
+
+
+def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
+                         bw_mode="int", relu=False, sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
+                         prepared_filter=None):
+    """conv2d_fprop + requant as one launch: x [N,H,W,C] int8, w [K,R,S,C] int8 -> ([N,P,Q,K] int8, device shift,
+    sync).  sync[0] holds max|sum| afterwards, sync[1] != 0 flags a timed-out wait (invalid output).  ``sync``, if
+    given, must hold conv_requant_sync_words(...) zeroed int32 words."""
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    if C2 != C:
+        raise RuntimeError("conv2d_fprop_requant: channel mismatch %d vs %d" % (C, C2))
+    P = (H + 2 * padding - R) // stride + 1
+    Q = (W + 2 * padding - S) // stride + 1
+    return _conv_requant("niti_conv2d_i8_fprop_requant", False, x, w, (N, P, Q, K), (N, H, W, C, K, R, S), stride, padding,
+                         f32_epilogue, target_bits, method, div_mode, bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out,
+                         prepared_filter)
+
+
+def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
+                         bw_mode="int", sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
+                         prepared_filter=None):
+    """conv2d_dgrad + requant as one launch: err [N,P,Q,K] int8, w [K,R,S,C] int8 -> ([N,H,W,C] int8, shift, sync)."""
+    N, P, Q, K = err.shape
+    K2, R, S, C = w.shape
+    if K2 != K:
+        raise RuntimeError("conv2d_dgrad_requant: channel mismatch")
+    H = P - 2 * padding + R - 1
+    W = Q - 2 * padding + S - 1
+    return _conv_requant("niti_conv2d_i8_dgrad_requant", True, err, w, (N, H, W, C), (N, H, W, C, K, R, S), stride, padding,
+                         f32_epilogue, target_bits, method, div_mode, bw_mode, False, sync, shift_out, exp_a, exp_b, exp_out,
+                         prepared_filter)
+
+
 def conv2d_wgrad(act, err, R, S, stride=1, padding=1, f32_epilogue=False, absmax=None):
     """act [N,H,W,C] int8, err [N,P,Q,K] int8 -> dw [K,R,S,C] int32 (stride 1)."""
     _chk_dev(act, err, absmax)

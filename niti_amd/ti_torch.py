@@ -184,6 +184,41 @@ def grad_calc(int32_acc, mu, absmax=None, rand=None):
     return y, shift
 
 
+FUSE_CONV_REQUANT = True     # run convolution + requantisation as one launch where the library covers the shape
+_fused_refused = set()       # (dgrad, input shape, filter shape, stride, padding) the device turned out too small for
+
+
+def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b):
+    """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
+    exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
+    single-launch kernel, or more workgroups than the device holds at once."""
+    method = _method_name(fn)
+    if not FUSE_CONV_REQUANT or method == "sto" or rand is not None:
+        return None
+    key = (dgrad, tuple(x.shape), tuple(w.shape), stride, padding)
+    if key in _fused_refused:
+        return None
+    N = x.shape[0]
+    K, R, S, C = w.shape
+    H, W = (x.shape[1] - 2 * padding + R - 1, x.shape[2] - 2 * padding + S - 1) if dgrad else (x.shape[1], x.shape[2])
+    if ops.conv_requant_sync_words(N, H, W, C, K, R, S, stride, padding, dgrad) == 0:
+        _fused_refused.add(key)
+        return None
+    from ._lib import NitiError
+    exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
+    call = ops.conv2d_dgrad_requant if dgrad else ops.conv2d_fprop_requant
+    kw = dict(relu=relu) if not dgrad else {}
+    try:
+        y, shift, _ = call(x, w, stride, padding, f32_epilogue=F32_EPILOGUE, target_bits=BITWIDTH, method=method,
+                           div_mode=DIV_MODE, bw_mode=BW_MODE, exp_a=exp_a, exp_b=exp_b, exp_out=exp_out, **kw)
+    except NitiError as e:
+        if "do not fit" not in str(e):
+            raise
+        _fused_refused.add(key)
+        return None
+    return y, shift, exp_out
+
+
 # ------------------------------------------------------------------------------------------
 # op wrappers (ti_torch.py:152-233)
 # ------------------------------------------------------------------------------------------
@@ -325,12 +360,17 @@ class TiConv2d(UpdateWeight):
     def forward(self, input, rand=None):
         self.act, self.act_in_exp = input
         dev = self.act.device
-        am = ops.new_scalar_u32(dev)
         self.act16 = _pad_channels16(self.act).contiguous()      # channel-padded copy, reused by the weight gradient
-        acc = ops.conv2d_fprop(self.act16, _pad_channels16(self.weight).contiguous(), self.stride, self.padding,
-                               f32_epilogue=F32_EPILOGUE, absmax=am)
+        w16 = _pad_channels16(self.weight).contiguous()
+        exp_a, exp_b = _exp_tensor(self.act_in_exp, dev), self._wexp()
+        fused = _conv_requant_fused(False, self.act16, w16, self.stride, self.padding, ACT_ROUND_METHOD, rand,
+                                    self.fuse_relu, exp_a, exp_b)
+        if fused is not None:
+            return fused[0], fused[2]
+        am = ops.new_scalar_u32(dev)
+        acc = ops.conv2d_fprop(self.act16, w16, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
         act_out, _, exp_out = _requant(acc, BITWIDTH, ACT_ROUND_METHOD, am, rand, relu=self.fuse_relu,
-                                       exp_a=_exp_tensor(self.act_in_exp, dev), exp_b=self._wexp(), want_exp=True)
+                                       exp_a=exp_a, exp_b=exp_b, want_exp=True)
         return act_out, exp_out
 
     def backward(self, input, rand=None, grad_rand=None):
@@ -341,10 +381,15 @@ class TiConv2d(UpdateWeight):
         self.err_exp = self.err_exp_in
         if not self.first_layer:
             # data gradient with the weights as they were in the forward pass
-            am = ops.new_scalar_u32(dev)
-            dx = ops.conv2d_dgrad(err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
-            err_out, _, new_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
-                                           exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
+            fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
+                                        False, self.err_exp_in, self._wexp())
+            if fused is not None:
+                err_out, _, new_exp = fused
+            else:
+                am = ops.new_scalar_u32(dev)
+                dx = ops.conv2d_dgrad(err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
+                err_out, _, new_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
+                                               exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
             self.err_exp = new_exp
         amg = ops.new_scalar_u32(dev)
         K, R, S, C = self.weight.shape

@@ -104,6 +104,113 @@ def test_conv_dgrad(dev, case):
     assert int(am.cpu()) == po.absmax(ref)
 
 
+# convolution + requantisation in one launch: N,Q,C,K (3x3, stride 1, pad 1), small sums / large sums / ragged tiles
+FUSED_CASES = [(4, 8, 16, 16), (4, 8, 64, 128), (8, 8, 80, 144), (1, 16, 16, 48), (3, 16, 192, 272), (2, 32, 16, 64),
+               (8, 32, 128, 128), (12, 8, 512, 128)]
+
+
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+@pytest.mark.parametrize("method", ["round", "psto"])
+@pytest.mark.parametrize("case", FUSED_CASES)
+def test_conv_fprop_requant(dev, case, method, div_mode):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_fprop_requant", case, method, div_mode)
+    g = torch.Generator().manual_seed(900 + N + C + K)
+    x, w = ri8(g, N, Q, Q, C), ri8(g, K, 3, 3, C)
+    acc = po.conv2d_fprop_i32(x, w, 1, 1)
+    words = ops.conv_requant_sync_words(N, Q, Q, C, K)
+    assert words >= 16 + (N * Q * Q // 256) * ((K + 127) // 128)
+    for tgt, relu in ((7, False), (7, True), (4, False)):
+        ref, sh_ref = po.act_calc(acc, 0, method, div_mode) if tgt == 7 else po.grad_calc(acc, tgt, method, div_mode)
+        ea = torch.tensor([3], dtype=torch.int32, device=dev)
+        eb = torch.tensor([-11], dtype=torch.int32, device=dev)
+        eo = torch.zeros(1, dtype=torch.int32, device=dev)
+        y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), 1, 1, target_bits=tgt, method=method, div_mode=div_mode,
+                                               relu=relu, exp_a=ea, exp_b=eb, exp_out=eo)
+        torch.cuda.synchronize()
+        sync = sync.cpu()
+        assert int(sync[1]) == 0, "grid-wide wait timed out"
+        assert int(sync[0]) == po.absmax(acc)
+        assert int(sh.cpu()) == sh_ref and int(eo.cpu()) == sh_ref + 3 - 11
+        assert torch.equal(y.cpu(), ref.clamp(min=0) if relu else ref)
+
+
+def test_conv_fprop_requant_wraps_when_no_shift(dev):
+    """Sums that already fit 7 bits (+ the 128 -> -128 wrap of the reference's int32 -> int8 cast)."""
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    _say("conv_fprop_requant no shift")
+    x = torch.zeros((4, 8, 8, 16), dtype=torch.int8)
+    w = torch.zeros((16, 3, 3, 16), dtype=torch.int8)
+    x[0, 3, 3, 0] = 64
+    w[2, 1, 1, 0] = 2          # one sum of exactly 128: bit width 7, shift 0, low byte wraps to -128
+    x[1, 2, 2, 1] = -5
+    w[3, 1, 1, 1] = 7
+    acc = po.conv2d_fprop_i32(x, w, 1, 1)
+    ref, sh_ref = po.act_calc(acc, 0)
+    assert sh_ref == 0 and int(ref.min()) == -128
+    y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev))
+    assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == 0 and int(sync.cpu()[1]) == 0
+
+
+def test_conv_fprop_requant_f32_epilogue(dev):
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    _say("conv_fprop_requant f32 epilogue, |acc| > 2^24")
+    x = torch.full((4, 8, 8, 256), 127, dtype=torch.int8)
+    x[0, 2, 2, 0] = 126
+    w = torch.full((16, 3, 3, 256), 127, dtype=torch.int8)
+    w[1] = -127
+    w[2, 0, 0, 5] = 1
+    acc = po.conv2d_fprop_i32(x, w)
+    assert int(acc.abs().max()) > 2 ** 24
+    for f32 in (True, False):
+        a = po.f32_roundtrip(acc) if f32 else acc
+        ref, sh_ref = po.act_calc(a, 0)
+        y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), f32_epilogue=f32)
+        assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(a)
+
+
+@pytest.mark.parametrize("case", [(4, 8, 96, 48), (1, 16, 32, 16), (2, 16, 256, 128), (8, 32, 128, 128), (4, 8, 16, 32)])
+def test_conv_dgrad_requant(dev, case):
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_dgrad_requant", case)
+    g = torch.Generator().manual_seed(950 + C + K)
+    e, w = ri8(g, N, Q, Q, K), ri8(g, K, 3, 3, C)
+    acc = co.conv_dgrad(e, w, Q, Q, 1, 1)
+    for method in ("round", "psto"):
+        ref, sh_ref = po.err_calc(acc, method)
+        wt = ops.conv_filter_prepare(w.to(dev), N, Q, Q, dgrad=True)
+        for prepared in (None, wt):
+            y, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), 1, 1, method=method, prepared_filter=prepared)
+            assert int(sync.cpu()[1]) == 0
+            assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
+
+
+def test_conv_requant_rejects_what_it_does_not_cover(dev):
+    from niti_amd import ops
+    from niti_amd._lib import NitiError
+    _say("conv_requant unsupported shapes")
+    assert ops.conv_requant_sync_words(3, 7, 9, 32, 40) == 0        # not square / not 8, 16, 32
+    assert ops.conv_requant_sync_words(2, 8, 8, 16, 10) == 0        # 128 pixels: not whole workgroups
+    assert ops.conv_requant_sync_words(4096, 32, 32, 16, 128) == 0  # far more workgroups than any device holds
+    x = torch.zeros((2, 8, 8, 16), dtype=torch.int8, device=dev)
+    w = torch.zeros((16, 3, 3, 16), dtype=torch.int8, device=dev)
+    with pytest.raises(NitiError):
+        ops.conv2d_fprop_requant(x, w)
+    # a launch that would not be resident at once is refused by the library, not started
+    N = 2048                                                          # 2048 workgroups of 256 pixels
+    assert ops.conv_requant_sync_words(N, 16, 16, 16, 16) > 0
+    x = torch.zeros((N, 16, 16, 16), dtype=torch.int8, device=dev)
+    with pytest.raises(NitiError):
+        ops.conv2d_fprop_requant(x, w)
+
+
 WGRAD_CASES = [(4, 32, 32, 16, 32, 3, 1), (8, 16, 16, 128, 64, 3, 1), (6, 8, 8, 80, 144, 3, 1), (2, 32, 32, 64, 128, 3, 1),
                (64, 8, 8, 64, 256, 3, 1), (16, 16, 16, 256, 128, 3, 1), (2, 8, 8, 16, 16, 3, 1), (16, 8, 8, 32, 48, 3, 1), (5, 7, 9, 40, 24, 3, 1), (32, 16, 16, 64, 128, 3, 1),
                (4, 8, 8, 3, 16, 3, 1), (6, 8, 8, 16, 10, 5, 2), (3, 6, 6, 8, 8, 3, 0), (128, 8, 8, 16, 16, 3, 1)]
