@@ -71,7 +71,11 @@ class ConvTriple:
                                                 dgrad=dgrad)
                 L[key] = (off, n)
                 off += n
+            n = ops.wgrad_update_sync_words(BATCH, L["hw"], L["hw"], L["x16"].shape[3], L["k"])
+            L["sync_w"] = (off, n)
+            off += n
         self.sync = torch.zeros(max(off, 1), dtype=torch.int32, device=dev)
+        self.ws = ops.scratch(256 << 20, dev)    # shared by all weight-gradient launches
         self.exp0 = torch.zeros(1, dtype=torch.int32, device=dev)
         self.ops_per_step = sum(conv_ops(BATCH, hw, c, k) * (2 if i == 0 else 3) for i, (c, k, hw) in enumerate(LAYERS))
         self.main_kernel_ops = []     # algorithmic ops of every launch bracketed by events, in launch order
@@ -120,10 +124,15 @@ class ConvTriple:
                 if not sn:
                     ops.requant(dx, am[1:2], 7, "round")
             # weight gradient + gradient rounding + weight update
-            dw = ops.conv2d_wgrad(L["x16"], L["err"], 3, 3, 1, 1, f32_epilogue=(i > 0), absmax=am[2:3])
-            if c % 16:
-                dw = dw[..., :c].contiguous()     # zero-padded input channels give zero gradient columns
-            ops.grad_update(dw, L["w"], am[2:3], 5, "psto")
+            so, sn = L["sync_w"]
+            if sn:
+                ops.conv2d_wgrad_update(L["x16"], L["err"], L["w"], 1, 1, f32_epilogue=(i > 0), mu=5, method="psto",
+                                        sync=self.sync[so:so + sn], workspace=self.ws)
+            else:
+                dw = ops.conv2d_wgrad(L["x16"], L["err"], 3, 3, 1, 1, f32_epilogue=(i > 0), absmax=am[2:3], workspace=self.ws)
+                if c % 16:
+                    dw = dw[..., :c].contiguous()     # zero-padded input channels give zero gradient columns
+                ops.grad_update(dw, L["w"], am[2:3], 5, "psto")
 
 
 def make_runner(step_fn, warmup, use_graph=True):

@@ -148,6 +148,32 @@ int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int 
                          size_t workspace_bytes, void* stream);
 
 /*
+ * Weight gradient, gradient rounding and weight update in one call.  Replaces the chain
+ *   cutlassconv_cuda.sp_conv_optimized on transposed operands (ti_torch.py:430-432) -> grad_calc
+ *   (ti_torch.py:135-147) -> UpdateWeight.weight_update (ti_torch.py:11-21)
+ * with the same result as niti_conv2d_i8_wgrad followed by niti_grad_update_i8, bit for bit; the int32 gradient
+ * is only written when dw_out is given.  The partial sums of the weight-gradient kernel are added up, the
+ * tensor-wide range is exchanged between the workgroups of the finishing kernel, and
+ *   g = round(dw >> max(bitwidth(max|dw|) - mu, 0)),  w = clip(w - g, +-127).
+ *
+ * Covered: the shapes of the native 3x3 weight-gradient kernel (3x3, stride 1, pad 1, square maps of side 8, 16
+ * or 32, C % 16 == 0, K % 16 == 0, N*H*W % 128 == 0, even N for side 8) with K*9*C <= 4M, rounding
+ * NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC.  niti_conv2d_i8_wgrad_update_sync_words returns 0 otherwise.
+ *
+ * act: [N,H,W,C] int8 (C may include zero channel padding); err: [N,H,W,K] int8; w: [K,3,3,w_channels] int8,
+ * updated in place, w_channels <= C (gradient columns beyond w_channels are padding and are dropped).
+ * g8_out (optional): rounded gradient, laid out like w.  dw_out (optional): int32 gradient [K,3,3,C].
+ * sync: as for niti_conv2d_i8_fprop_requant (zero on entry; word 0 = max |dw|, word 1 = wait timed out).
+ * workspace: niti_conv2d_i8_wgrad_workspace bytes.  flags: NITI_EPI_F32_ROUNDTRIP.
+ */
+size_t niti_conv2d_i8_wgrad_update_sync_words(int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
+int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int W, int C,
+                                int K, int R, int S, int stride, int pad, unsigned flags, int mu, int method, int div_mode,
+                                int bw_mode, uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* dw_out,
+                                int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * int8 x int8 -> exact int32 GEMM, replaces int8mm_cuda.int8_mm
  * (pytorch/int8mm-extension/int8mm.cpp:9-14, int8mm_kernel.cu:8-34):
  *   c[m,n] = sum_k opA[m,k] * opB[k,n],  c row-major with leading dimension n.

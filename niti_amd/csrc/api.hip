@@ -1,6 +1,7 @@
 // extern "C" surface of libniti_gfx950: argument checking, workspace carving and the
 // composition of kernels behind each entry point declared in include/niti_gfx950.h.
 #include <stdarg.h>
+#include <stdint.h>
 #include <stdlib.h>
 #include <string.h>
 
@@ -190,6 +191,17 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
 }
 
 // ---- convolution + requantisation in one launch -------------------------------------------------------
+// wall-clock ticks (100 MHz) a grid-wide wait may last; NITI_SYNC_TIMEOUT_MS overrides the 10 s default
+static long long sync_spin_limit() {
+  static long long spin_limit = -1;
+  if (spin_limit < 0) {
+    const char* e = getenv("NITI_SYNC_TIMEOUT_MS");
+    const long long ms = e != nullptr ? atoll(e) : 10000;
+    spin_limit = (ms > 0 ? ms : 1) * 100000LL;
+  }
+  return spin_limit;
+}
+
 static int fused_blocks(int N, int H, int W, int C, int K, int R, int S, int stride, int pad, int dgrad) {
   if (halo_off()) return 0;
   if (!dgrad) return conv3x3_halo_requant_blocks(N, H, W, C, K, R, S, stride, pad);
@@ -237,13 +249,7 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
     if (st != NITI_OK) return st;
     wp = static_cast<const int8_t*>(workspace);
   }
-  static long long spin_limit = -1;  // 100 MHz ticks; NITI_SYNC_TIMEOUT_MS overrides the 10 s default
-  if (spin_limit < 0) {
-    const char* e = getenv("NITI_SYNC_TIMEOUT_MS");
-    const long long ms = e != nullptr ? atoll(e) : 10000;
-    spin_limit = (ms > 0 ? ms : 1) * 100000LL;
-  }
-  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, spin_limit, shift_out, exp_a, exp_b, exp_out};
+  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out};
   return launch_conv3x3_halo_requant(x, wp, y8, N, Hk, Ck, Kk, flags, sync, rq, s);
 }
 
@@ -314,6 +320,44 @@ extern "C" int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_
   st = launch_conv_igemm(p, s);
   if (st != NITI_OK) return st;
   return launch_post_i32(dw, nout, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, absmax, s);
+}
+
+extern "C" size_t niti_conv2d_i8_wgrad_update_sync_words(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
+  if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0) return 0;
+  if (!wgrad3x3_supported(N, H, W, C, K, R, S, stride, pad)) return 0;
+  const int nb = wgrad3x3_finish_blocks(C, K);
+  return nb > 0 ? wgrad3x3_sync_words(nb) : 0;
+}
+
+extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int W,
+                                           int C, int K, int R, int S, int stride, int pad, unsigned flags, int mu, int method,
+                                           int div_mode, int bw_mode, uint32_t* sync, size_t sync_words, int8_t* g8_out,
+                                           int32_t* dw_out, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b,
+                                           int32_t* exp_out, void* workspace, size_t workspace_bytes, void* stream) {
+  clear_error();
+  int st = check_conv_dims("conv_wgrad_update", N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
+  if (act == nullptr || err == nullptr || w == nullptr || sync == nullptr)
+    return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: null pointer");
+  if (w_channels < 1 || w_channels > C) return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: w_channels=%d outside 1..C=%d", w_channels, C);
+  if (mu < 1 || mu > 7) return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: mu=%d outside 1..7", mu);
+  if (method != NITI_ROUND_NEAREST && method != NITI_ROUND_PSEUDO_STOCHASTIC)
+    return fail(NITI_ERR_UNSUPPORTED, "conv_wgrad_update: rounding method %d needs random input; use the two-pass path", method);
+  if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: div_mode=%d", div_mode);
+  if (bw_mode != NITI_BW_INT && bw_mode != NITI_BW_F32) return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: bw_mode=%d", bw_mode);
+  const size_t words = niti_conv2d_i8_wgrad_update_sync_words(N, H, W, C, K, R, S, stride, pad);
+  if (words == 0) return fail(NITI_ERR_UNSUPPORTED, "conv_wgrad_update: shape not covered by the single-pass path; use the two-pass path");
+  if (sync_words < words) return fail(NITI_ERR_WORKSPACE, "conv_wgrad_update: needs %zu zeroed sync words, got %zu", words, sync_words);
+  const size_t need = niti_conv2d_i8_wgrad_workspace(N, H, W, C, K, R, S, pad);
+  if (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))
+    return fail(NITI_ERR_WORKSPACE, "conv_wgrad_update: needs %zu workspace bytes (16-byte aligned), got %zu", need, workspace_bytes);
+  if (!aligned16(act) || !aligned16(err) || (dw_out != nullptr && !aligned16(dw_out)))
+    return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: act, err and dw_out must be 16-byte aligned");
+  if (w_channels == C && (reinterpret_cast<uintptr_t>(w) % 4 != 0 || (g8_out != nullptr && reinterpret_cast<uintptr_t>(g8_out) % 4 != 0)))
+    return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: w and g8_out must be 4-byte aligned");
+  RequantSpec rq{mu, method, div_mode == NITI_DIV_TRUNC, bw_mode, 0u, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out};
+  return launch_wgrad3x3_update(act, err, w, w_channels, N, H, C, K, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, sync, rq, g8_out,
+                                dw_out, workspace, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t niti_gemm_i8_workspace(int trans_a, int trans_b, int m, int n, int k) {

@@ -248,21 +248,16 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         vmax = max(vmax, max(acc[i][j][e], acc[i][j][e + 1]));
         vmin = min(vmin, min(acc[i][j][e], acc[i][j][e + 1]));
       }
-  uint32_t lmax = max(static_cast<uint32_t>(vmax), 0u - static_cast<uint32_t>(vmin));
-  if (roundtrip && wave_max_u32(lmax) > (1u << 24)) {
-    lmax = 0;
-#pragma unroll
-    for (int i = 0; i < 2; ++i)
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int e = 0; e < 16; ++e) {
-          const int t = f32_roundtrip(acc[i][j][e]);
-          acc[i][j][e] = t;
-          const uint32_t u = uabs(t);
-          lmax = u > lmax ? u : lmax;
-        }
+  // The fp32 round trip is the identity up to 2^24, so it is applied (wavefront-uniformly) only beyond; it is
+  // monotonic and odd, so the range after it follows from the extreme values alone, and the sums themselves
+  // are converted where they are consumed below instead of in a second copy of the accumulators.
+  bool rt = false;
+  if (roundtrip) rt = wave_max_u32(max(static_cast<uint32_t>(vmax), 0u - static_cast<uint32_t>(vmin))) > (1u << 24);
+  if (rt) {
+    vmax = f32_roundtrip(vmax);
+    vmin = f32_roundtrip(vmin);
   }
+  const uint32_t lmax = max(static_cast<uint32_t>(vmax), 0u - static_cast<uint32_t>(vmin));
   const long long total_pix = static_cast<long long>(a.N) * Q * Q;
   if constexpr (!kFused) {
   hc_sync();  // all wavefronts are done with the tiles: reuse LDS as per-wavefront transposition patches
@@ -277,7 +272,11 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     for (int i = 0; i < 2; ++i) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const v4i v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        v4i v = {acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3]};
+        if (rt) {
+#pragma unroll
+          for (int e = 0; e < 4; ++e) v[e] = f32_roundtrip(v[e]);
+        }
         *reinterpret_cast<v4i*>(patch + lr * ROWB + (g * 8 + lk * 4) * 4) = v;
       }
       // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
@@ -351,7 +350,8 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         uint32_t packed = 0;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          const int x = acc[i][j][4 * g + e];
+          int x = acc[i][j][4 * g + e];
+          if (rt) x = f32_roundtrip(x);
           int r;
           if (shift >= 1) r = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
           else r = wrap_to_i8(x);

@@ -21,6 +21,7 @@
 #include <stdlib.h>
 
 #include "common.h"
+#include "requant_math.h"
 
 namespace niti {
 namespace {
@@ -261,6 +262,146 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const int32_t* __rest
   if (absmax != nullptr && wave == 0) fold_absmax(absmax, lmax);
 }
 
+// Partial sums -> rounded gradient -> updated weights in one launch (the int32 gradient is not stored unless
+// asked for).  A workgroup owns kFinishV x 64 int4 columns at a grid-wide stride; its 4 wavefronts each add every
+// 4th slice and combine in LDS, wavefront 0 keeps the sums in registers, publishes the workgroup's largest
+// magnitude in its slot, waits for the slots of all workgroups (all resident: the host sizes the grid for that;
+// the wait is bounded by a wall-clock limit), derives the shift from the maximum over the slots and applies
+// w = clip(w - round(sum >> shift)).
+constexpr int kFinishV = 16;
+constexpr int kFinishSlot0 = 16;
+struct FinishArgs {
+  const int32_t* partial;
+  long long slice_stride;
+  int splits;
+  long long nv;        // int4 columns of the gradient: K*9*C / 4
+  int C, Cw;           // channels per gradient row / per weight row (Cw <= C; the rest is channel padding)
+  int8_t* w;           // [K][9][Cw], updated in place
+  int8_t* g8;          // optional rounded gradient, laid out like w
+  int32_t* dw;         // optional int32 gradient [K][9][C]
+  uint32_t* sync;      // word 0: max |sum| (output); word 1: wait gave up; words kFinishSlot0..: slots, zero on entry
+  int roundtrip, target_bits, method, trunc, bw_mode;
+  long long spin_limit;
+  int32_t* shift_out;
+  const int32_t* exp_a;
+  const int32_t* exp_b;
+  int32_t* exp_out;
+};
+
+__global__ __launch_bounds__(256) void wgrad_finish_kernel(const FinishArgs a) {
+  __shared__ v4i part[3][64];
+  __shared__ uint32_t gshare;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  v4i sum[kFinishV];
+  uint32_t lmax = 0;
+#pragma unroll
+  for (int v = 0; v < kFinishV; ++v) {
+    const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
+    if (static_cast<long long>(v) * gridDim.x * 64 >= a.nv) {  // uniform over the grid: nothing left at this stride
+      sum[v] = v4i{0, 0, 0, 0};
+      continue;
+    }
+    v4i s = {0, 0, 0, 0};
+    if (col < a.nv) {
+      int z = wave;
+      for (; z + 12 < a.splits; z += 16) {
+        const v4i v0 = reinterpret_cast<const v4i*>(a.partial + (z + 0) * a.slice_stride)[col];
+        const v4i v1 = reinterpret_cast<const v4i*>(a.partial + (z + 4) * a.slice_stride)[col];
+        const v4i v2 = reinterpret_cast<const v4i*>(a.partial + (z + 8) * a.slice_stride)[col];
+        const v4i v3 = reinterpret_cast<const v4i*>(a.partial + (z + 12) * a.slice_stride)[col];
+        s += (v0 + v1) + (v2 + v3);
+      }
+      for (; z < a.splits; z += 4) s += reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
+    }
+    if (wave > 0) part[wave - 1][lane] = s;
+    __syncthreads();
+    if (wave == 0) {
+      s += part[0][lane] + part[1][lane] + part[2][lane];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
+        const uint32_t u = uabs(s[e]);
+        lmax = u > lmax ? u : lmax;
+      }
+    }
+    sum[v] = s;
+    __syncthreads();
+  }
+  if (wave == 0) {
+    const uint32_t bmax = wave_max_u32(lmax);
+    const int nb = gridDim.x;
+    uint32_t* const slots = a.sync + kFinishSlot0;
+    if (lane == 0) __hip_atomic_store(&slots[blockIdx.x], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const long long t0 = wall_clock64();
+    uint32_t g = 0;
+    for (;;) {
+      bool ok = true;
+      g = 0;
+      for (int i = lane; i < nb; i += 64) {
+        const uint32_t v = __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && v != 0u;
+        g = v > g ? v : g;
+      }
+      if (__all(ok)) break;
+      if (wall_clock64() - t0 > a.spin_limit) {
+        if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        break;
+      }
+      __builtin_amdgcn_s_sleep(4);
+    }
+    g = wave_max_u32(g);
+    const uint32_t gmax = g != 0u ? g - 1u : 0u;
+    const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
+    if (blockIdx.x == 0 && lane == 0) {
+      const int sh = shift > 0 ? shift : 0;
+      a.sync[0] = gmax;
+      if (a.shift_out != nullptr) *a.shift_out = sh;
+      if (a.exp_out != nullptr)
+        *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+    }
+    const bool trunc = a.trunc != 0;
+    const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
+    const bool same_layout = a.Cw == a.C;
+#pragma unroll
+    for (int v = 0; v < kFinishV; ++v) {
+      const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
+      if (col >= a.nv) continue;
+      const v4i s = sum[v];
+      if (a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
+      int r[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
+        else r[e] = wrap_to_i8(s[e]);
+      }
+      if (same_layout) {
+        const uint32_t wold = reinterpret_cast<const uint32_t*>(a.w)[col];
+        uint32_t wnew = 0, gp = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * e)) & 0xFFu));
+          wnew |= (static_cast<uint32_t>(clip127(wo - r[e])) & 0xFFu) << (8 * e);
+          gp |= (static_cast<uint32_t>(r[e]) & 0xFFu) << (8 * e);
+        }
+        reinterpret_cast<uint32_t*>(a.w)[col] = wnew;
+        if (a.g8 != nullptr) reinterpret_cast<uint32_t*>(a.g8)[col] = gp;
+      } else {
+        const long long e0 = col * 4;
+        const long long row = e0 / a.C;
+        const int c0 = static_cast<int>(e0 - row * a.C);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (c0 + e < a.Cw) {
+            const long long wi = row * a.Cw + c0 + e;
+            a.w[wi] = static_cast<int8_t>(clip127(static_cast<int>(a.w[wi]) - r[e]));
+            if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
+          }
+        }
+      }
+    }
+  }
+}
+
 // Slices are spaced so that the same element of consecutive slices falls into different memory
 // channels (a stride that is a multiple of 64 KB would put them all into one).
 long long slice_stride_for(int C, int K) {
@@ -319,9 +460,8 @@ size_t wgrad3x3_workspace(int N, int H, int C, int K) {
   return static_cast<size_t>(pick_splits(N, H, C, K)) * slice_stride_for(C, K) * sizeof(int32_t);
 }
 
-int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, int H, int C, int K, bool roundtrip,
-                    uint32_t* absmax, void* workspace, hipStream_t stream) {
-  WgradArgs a;
+static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N, int H, int C, int K, void* workspace,
+                                    WgradArgs& a, int& splits, hipStream_t stream) {
   a.act = act;
   a.err = err;
   a.partial = static_cast<int32_t*>(workspace);
@@ -330,14 +470,20 @@ int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, in
   a.C = C;
   a.K = K;
   a.bands = N * H * H / 128;
-  const int splits = pick_splits(N, H, C, K);
+  splits = pick_splits(N, H, C, K);
   a.bands_per_split = (a.bands + splits - 1) / splits;
   a.act_bytes = static_cast<long long>(N) * H * H * C;
   a.err_bytes = static_cast<long long>(N) * H * H * K;
-  int st;
-  if (H == 32) st = launch_geom<32, 4, 1>(a, splits, stream);
-  else if (H == 16) st = launch_geom<16, 8, 1>(a, splits, stream);
-  else st = launch_geom<8, 8, 2>(a, splits, stream);
+  if (H == 32) return launch_geom<32, 4, 1>(a, splits, stream);
+  if (H == 16) return launch_geom<16, 8, 1>(a, splits, stream);
+  return launch_geom<8, 8, 2>(a, splits, stream);
+}
+
+int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, int H, int C, int K, bool roundtrip,
+                    uint32_t* absmax, void* workspace, hipStream_t stream) {
+  WgradArgs a;
+  int splits = 1;
+  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, workspace, a, splits, stream);
   if (st != NITI_OK) return st;
   const int64_t n = static_cast<int64_t>(K) * 9 * C;
   int64_t g = (n / 4 + 63) / 64;
@@ -345,6 +491,60 @@ int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, in
   hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0, stream, a.partial, dw, n,
                      static_cast<int64_t>(a.slice_stride), splits, roundtrip ? 1 : 0, absmax);
   return check_launch("wgrad_reduce");
+}
+
+// Workgroups of the finishing kernel for a [K][9][C] gradient (= sync slots), or 0 when it is too large for
+// the kernel's per-workgroup share.
+int wgrad3x3_finish_blocks(int C, int K) {
+  const long long groups = (static_cast<long long>(K) * 9 * C / 4 + 63) / 64;
+  const long long nb = groups < 1024 ? groups : 1024;
+  if (groups > nb * kFinishV) return 0;
+  return static_cast<int>(nb < 1 ? 1 : nb);
+}
+
+size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0 + (blocks + 15) / 16 * 16); }
+
+int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
+                           bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, void* workspace,
+                           hipStream_t stream) {
+  const int nb = wgrad3x3_finish_blocks(C, K);
+  if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large for the single-pass finish", K, C);
+  static int resident = 0;
+  if (resident == 0) {
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(wgrad_finish_kernel), 256, 0) != hipSuccess)
+      return fail(NITI_ERR_LAUNCH, "wgrad_update: cannot query occupancy");
+    resident = cus * per_cu;
+  }
+  if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: %d workgroups do not fit on the device at once (%d)", nb, resident);
+  WgradArgs a;
+  int splits = 1;
+  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, workspace, a, splits, stream);
+  if (st != NITI_OK) return st;
+  FinishArgs f{};
+  f.partial = a.partial;
+  f.slice_stride = a.slice_stride;
+  f.splits = splits;
+  f.nv = static_cast<long long>(K) * 9 * C / 4;
+  f.C = C;
+  f.Cw = w_channels;
+  f.w = w;
+  f.g8 = g8;
+  f.dw = dw;
+  f.sync = sync;
+  f.roundtrip = roundtrip ? 1 : 0;
+  f.target_bits = rq.target_bits;
+  f.method = rq.method;
+  f.trunc = rq.trunc;
+  f.bw_mode = rq.bw_mode;
+  f.spin_limit = rq.spin_limit;
+  f.shift_out = rq.shift_out;
+  f.exp_a = rq.exp_a;
+  f.exp_b = rq.exp_b;
+  f.exp_out = rq.exp_out;
+  hipLaunchKernelGGL(wgrad_finish_kernel, dim3(nb), dim3(256), 0, stream, f);
+  return check_launch("wgrad_finish");
 }
 
 }  // namespace niti

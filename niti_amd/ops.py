@@ -172,18 +172,77 @@ def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target
                          prepared_filter)
 
 
-def conv2d_wgrad(act, err, R, S, stride=1, padding=1, f32_epilogue=False, absmax=None):
-    """act [N,H,W,C] int8, err [N,P,Q,K] int8 -> dw [K,R,S,C] int32 (stride 1)."""
-    _chk_dev(act, err, absmax)
+_scratch = {}
+
+
+def scratch(nbytes: int, device) -> torch.Tensor:
+    """One grow-only int8 buffer per device for kernel workspaces that live only inside a call.  Calls on one
+    stream run in order, so they can all use the same memory - which also keeps the partial sums of
+    consecutive weight-gradient launches in the same cache-resident region instead of walking through fresh
+    allocations.  Not for use from several streams at once."""
+    key = str(device)
+    buf = _scratch.get(key)
+    if buf is None or buf.numel() < nbytes:
+        buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.int8, device=device)
+        _scratch[key] = buf
+    return buf
+
+
+def conv2d_wgrad(act, err, R, S, stride=1, padding=1, f32_epilogue=False, absmax=None, workspace=None):
+    """act [N,H,W,C] int8, err [N,P,Q,K] int8 -> dw [K,R,S,C] int32 (stride 1).  ``workspace``: int8 tensor of
+    at least niti_conv2d_i8_wgrad_workspace bytes (default: a fresh allocation)."""
+    _chk_dev(act, err, absmax, workspace)
     N, H, W, C = act.shape
     K = err.shape[3]
     dw = torch.empty((K, R, S, C), dtype=torch.int32, device=act.device)
     nbytes = L.lib().niti_conv2d_i8_wgrad_workspace(N, H, W, C, K, R, S, padding)
-    ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=act.device)
+    ws = workspace if workspace is not None else torch.empty(max(nbytes, 16), dtype=torch.int8, device=act.device)
+    if ws.numel() < nbytes:
+        raise RuntimeError("conv2d_wgrad: workspace of %d bytes needed, got %d" % (nbytes, ws.numel()))
     st = L.lib().niti_conv2d_i8_wgrad(_ptr(act), _ptr(err), _ptr(dw), N, H, W, C, K, R, S, stride, padding,
                                       _flags(f32_epilogue), _ptr(absmax), _ptr(ws), nbytes, _stream(act))
     L.check(st, "niti_conv2d_i8_wgrad")
     return dw
+
+
+def wgrad_update_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1) -> int:
+    """uint32 words of the sync buffer conv2d_wgrad_update needs; 0 when only the two-pass path covers the shape."""
+    return int(L.lib().niti_conv2d_i8_wgrad_update_sync_words(N, H, W, C, K, R, S, stride, padding))
+
+
+def conv2d_wgrad_update(act, err, w, stride=1, padding=1, f32_epilogue=False, mu=5, method="psto", div_mode="floor",
+                        bw_mode="int", sync=None, want_grad=False, want_dw=False, shift_out=None, exp_a=None, exp_b=None,
+                        exp_out=None, workspace=None):
+    """Weight gradient + grad_calc + weight update: act [N,H,W,C] int8 (C may carry zero channel padding), err
+    [N,H,W,K] int8, w [K,3,3,Cw] int8 updated in place.  Returns (g8 or None, dw int32 or None, device shift, sync)."""
+    _chk_dev(act, err, w, sync, shift_out, exp_a, exp_b, exp_out, workspace)
+    if act.dtype != torch.int8 or err.dtype != torch.int8 or w.dtype != torch.int8:
+        raise RuntimeError("conv2d_wgrad_update: int8 tensors expected")
+    N, H, W, C = act.shape
+    K, R, S, Cw = w.shape
+    if err.shape[3] != K:
+        raise RuntimeError("conv2d_wgrad_update: channel mismatch")
+    words = wgrad_update_sync_words(N, H, W, C, K, R, S, stride, padding)
+    if words == 0:
+        raise L.NitiError("conv2d_wgrad_update: shape not covered by the single-pass path")
+    if sync is None:
+        sync = torch.zeros(words, dtype=torch.int32, device=act.device)
+    elif sync.dtype != torch.int32 or sync.numel() < words:
+        raise RuntimeError("conv2d_wgrad_update: sync must be a zeroed int32 tensor of at least %d words" % words)
+    nbytes = L.lib().niti_conv2d_i8_wgrad_workspace(N, H, W, C, K, R, S, padding)
+    ws = workspace if workspace is not None else torch.empty(max(nbytes, 16), dtype=torch.int8, device=act.device)
+    if ws.numel() < nbytes:
+        raise RuntimeError("conv2d_wgrad_update: workspace of %d bytes needed, got %d" % (nbytes, ws.numel()))
+    g8 = torch.empty(w.shape, dtype=torch.int8, device=w.device) if want_grad else None
+    dw = torch.empty((K, R, S, C), dtype=torch.int32, device=w.device) if want_dw else None
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=w.device)
+    st = L.lib().niti_conv2d_i8_wgrad_update(_ptr(act), _ptr(err), _ptr(w), Cw, N, H, W, C, K, R, S, stride, padding,
+                                             _flags(f32_epilogue), mu, L.ROUND[method], L.DIV[div_mode], L.BW[bw_mode],
+                                             _ptr(sync), sync.numel(), _ptr(g8), _ptr(dw), _ptr(shift_out), _ptr(exp_a),
+                                             _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes, _stream(act))
+    L.check(st, "niti_conv2d_i8_wgrad_update")
+    return g8, dw, shift_out, sync
 
 
 def gemm(a, b, trans_a=False, trans_b=False, absmax=None, out=None):

@@ -185,6 +185,7 @@ def grad_calc(int32_acc, mu, absmax=None, rand=None):
 
 
 FUSE_CONV_REQUANT = True     # run convolution + requantisation as one launch where the library covers the shape
+KEEP_INT32_GRAD = False      # also store layer.grad_int32acc when the weight gradient is rounded and applied in one call
 _fused_refused = set()       # (dgrad, input shape, filter shape, stride, padding) the device turned out too small for
 
 
@@ -391,15 +392,46 @@ class TiConv2d(UpdateWeight):
                 err_out, _, new_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
                                                exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
             self.err_exp = new_exp
-        amg = ops.new_scalar_u32(dev)
         K, R, S, C = self.weight.shape
+        if self._wgrad_update_fused(err_in, grad_rand):
+            if not self.first_layer:
+                return err_out, self.err_exp
+            return None
+        amg = ops.new_scalar_u32(dev)
         dw = ops.conv2d_wgrad(self.act16, err_in, R, S, self.stride, self.padding,
-                              f32_epilogue=F32_EPILOGUE and not self.first_layer, absmax=amg)
+                              f32_epilogue=F32_EPILOGUE and not self.first_layer, absmax=amg,
+                              workspace=self._wgrad_workspace(err_in))
         # zero-padded input channels give zero gradient columns: drop them (they cannot raise the range)
         self.grad_int32acc = dw if dw.shape[3] == C else dw[..., :C].contiguous()
         self.weight_update(amg, grad_rand)
         if not self.first_layer:
             return err_out, self.err_exp
+
+    def _wgrad_workspace(self, err_in):
+        from . import _lib
+        N, H, W, C16 = self.act16.shape
+        K, R, S, _ = self.weight.shape
+        return ops.scratch(_lib.lib().niti_conv2d_i8_wgrad_workspace(N, H, W, C16, K, R, S, self.padding), err_in.device)
+
+    def _wgrad_update_fused(self, err_in, grad_rand):
+        """Weight gradient, grad_calc and the weight update as one call into the library (no int32 gradient in
+        memory unless KEEP_INT32_GRAD).  False when the call needs the separate steps."""
+        method = _method_name(GRAD_ROUND_METHOD)
+        if not FUSE_CONV_REQUANT or method == "sto" or grad_rand is not None or not self.weight.is_contiguous():
+            return False
+        N, H, W, C16 = self.act16.shape
+        K, R, S, C = self.weight.shape
+        if ops.wgrad_update_sync_words(N, H, W, C16, K, R, S, self.stride, self.padding) == 0:
+            return False
+        dev = err_in.device
+        self.grad_exp = torch.empty(1, dtype=torch.int32, device=dev)
+        self.grad, dw, self.grad_shift, _ = ops.conv2d_wgrad_update(
+            self.act16, err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE and not self.first_layer,
+            mu=GRAD_BITWIDTH, method=method, div_mode=DIV_MODE, bw_mode=BW_MODE, want_grad=self.keep_grad,
+            want_dw=KEEP_INT32_GRAD, exp_a=_exp_tensor(self.err_exp, dev), exp_b=_exp_tensor(self.act_in_exp, dev),
+            exp_out=self.grad_exp, workspace=self._wgrad_workspace(err_in))
+        self.grad_int32acc = None if dw is None else (dw if dw.shape[3] == C else dw[..., :C].contiguous())
+        return True
 
 
 class TiLinear(UpdateWeight):

@@ -192,6 +192,43 @@ def test_conv_dgrad_requant(dev, case):
             assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
 
 
+@pytest.mark.parametrize("case", [(4, 32, 16, 32), (8, 16, 128, 64), (6, 8, 80, 144), (64, 8, 64, 256), (16, 16, 256, 128),
+                                  (2, 8, 16, 16), (4, 8, 3, 16), (8, 32, 3, 128), (32, 8, 512, 512)])
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+def test_conv_wgrad_update(dev, case, div_mode):
+    """wgrad + grad_calc + weight update in one call against the oracle's three steps."""
+    import torch.nn.functional as F
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_wgrad_update", case, div_mode)
+    g = torch.Generator().manual_seed(970 + C + K)
+    act, err, w = ri8(g, N, Q, Q, C), ri8(g, N, Q, Q, K, lo=-40, hi=40), ri8(g, K, 3, 3, C)
+    dw_ref = co.conv_wgrad(act, err, 3, 3, 1, 1)
+    act16 = F.pad(act, (0, 16 - C % 16)) if C % 16 else act
+    for method, mu in (("psto", 5), ("round", 3)):
+        g8_ref, sh_ref = po.grad_calc(dw_ref, mu, method, div_mode)
+        w_ref = po.weight_update(w, g8_ref)
+        wd = w.to(dev).clone()
+        ea = torch.tensor([-4], dtype=torch.int32, device=dev)
+        eo = torch.zeros(1, dtype=torch.int32, device=dev)
+        g8, dw, sh, sync = ops.conv2d_wgrad_update(act16.to(dev).contiguous(), err.to(dev), wd, mu=mu, method=method,
+                                                   div_mode=div_mode, want_grad=True, want_dw=True, exp_a=ea, exp_out=eo)
+        torch.cuda.synchronize()
+        sync = sync.cpu()
+        assert int(sync[1]) == 0, "grid-wide wait timed out"
+        assert int(sync[0]) == po.absmax(dw_ref)
+        assert torch.equal(dw.cpu()[..., :C], dw_ref)
+        assert int(sh.cpu()) == sh_ref and int(eo.cpu()) == sh_ref - 4
+        assert torch.equal(g8.cpu(), g8_ref)
+        assert torch.equal(wd.cpu(), w_ref)
+        # without the optional outputs
+        wd2 = w.to(dev).clone()
+        ops.conv2d_wgrad_update(act16.to(dev).contiguous(), err.to(dev), wd2, mu=mu, method=method, div_mode=div_mode)
+        assert torch.equal(wd2.cpu(), w_ref)
+
+
 def test_conv_requant_rejects_what_it_does_not_cover(dev):
     from niti_amd import ops
     from niti_amd._lib import NitiError
