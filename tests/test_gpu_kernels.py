@@ -109,6 +109,48 @@ FUSED_CASES = [(4, 8, 16, 16), (4, 8, 64, 128), (8, 8, 80, 144), (1, 16, 16, 48)
                (8, 32, 128, 128), (12, 8, 512, 128)]
 
 
+@pytest.fixture(params=["auto", "64", "128"])
+def halo_tile(request):
+    """Channel tile of the 3x3 halo kernel: the library's own choice, or pinned to either width."""
+    import os
+    old = os.environ.get("NITI_HALO_KT")
+    if request.param != "auto":
+        os.environ["NITI_HALO_KT"] = request.param
+    yield request.param
+    if old is None:
+        os.environ.pop("NITI_HALO_KT", None)
+    else:
+        os.environ["NITI_HALO_KT"] = old
+
+
+@pytest.mark.parametrize("case", [(8, 8, 64, 128), (4, 8, 80, 24), (3, 16, 192, 260), (2, 32, 16, 64), (8, 32, 128, 256), (12, 8, 512, 128)])
+def test_conv_halo_tiles(dev, case, halo_tile):
+    """Forward, data gradient and the requantising variant with both channel tiles of the halo kernel."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_halo_tiles", case, halo_tile)
+    g = torch.Generator().manual_seed(990 + C + K)
+    x, w = ri8(g, N, Q, Q, C), ri8(g, K, 3, 3, C)
+    ref = po.conv2d_fprop_i32(x, w, 1, 1)
+    am = ops.new_scalar_u32(dev)
+    y = ops.conv2d_fprop(x.to(dev), w.to(dev), 1, 1, absmax=am)
+    assert torch.equal(y.cpu(), ref) and int(am.cpu()) == po.absmax(ref)
+    if K % 16 == 0:
+        r8, sh_ref = po.act_calc(ref, 0)
+        y8, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev))
+        assert int(sync.cpu()[1]) == 0 and int(sync.cpu()[0]) == po.absmax(ref)
+        assert torch.equal(y8.cpu(), r8) and int(sh.cpu()) == sh_ref
+        e = ri8(g, N, Q, Q, K)
+        dref = co.conv_dgrad(e, w, Q, Q, 1, 1)
+        d8, dsh = po.err_calc(dref)
+        dx = ops.conv2d_dgrad(e.to(dev), w.to(dev), 1, 1)
+        assert torch.equal(dx.cpu(), dref)
+        dx8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev))
+        assert int(sync.cpu()[1]) == 0 and torch.equal(dx8.cpu(), d8) and int(sh.cpu()) == dsh
+
+
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 @pytest.mark.parametrize("method", ["round", "psto"])
 @pytest.mark.parametrize("case", FUSED_CASES)
