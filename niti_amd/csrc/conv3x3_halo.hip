@@ -364,24 +364,30 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
     constexpr int PROW = NWF * 32 + 16;  // the wavefront's channels of one pixel, padded
     int8_t* patch = smem + wave * (64 * PROW);
+    // the vector ALU work of this block is what the whole device does at this moment (every workgroup is here
+    // at the same time), so the common rounding mode gets a short form
+    const bool fast = shift >= 1 && !trunc && !psto;
+    const int sm1 = shift - 1, lo = relu ? 0 : -127;
 #pragma unroll
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          uint32_t packed = 0;
+          int r[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             int x = acc[i][j][4 * g + e];
             if (rt) x = f32_roundtrip(x);
-            int r;
-            if (shift >= 1) r = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
-            else r = wrap_to_i8(x);
-            if (relu && r < 0) r = 0;
-            packed |= (static_cast<uint32_t>(r) & 0xFFu) << (8 * e);
+            if (fast) {
+              r[e] = round_nearest_floor_fast(x, sm1, lo);
+            } else {
+              if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
+              else r[e] = wrap_to_i8(x);
+              if (relu && r[e] < 0) r[e] = 0;
+            }
           }
-          *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = packed;
+          *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = pack4_i8(r[0], r[1], r[2], r[3]);
         }
     // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y8, 0, a.y8_bytes, 0x00020000);

@@ -72,6 +72,22 @@ __host__ __device__ inline int round_one32(int x, int s, bool trunc) {
   return r > 127 ? 127 : (r < -127 ? -127 : r);
 }
 
+// Four rounded values -> four bytes (value e in byte e), two's complement low bytes.
+__device__ inline uint32_t pack4_i8(int r0, int r1, int r2, int r3) {
+  // v_perm_b32: selector byte 0x00-0x03 picks a byte of the second operand, 0x04-0x07 of the first, 0x0c is zero
+  const uint32_t lo = __builtin_amdgcn_perm(static_cast<uint32_t>(r1), static_cast<uint32_t>(r0), 0x0c0c0400u);
+  const uint32_t hi = __builtin_amdgcn_perm(static_cast<uint32_t>(r3), static_cast<uint32_t>(r2), 0x0c0c0400u);
+  return lo | (hi << 16);
+}
+
+// Nearest rounding with floor division for 1 <= s and |x| < 2^(s + 7) (true when s comes from the tensor's own
+// range): floor((x + 2^(s-1)) / 2^s) = ((x >> (s-1)) + 1) >> 1, then clip to [lo, 127] (lo = -127, or 0 for a
+// fused ReLU).  Three shifts/adds and one median instead of the general path's dozen operations.
+__device__ inline int round_nearest_floor_fast(int x, int sm1, int lo) {
+  const int r = ((x >> sm1) + 1) >> 1;
+  return min(max(r, lo), 127);
+}
+
 // shift < 1: the reference converts int32 to int8 by keeping the low byte
 __device__ inline int wrap_to_i8(int x) { return static_cast<int>(static_cast<int8_t>(static_cast<uint32_t>(x) & 0xFFu)); }
 
