@@ -78,13 +78,14 @@ struct HaloArgs {
 constexpr int kSyncSlot0 = 16;
 
 // Q: image width = height; BR: output rows of one image per workgroup; NI: images per workgroup; BR*NI*Q == 256.
-// The halo tile is NI*(BR+2) rows of RP slots of 32 bytes; RP is a multiple of 8 so that the bank of a slot
+// The halo tile is NI*(BR+2) rows of Q slots of 32 bytes; Q is a multiple of 8 so that the bank of a slot
 // depends on its column only, and the 16-byte halves of a slot are swapped where ((column >> 3) ^ row) is odd:
 // 16 lanes reading consecutive columns of one row, or 8 + 8 columns of two adjacent rows, then hit 16 distinct
 // bank groups.
 template <int Q, int BR, int NI, int KT>
 struct HGeom {
-  static constexpr int RP = (Q + 2 + 7) / 8 * 8;
+  static constexpr int RP = Q;                             // no halo columns: horizontal neighbours come from lane shifts
+  static_assert(Q % 8 == 0, "bank mapping");
   static constexpr int HR = BR + 2;
   static constexpr int SLOTS = NI * HR * RP;
   static constexpr int ACT_INSTR = (SLOTS + 31) / 32;      // one instruction fills 32 slots
@@ -129,7 +130,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const int row = slot / G::RP, col = slot - row * G::RP;
     const int ni = row / G::HR, h = row - ni * G::HR;
     const int half = (lane & 1) ^ (((col >> 3) ^ row) & 1);
-    const int ih = p0 + h - 1, iw = col - 1;
+    const int ih = p0 + h - 1, iw = col;
     int off = kOob;
     if (slot < G::SLOTS && n0 + ni < a.N && ih >= 0 && ih < Q && iw >= 0 && iw < Q)
       off = (((n0 + ni) * Q + ih) * Q + iw) * a.C + half * 16;
@@ -185,18 +186,17 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const int grow = KT == 128 ? i * 32 + lr : wc * 32 + lr;
     w_addr[i] = (KT == 128 ? wc * 6144 : 0) + grow * 32 + ((lk ^ ((grow >> 3) & 1)) << 4);
   }
-  int p_addr[2][3];           // [pixel tile][s]: halo slot of this lane's pixel for filter column s, filter row 0
+  int p_addr[2];              // [pixel tile]: halo slot of this lane's pixel, filter row 0
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
     const int pix = wp_ * 64 + j * 32 + lr;       // output pixel inside the workgroup's 256
     const int prow = pix / Q, pw = pix % Q;        // row inside the workgroup's rows, column
     const int hrow = (prow / BR) * G::HR + (prow % BR);
-#pragma unroll
-    for (int s = 0; s < 3; ++s) {
-      const int col = pw + s;
-      p_addr[j][s] = (hrow * G::RP + col) * 32 + ((lk ^ (((col >> 3) ^ hrow) & 1)) << 4);
-    }
+    p_addr[j] = (hrow * G::RP + pw) * 32 + ((lk ^ (((pw >> 3) ^ hrow) & 1)) << 4);
   }
+  // lanes whose left / right neighbour lies outside the image take the zero padding instead of the shifted value
+  const int keep_l = (lr % Q) != 0 ? -1 : 0;
+  const int keep_r = (lr % Q) != Q - 1 ? -1 : 0;
 
   v16i acc[NWF][2];  // [channel tile][pixel tile]
 #pragma unroll
@@ -232,23 +232,38 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (r == 0 && more) issue_act(ci + 1, (ci + 1) & 1);
       const int8_t* sw = w_buf + (t % G::WSTAGES) * G::W_BYTES;
       const int roff = r * G::RP * 32;
-      v4i wf[2][NWF], pf[2][2];
-      auto fetch = [&](int s, int slot) {
+      // pixels under the centre column of this filter row; the fragment layout is lane -> (pixel lane % 32,
+      // 16 channels lane / 32), so the pixel to the left is one lane down and the one to the right one lane up
+      v4i pc[2];
 #pragma unroll
-        for (int i = 0; i < NWF; ++i) wf[slot][i] = *reinterpret_cast<const v4i*>(sw + w_addr[i] + s * 2048);
+      for (int j = 0; j < 2; ++j) pc[j] = *reinterpret_cast<const v4i*>(sa + ((p_addr[j] + roff) ^ ((r & 1) << 4)));
+      v4i wf[3][NWF];
 #pragma unroll
-        for (int j = 0; j < 2; ++j) pf[slot][j] = *reinterpret_cast<const v4i*>(sa + ((p_addr[j][s] + roff) ^ ((r & 1) << 4)));
-      };
-      fetch(0, 0);
-      fetch(1, 1);
+      for (int s = 0; s < 3; ++s)
 #pragma unroll
-      for (int s = 0; s < 3; ++s) {
+        for (int i = 0; i < NWF; ++i) wf[s][i] = *reinterpret_cast<const v4i*>(sw + w_addr[i] + ((s + 1) % 3) * 2048);
+      // order: centre tap (needs no shifting) first, then left, then right; wf[0] = tap s=1, wf[1] = s=2, wf[2] = s=0
 #pragma unroll
-        for (int i = 0; i < NWF; ++i)
+      for (int i = 0; i < NWF; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[s & 1][i], pf[s & 1][j], acc[i][j], 0, 0, 0);
-        if (s == 0) fetch(2, 0);
-      }
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
+      v4i ps[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
+#pragma unroll
+      for (int i = 0; i < NWF; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
+#pragma unroll
+      for (int i = 0; i < NWF; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
     }
   }
 
