@@ -294,13 +294,11 @@ __global__ __launch_bounds__(256) void wgrad_finish_kernel(const FinishArgs a) {
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   v4i sum[kFinishV];
   uint32_t lmax = 0;
+  // phase 1: every wavefront adds its share of the slices for all of the workgroup's columns; no barrier in
+  // here, so the loads of all columns are in flight together
 #pragma unroll
   for (int v = 0; v < kFinishV; ++v) {
     const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
-    if (static_cast<long long>(v) * gridDim.x * 64 >= a.nv) {  // uniform over the grid: nothing left at this stride
-      sum[v] = v4i{0, 0, 0, 0};
-      continue;
-    }
     v4i s = {0, 0, 0, 0};
     if (col < a.nv) {
       int z = wave;
@@ -313,18 +311,24 @@ __global__ __launch_bounds__(256) void wgrad_finish_kernel(const FinishArgs a) {
       }
       for (; z < a.splits; z += 4) s += reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
     }
-    if (wave > 0) part[wave - 1][lane] = s;
+    sum[v] = s;
+  }
+  // phase 2: combine the four wavefronts' shares in LDS; wavefront 0 keeps the totals
+#pragma unroll
+  for (int v = 0; v < kFinishV; ++v) {
+    if (static_cast<long long>(v) * gridDim.x * 64 >= a.nv) continue;  // uniform over the grid: nothing at this stride
+    if (wave > 0) part[wave - 1][lane] = sum[v];
     __syncthreads();
     if (wave == 0) {
-      s += part[0][lane] + part[1][lane] + part[2][lane];
+      v4i s = sum[v] + part[0][lane] + part[1][lane] + part[2][lane];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
         const uint32_t u = uabs(s[e]);
         lmax = u > lmax ? u : lmax;
       }
+      sum[v] = s;
     }
-    sum[v] = s;
     __syncthreads();
   }
   if (wave == 0) {
