@@ -121,6 +121,11 @@ int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N,
  * flags: NITI_EPI_F32_ROUNDTRIP, NITI_CONV_FILTER_PREPARED (w is a copy made by niti_conv2d_i8_filter_prepare;
  * otherwise workspace must hold niti_conv2d_i8_filter_workspace bytes).  rq_flags: NITI_RQ_RELU.
  * shift_out / exp_a / exp_b / exp_out as in niti_requant_i32_i8 (each may be NULL).
+ * relu_mask (data gradient only, may be NULL): int8 [N,H,W,C] like dx8; elements whose mask byte is not positive
+ * are stored as zero AFTER the range and the rounding were taken from the unmasked sums.  Passing the layer's
+ * own input activations folds in the backward pass of a ReLU that precedes the layer (TiReLU.backward,
+ * ti_torch.py:284-290) - also across a max-pool in between, whose backward routes gradients only to positions
+ * equal to the pooled maximum.
  */
 size_t niti_conv2d_i8_requant_sync_words(int N, int H, int W, int C, int K, int R, int S, int stride, int pad, int dgrad);
 int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, int8_t* y8, int N, int H, int W, int C, int K, int R,
@@ -130,7 +135,8 @@ int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, int8_t* y8, i
                                  size_t workspace_bytes, void* stream);
 int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int N, int H, int W, int C, int K, int R,
                                  int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
-                                 int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
+                                 int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync, size_t sync_words,
+                                 int32_t* shift_out,
                                  const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
                                  size_t workspace_bytes, void* stream);
 

@@ -219,9 +219,9 @@ extern "C" size_t niti_conv2d_i8_requant_sync_words(int N, int H, int W, int C, 
 
 static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_t* w, int8_t* y8, int N, int H, int W, int C,
                         int K, int R, int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
-                        int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
-                        const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace, size_t workspace_bytes,
-                        void* stream) {
+                        int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync, size_t sync_words,
+                        int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
+                        size_t workspace_bytes, void* stream) {
   clear_error();
   int st = check_conv_dims(who, N, H, W, C, K, R, S, stride, pad);
   if (st != NITI_OK) return st;
@@ -249,7 +249,8 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
     if (st != NITI_OK) return st;
     wp = static_cast<const int8_t*>(workspace);
   }
-  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out};
+  if (relu_mask != nullptr && !aligned16(relu_mask)) return fail(NITI_ERR_INVALID_ARG, "%s: relu_mask must be 16-byte aligned", who);
+  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out, relu_mask};
   return launch_conv3x3_halo_requant(x, wp, y8, N, Hk, Ck, Kk, flags, sync, rq, s);
 }
 
@@ -259,16 +260,16 @@ extern "C" int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, in
                                             int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
                                             void* workspace, size_t workspace_bytes, void* stream) {
   return conv_requant("conv_fprop_requant", 0, x, w, y8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method, div_mode,
-                      bw_mode, rq_flags, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
+                      bw_mode, rq_flags, nullptr, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
 }
 
 extern "C" int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int N, int H, int W, int C, int K,
                                             int R, int S, int stride, int pad, unsigned flags, int target_bits, int method,
-                                            int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words,
-                                            int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
-                                            void* workspace, size_t workspace_bytes, void* stream) {
+                                            int div_mode, int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync,
+                                            size_t sync_words, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b,
+                                            int32_t* exp_out, void* workspace, size_t workspace_bytes, void* stream) {
   return conv_requant("conv_dgrad_requant", 1, err, w, dx8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method, div_mode,
-                      bw_mode, rq_flags, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
+                      bw_mode, rq_flags, relu_mask, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
 }
 
 extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad) {
@@ -355,7 +356,7 @@ extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err,
     return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: act, err and dw_out must be 16-byte aligned");
   if (w_channels == C && (reinterpret_cast<uintptr_t>(w) % 4 != 0 || (g8_out != nullptr && reinterpret_cast<uintptr_t>(g8_out) % 4 != 0)))
     return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: w and g8_out must be 4-byte aligned");
-  RequantSpec rq{mu, method, div_mode == NITI_DIV_TRUNC, bw_mode, 0u, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out};
+  RequantSpec rq{mu, method, div_mode == NITI_DIV_TRUNC, bw_mode, 0u, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out, nullptr};
   return launch_wgrad3x3_update(act, err, w, w_channels, N, H, C, K, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, sync, rq, g8_out,
                                 dw_out, workspace, static_cast<hipStream_t>(stream));
 }
@@ -407,5 +408,19 @@ extern "C" int niti_gemm_i8(int trans_a, int trans_b, const int8_t* a, const int
   if (!aligned16(a_use) || !aligned16(b_use)) return fail(NITI_ERR_INVALID_ARG, "gemm: operands must be 16-byte aligned");
   // a 1x1 convolution over an m x 1 x 1 "image" with kp channels and n filters
   ConvProblem p{a_use, b_use, c, absmax, m, 1, 1, kp, n, 1, 1, 1, 0, n, n, n, 1, 1, flags};
+  // few output tiles and a long reduction (a fully connected layer on a batch): split the reduction over
+  // workgroups that add into the zeroed output (integer addition: any split gives the same bits), then one
+  // pass for the range
+  const long long tiles = static_cast<long long>((m + 127) / 128) * ((n + 127) / 128);
+  const int split = tiles >= 128 ? 1 : pick_split(tiles, (kp + 63) / 64);
+  if (split > 1) {
+    const int64_t nout = static_cast<int64_t>(m) * n;
+    if ((st = launch_fill_u32(reinterpret_cast<uint32_t*>(c), nout, 0u, s)) != NITI_OK) return st;
+    p.absmax = nullptr;
+    p.split_k = split;
+    if ((st = launch_conv_igemm(p, s)) != NITI_OK) return st;
+    if (absmax == nullptr && !(flags & NITI_EPI_F32_ROUNDTRIP)) return NITI_OK;
+    return launch_post_i32(c, nout, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, absmax, s);
+  }
   return launch_conv_igemm(p, s);
 }

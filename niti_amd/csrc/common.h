@@ -131,6 +131,7 @@ struct RequantSpec {
   const int32_t* exp_a;
   const int32_t* exp_b;
   int32_t* exp_out;
+  const int8_t* mask;      // conv + requantisation only: optional ReLU-backward mask, laid out like the output
 };
 int wgrad3x3_finish_blocks(int C, int K);
 size_t wgrad3x3_sync_words(int blocks);

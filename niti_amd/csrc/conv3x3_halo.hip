@@ -64,6 +64,7 @@ struct HaloArgs {
   unsigned flags;
   // requantising variant only
   int8_t* y8;         // [N,Q,Q,K] int8
+  const int8_t* mask; // optional [N,Q,Q,K] int8: outputs whose mask byte is not positive are stored as zero
   uint32_t* sync;     // word 0: max |sum| of the launch (output), word 1: set when the wait gave up,
                       // words kSyncSlot0..: one slot per workgroup, max + 1; all zero on entry
   long long y8_bytes;
@@ -413,9 +414,15 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
     for (int t = 0; t < 64 / PPI; ++t) {
       const int pl = t * PPI + prow;
-      const v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
+      v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
       const int m = pixbase + wp_ * 64 + pl;
       const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
+      if (a.mask != nullptr) {  // ReLU backward of the layer below, folded in: its output is this layer's input
+        const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
+        const auto mk = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] &= static_cast<int>(positive_bytes(static_cast<uint32_t>(mk[q])));
+      }
       __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0);
     }
   }
@@ -574,6 +581,7 @@ int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, i
   HaloArgs a;
   fill_common(a, x, wp, N, H, C, K, flags);
   a.y8 = y8;
+  a.mask = rq.mask;
   a.sync = sync;
   a.y8_bytes = static_cast<long long>(N) * H * H * K;
   a.target_bits = rq.target_bits;

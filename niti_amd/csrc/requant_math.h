@@ -88,6 +88,13 @@ __device__ inline int round_nearest_floor_fast(int x, int sm1, int lo) {
   return min(max(r, lo), 127);
 }
 
+// 0xFF in every byte of m that is positive as an int8, 0x00 elsewhere (the ReLU-backward test on four activations)
+__host__ __device__ inline uint32_t positive_bytes(uint32_t m) {
+  const uint32_t nz = (((m & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | m) & 0x80808080u;  // bit 7 where the byte is non-zero
+  const uint32_t pos = nz & ~m;                                               // ... and its sign bit is clear
+  return (pos >> 7) * 0xFFu;
+}
+
 // shift < 1: the reference converts int32 to int8 by keeping the low byte
 __device__ inline int wrap_to_i8(int x) { return static_cast<int>(static_cast<int8_t>(static_cast<uint32_t>(x) & 0xFFu)); }
 

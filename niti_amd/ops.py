@@ -110,14 +110,18 @@ def conv_requant_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1, dgrad=
 
 
 def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epilogue, target_bits, method, div_mode,
-                  bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter):
-    _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter)
+                  bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None):
+    _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask)
+    if relu_mask is not None and (relu_mask.dtype != torch.int8 or tuple(relu_mask.shape) != tuple(out_shape)):
+        raise RuntimeError("%s: relu_mask must be int8 and shaped like the output" % entry)
     if x.dtype != torch.int8 or w.dtype != torch.int8:
         raise RuntimeError("%s: int8 tensors expected" % entry)
     N, H, W, C, K, R, S = dims
     words = conv_requant_sync_words(N, H, W, C, K, R, S, stride, padding, dgrad)
     if words == 0:
         raise L.NitiError("%s: shape not covered by the single-launch path" % entry)
+    if sync is None:
+        sync = sync_arena.take(words, x.device)
     if sync is None:
         sync = torch.zeros(words, dtype=torch.int32, device=x.device)
     elif sync.dtype != torch.int32 or sync.numel() < words:
@@ -132,10 +136,10 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
         nbytes = L.lib().niti_conv2d_i8_filter_workspace(N, H, W, C, K, R, S, stride, padding, int(dgrad))
         ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=x.device)
         wptr = _ptr(w)
-    st = getattr(L.lib(), entry)(_ptr(x), wptr, _ptr(y), N, H, W, C, K, R, S, stride, padding, flags, target_bits,
-                                 L.ROUND[method], L.DIV[div_mode], L.BW[bw_mode], L.RQ_RELU if relu else 0, _ptr(sync),
-                                 sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes,
-                                 _stream(x))
+    head = (_ptr(x), wptr, _ptr(y), N, H, W, C, K, R, S, stride, padding, flags, target_bits, L.ROUND[method],
+            L.DIV[div_mode], L.BW[bw_mode], L.RQ_RELU if relu else 0)
+    tail = (_ptr(sync), sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes, _stream(x))
+    st = getattr(L.lib(), entry)(*(head + ((_ptr(relu_mask),) if dgrad else ()) + tail))
     L.check(st, entry)
     return y, shift_out, sync
 
@@ -159,8 +163,10 @@ def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_b
 
 def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None):
-    """conv2d_dgrad + requant as one launch: err [N,P,Q,K] int8, w [K,R,S,C] int8 -> ([N,H,W,C] int8, shift, sync)."""
+                         prepared_filter=None, relu_mask=None):
+    """conv2d_dgrad + requant as one launch: err [N,P,Q,K] int8, w [K,R,S,C] int8 -> ([N,H,W,C] int8, shift, sync).
+    ``relu_mask`` (int8 [N,H,W,C]): results whose mask element is not positive are stored as zero, after range
+    and rounding were taken from the unmasked sums (the backward pass of a ReLU in front of the layer)."""
     N, P, Q, K = err.shape
     K2, R, S, C = w.shape
     if K2 != K:
@@ -169,7 +175,7 @@ def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target
     W = Q - 2 * padding + S - 1
     return _conv_requant("niti_conv2d_i8_dgrad_requant", True, err, w, (N, H, W, C), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, False, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter)
+                         prepared_filter, relu_mask)
 
 
 _scratch = {}
@@ -186,6 +192,40 @@ def scratch(nbytes: int, device) -> torch.Tensor:
         buf = torch.empty(max(nbytes, 1 << 20), dtype=torch.int8, device=device)
         _scratch[key] = buf
     return buf
+
+
+class _SyncArena:
+    """Zeroed int32 words for the single-launch kernels of one training step: one fill per step instead of one
+    per kernel.  ``reset`` zeroes the whole arena and starts handing out slices from its beginning; ``take``
+    returns the next zeroed slice, or None when the arena has not been reset since it ran out (the caller then
+    allocates its own zeroed words).  Slices are handed out once per reset, so a kernel never sees words another
+    kernel of the same step wrote."""
+
+    WORDS = 1 << 16
+
+    def __init__(self):
+        self.buf = {}
+        self.off = {}
+
+    def reset(self, device):
+        key = str(device)
+        if key not in self.buf:
+            self.buf[key] = torch.zeros(self.WORDS, dtype=torch.int32, device=device)
+        else:
+            self.buf[key].zero_()
+        self.off[key] = 0
+
+    def take(self, words, device):
+        key = str(device)
+        off = self.off.get(key)
+        if off is None or off + words > self.WORDS:
+            self.off[key] = None
+            return None
+        self.off[key] = off + (words + 31) // 32 * 32
+        return self.buf[key][off:off + words]
+
+
+sync_arena = _SyncArena()
 
 
 def conv2d_wgrad(act, err, R, S, stride=1, padding=1, f32_epilogue=False, absmax=None, workspace=None):
@@ -225,6 +265,8 @@ def conv2d_wgrad_update(act, err, w, stride=1, padding=1, f32_epilogue=False, mu
     words = wgrad_update_sync_words(N, H, W, C, K, R, S, stride, padding)
     if words == 0:
         raise L.NitiError("conv2d_wgrad_update: shape not covered by the single-pass path")
+    if sync is None:
+        sync = sync_arena.take(words, act.device)
     if sync is None:
         sync = torch.zeros(words, dtype=torch.int32, device=act.device)
     elif sync.dtype != torch.int32 or sync.numel() < words:

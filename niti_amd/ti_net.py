@@ -4,7 +4,7 @@ import collections
 import torch
 from torch.nn.modules import Module
 
-from . import ti_torch
+from . import ops, ti_torch
 from .ti_loss import TiLoss
 
 
@@ -20,6 +20,18 @@ class TiNet(Module):
             if isinstance(a, ti_torch.TiConv2d) and isinstance(b, ti_torch.TiReLU):
                 a.fuse_relu = True
                 b.fused = True
+        # ReLU [-> max-pool] -> TiConv2d: the convolution zeroes its data gradient where its own input (the ReLU's
+        # possibly pooled output) is not positive, which is that ReLU's backward pass (a max-pool routes gradients
+        # only to elements equal to the pooled maximum, so masking before or after its backward is the same)
+        for i, l in enumerate(layers):
+            if not isinstance(l, ti_torch.TiReLU):
+                continue
+            j = i + 1
+            if j < len(layers) and isinstance(layers[j], ti_torch.TiMaxpool2d):
+                j += 1
+            if j < len(layers) and isinstance(layers[j], ti_torch.TiConv2d) and not layers[j].first_layer:
+                layers[j].relu_below = True
+                l.bwd_folded = True
         return self
 
     def forward(self, x):
@@ -30,6 +42,7 @@ class TiNet(Module):
 
     def forward_int8(self, x_data, x_exp=0):
         """Same as forward() for a batch that already is int8 NHWC with exponent ``x_exp``."""
+        ops.sync_arena.reset(x_data.device)     # one fill for the range-exchange words of the whole step
         self.out, self.out_exp = self.forward_layers((x_data, x_exp))
         return self.out, self.out_exp
 

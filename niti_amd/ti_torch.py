@@ -189,7 +189,7 @@ KEEP_INT32_GRAD = False      # also store layer.grad_int32acc when the weight gr
 _fused_refused = set()       # (dgrad, input shape, filter shape, stride, padding) the device turned out too small for
 
 
-def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b):
+def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None):
     """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
     exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
     single-launch kernel, or more workgroups than the device holds at once."""
@@ -208,7 +208,7 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
     from ._lib import NitiError
     exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
     call = ops.conv2d_dgrad_requant if dgrad else ops.conv2d_fprop_requant
-    kw = dict(relu=relu) if not dgrad else {}
+    kw = dict(relu=relu) if not dgrad else dict(relu_mask=relu_mask)
     try:
         y, shift, _ = call(x, w, stride, padding, f32_epilogue=F32_EPILOGUE, target_bits=BITWIDTH, method=method,
                            div_mode=DIV_MODE, bw_mode=BW_MODE, exp_a=exp_a, exp_b=exp_b, exp_out=exp_out, **kw)
@@ -357,6 +357,7 @@ class TiConv2d(UpdateWeight):
         self.stride = stride
         self.padding = padding
         self.fuse_relu = False
+        self.relu_below = False
 
     def forward(self, input, rand=None):
         self.act, self.act_in_exp = input
@@ -382,8 +383,11 @@ class TiConv2d(UpdateWeight):
         self.err_exp = self.err_exp_in
         if not self.first_layer:
             # data gradient with the weights as they were in the forward pass
+            # relu_below: the ReLU in front of this layer (possibly with a max-pool in between) leaves its backward
+            # pass to this layer, whose input is that ReLU's (pooled) output
+            mask = self.act.contiguous() if self.relu_below else None
             fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
-                                        False, self.err_exp_in, self._wexp())
+                                        False, self.err_exp_in, self._wexp(), relu_mask=mask)
             if fused is not None:
                 err_out, _, new_exp = fused
             else:
@@ -391,6 +395,8 @@ class TiConv2d(UpdateWeight):
                 dx = ops.conv2d_dgrad(err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
                 err_out, _, new_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
                                                exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
+                if mask is not None:
+                    err_out = ops.relu_bwd(mask, err_out)
             self.err_exp = new_exp
         K, R, S, C = self.weight.shape
         if self._wgrad_update_fused(err_in, grad_rand):
@@ -476,6 +482,7 @@ class TiReLU(Module):
     def __init__(self):
         super().__init__()
         self.fused = False
+        self.bwd_folded = False
 
     def forward(self, input):
         self.act_in = input
@@ -485,6 +492,8 @@ class TiReLU(Module):
         return ops.relu_fwd(act_in.contiguous()), exp_in
 
     def backward(self, input):
+        if self.bwd_folded:      # the convolution above this layer masked its data gradient already
+            return input
         err_in, err_exp = input
         act, _ = self.act_in
         return ops.relu_bwd(act.contiguous(), err_in.contiguous()), err_exp

@@ -232,6 +232,12 @@ def test_conv_dgrad_requant(dev, case):
             y, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), 1, 1, method=method, prepared_filter=prepared)
             assert int(sync.cpu()[1]) == 0
             assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
+        # ReLU backward of the layer below folded in: zero where the mask is not positive, range from the unmasked sums
+        mask = ri8(g, N, Q, Q, C)
+        mask[0, 0, 0, :4] = torch.tensor([0, -128, 1, 127], dtype=torch.int8)
+        y, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), 1, 1, method=method, relu_mask=mask.to(dev))
+        assert torch.equal(y.cpu(), torch.where(mask > 0, ref, torch.zeros_like(ref)))
+        assert int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
 
 
 @pytest.mark.parametrize("case", [(4, 32, 16, 32), (8, 16, 128, 64), (6, 8, 80, 144), (64, 8, 64, 256), (16, 16, 256, 128),
@@ -314,7 +320,7 @@ def test_conv_wgrad(dev, case):
     assert int(am.cpu()) == po.absmax(ref)
 
 
-GEMM_CASES = [(16, 16, 16), (128, 128, 64), (100, 10, 512), (7, 5, 3), (130, 70, 100), (128, 1024, 1024), (33, 12, 8192)]
+GEMM_CASES = [(128, 10, 8192), (16, 16, 16), (128, 128, 64), (100, 10, 512), (7, 5, 3), (130, 70, 100), (128, 1024, 1024), (33, 12, 8192)]
 
 
 @pytest.mark.parametrize("mnk", GEMM_CASES)
