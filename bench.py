@@ -89,9 +89,14 @@ class ConvTriple:
         for i, L in enumerate(self.layers):
             c, k, hw = L["c"], L["k"], L["hw"]
             am = self.absmax[3 * i: 3 * i + 3]
-            w16 = F.pad(L["w"], (0, 16 - c % 16)).contiguous() if c % 16 else L["w"]
-            # forward + activation requantisation
-            wp = ops.conv_filter_prepare(w16, BATCH, hw, hw)
+            if L.get("wp") is None or not c % 16:
+                L["w16"] = F.pad(L["w"], (0, 16 - c % 16)).contiguous() if c % 16 else L["w"]
+            w16 = L["w16"]        # with a maintained filter copy only its shape is used
+            # forward + activation requantisation; the kernel-ready forward filter copy is made once and from then
+            # on maintained by the weight update below
+            wp = L.get("wp")
+            if wp is None:
+                wp = L["wp"] = ops.conv_filter_prepare(w16, BATCH, hw, hw)
             if record:
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                 e0.record()
@@ -127,8 +132,9 @@ class ConvTriple:
             so, sn = L["sync_w"]
             if sn:
                 ops.conv2d_wgrad_update(L["x16"], L["err"], L["w"], 1, 1, f32_epilogue=(i > 0), mu=5, method="psto",
-                                        sync=self.sync[so:so + sn], workspace=self.ws)
+                                        sync=self.sync[so:so + sn], workspace=self.ws, prepared_filter=L["wp"])
             else:
+                L["wp"] = None
                 dw = ops.conv2d_wgrad(L["x16"], L["err"], 3, 3, 1, 1, f32_epilogue=(i > 0), absmax=am[2:3], workspace=self.ws)
                 if c % 16:
                     dw = dw[..., :c].contiguous()     # zero-padded input channels give zero gradient columns

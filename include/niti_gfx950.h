@@ -169,6 +169,9 @@ int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int 
  * act: [N,H,W,C] int8 (C may include zero channel padding); err: [N,H,W,K] int8; w: [K,3,3,w_channels] int8,
  * updated in place, w_channels <= C (gradient columns beyond w_channels are padding and are dropped).
  * g8_out (optional): rounded gradient, laid out like w.  dw_out (optional): int32 gradient [K,3,3,C].
+ * w_prepared (optional): the copy niti_conv2d_i8_filter_prepare(.., dgrad = 0) made of the filter [K,3,3,C] (w
+ * zero-padded to C channels); the updated weights are written into it as well, so the next forward pass can run
+ * with NITI_CONV_FILTER_PREPARED without a new copy.
  * sync: as for niti_conv2d_i8_fprop_requant (zero on entry; word 0 = max |dw|, word 1 = wait timed out).
  * workspace: niti_conv2d_i8_wgrad_workspace bytes.  flags: NITI_EPI_F32_ROUNDTRIP.
  */
@@ -176,7 +179,7 @@ size_t niti_conv2d_i8_wgrad_update_sync_words(int N, int H, int W, int C, int K,
 int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int W, int C,
                                 int K, int R, int S, int stride, int pad, unsigned flags, int mu, int method, int div_mode,
                                 int bw_mode, uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* dw_out,
-                                int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                int8_t* w_prepared, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
                                 void* workspace, size_t workspace_bytes, void* stream);
 
 /*

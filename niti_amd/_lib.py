@@ -39,7 +39,7 @@ SIGNATURES = {
     "niti_conv2d_i8_wgrad": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _vp, _vp, _sz, _vp]),
     "niti_conv2d_i8_wgrad_update_sync_words": (_sz, [_i] * 9),
     "niti_conv2d_i8_wgrad_update": (_i, [_vp, _vp, _vp] + [_i] * 10 + [_u, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp,
-                                         _vp, _sz, _vp]),
+                                         _vp, _vp, _sz, _vp]),
     "niti_gemm_i8_workspace": (_sz, [_i] * 5),
     "niti_gemm_i8": (_i, [_i, _i, _vp, _vp, _vp, _i, _i, _i, _u, _vp, _vp, _sz, _vp]),
     "niti_absmax_i32": (_i, [_vp, _i64, _vp, _vp]),

@@ -333,8 +333,9 @@ extern "C" size_t niti_conv2d_i8_wgrad_update_sync_words(int N, int H, int W, in
 extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int W,
                                            int C, int K, int R, int S, int stride, int pad, unsigned flags, int mu, int method,
                                            int div_mode, int bw_mode, uint32_t* sync, size_t sync_words, int8_t* g8_out,
-                                           int32_t* dw_out, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b,
-                                           int32_t* exp_out, void* workspace, size_t workspace_bytes, void* stream) {
+                                           int32_t* dw_out, int8_t* w_prepared, int32_t* shift_out, const int32_t* exp_a,
+                                           const int32_t* exp_b, int32_t* exp_out, void* workspace, size_t workspace_bytes,
+                                           void* stream) {
   clear_error();
   int st = check_conv_dims("conv_wgrad_update", N, H, W, C, K, R, S, stride, pad);
   if (st != NITI_OK) return st;
@@ -356,9 +357,11 @@ extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err,
     return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: act, err and dw_out must be 16-byte aligned");
   if (w_channels == C && (reinterpret_cast<uintptr_t>(w) % 4 != 0 || (g8_out != nullptr && reinterpret_cast<uintptr_t>(g8_out) % 4 != 0)))
     return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: w and g8_out must be 4-byte aligned");
+  if (w_prepared != nullptr && (filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 0) != 2 || reinterpret_cast<uintptr_t>(w_prepared) % 4 != 0))
+    return fail(NITI_ERR_UNSUPPORTED, "conv_wgrad_update: w_prepared needs a shape whose forward pass uses a kernel-ready filter copy, 4-byte aligned");
   RequantSpec rq{mu, method, div_mode == NITI_DIV_TRUNC, bw_mode, 0u, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out, nullptr};
   return launch_wgrad3x3_update(act, err, w, w_channels, N, H, C, K, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, sync, rq, g8_out,
-                                dw_out, workspace, static_cast<hipStream_t>(stream));
+                                dw_out, w_prepared, workspace, static_cast<hipStream_t>(stream));
 }
 
 extern "C" size_t niti_gemm_i8_workspace(int trans_a, int trans_b, int m, int n, int k) {

@@ -279,6 +279,7 @@ struct FinishArgs {
   int8_t* w;           // [K][9][Cw], updated in place
   int8_t* g8;          // optional rounded gradient, laid out like w
   int32_t* dw;         // optional int32 gradient [K][9][C]
+  int8_t* wprep;       // optional: the halo convolution kernel's forward copy of the [K][9][C] filter, kept in step with w
   uint32_t* sync;      // word 0: max |sum| (output); word 1: wait gave up; words kFinishSlot0..: slots, zero on entry
   int roundtrip, target_bits, method, trunc, bw_mode;
   long long spin_limit;
@@ -378,9 +379,10 @@ __global__ __launch_bounds__(256) void wgrad_finish_kernel(const FinishArgs a) {
         if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
         else r[e] = wrap_to_i8(s[e]);
       }
+      uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
       if (same_layout) {
         const uint32_t wold = reinterpret_cast<const uint32_t*>(a.w)[col];
-        uint32_t wnew = 0, gp = 0;
+        uint32_t gp = 0;
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * e)) & 0xFFu));
@@ -397,10 +399,23 @@ __global__ __launch_bounds__(256) void wgrad_finish_kernel(const FinishArgs a) {
         for (int e = 0; e < 4; ++e) {
           if (c0 + e < a.Cw) {
             const long long wi = row * a.Cw + c0 + e;
-            a.w[wi] = static_cast<int8_t>(clip127(static_cast<int>(a.w[wi]) - r[e]));
+            const int wn = clip127(static_cast<int>(a.w[wi]) - r[e]);
+            a.w[wi] = static_cast<int8_t>(wn);
+            wnew |= (static_cast<uint32_t>(wn) & 0xFFu) << (8 * e);
             if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
           }
         }
+      }
+      if (a.wprep != nullptr) {
+        // [64-channel group][32-channel slice][tap][64 rows][32 bytes], 16-byte halves swapped where (row >> 3) is odd
+        const long long e0 = col * 4;
+        const long long rt = e0 / a.C;                  // k * 9 + tap
+        const int c0 = static_cast<int>(e0 - rt * a.C);
+        const int k = static_cast<int>(rt / 9), tap = static_cast<int>(rt - static_cast<long long>(k) * 9);
+        const int row = k & 63, cs = c0 >> 5;
+        const int half = ((c0 >> 4) & 1) ^ ((row >> 3) & 1);
+        const long long dst = ((((static_cast<long long>(k >> 6) * ((a.C + 31) >> 5) + cs) * 9 + tap) * 64 + row) << 5) + half * 16 + (c0 & 15);
+        *reinterpret_cast<uint32_t*>(a.wprep + dst) = wnew;
       }
     }
   }
@@ -509,8 +524,8 @@ int wgrad3x3_finish_blocks(int C, int K) {
 size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0 + (blocks + 15) / 16 * 16); }
 
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
-                           bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, void* workspace,
-                           hipStream_t stream) {
+                           bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
+                           void* workspace, hipStream_t stream) {
   const int nb = wgrad3x3_finish_blocks(C, K);
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large for the single-pass finish", K, C);
   static int resident = 0;
@@ -536,6 +551,7 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   f.w = w;
   f.g8 = g8;
   f.dw = dw;
+  f.wprep = wprep;
   f.sync = sync;
   f.roundtrip = roundtrip ? 1 : 0;
   f.target_bits = rq.target_bits;

@@ -189,7 +189,7 @@ KEEP_INT32_GRAD = False      # also store layer.grad_int32acc when the weight gr
 _fused_refused = set()       # (dgrad, input shape, filter shape, stride, padding) the device turned out too small for
 
 
-def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None):
+def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None, prepared_filter=None):
     """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
     exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
     single-launch kernel, or more workgroups than the device holds at once."""
@@ -208,7 +208,7 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
     from ._lib import NitiError
     exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
     call = ops.conv2d_dgrad_requant if dgrad else ops.conv2d_fprop_requant
-    kw = dict(relu=relu) if not dgrad else dict(relu_mask=relu_mask)
+    kw = dict(relu=relu, prepared_filter=prepared_filter) if not dgrad else dict(relu_mask=relu_mask)
     try:
         y, shift, _ = call(x, w, stride, padding, f32_epilogue=F32_EPILOGUE, target_bits=BITWIDTH, method=method,
                            div_mode=DIV_MODE, bw_mode=BW_MODE, exp_a=exp_a, exp_b=exp_b, exp_out=exp_out, **kw)
@@ -344,6 +344,7 @@ class UpdateWeight(Module):
         self.grad, self.grad_shift = ops.grad_update(
             g, self.weight, absmax, GRAD_BITWIDTH, method, DIV_MODE, BW_MODE, rand, want_grad=self.keep_grad,
             exp_a=_exp_tensor(self.err_exp, g.device), exp_b=_exp_tensor(self.act_in_exp, g.device), exp_out=self.grad_exp)
+        self._wprep_key = None      # any kernel-ready copy of the old weights is stale now
 
 
 class TiConv2d(UpdateWeight):
@@ -366,7 +367,7 @@ class TiConv2d(UpdateWeight):
         w16 = _pad_channels16(self.weight).contiguous()
         exp_a, exp_b = _exp_tensor(self.act_in_exp, dev), self._wexp()
         fused = _conv_requant_fused(False, self.act16, w16, self.stride, self.padding, ACT_ROUND_METHOD, rand,
-                                    self.fuse_relu, exp_a, exp_b)
+                                    self.fuse_relu, exp_a, exp_b, prepared_filter=self._forward_filter(w16))
         if fused is not None:
             return fused[0], fused[2]
         am = ops.new_scalar_u32(dev)
@@ -413,11 +414,29 @@ class TiConv2d(UpdateWeight):
         if not self.first_layer:
             return err_out, self.err_exp
 
+    def _forward_filter(self, w16):
+        """Kernel-ready copy of the (channel-padded) filter for the forward pass.  Made when the weight tensor was
+        replaced or modified through torch; the fused weight update keeps it in step with its own changes."""
+        key = (self.weight.data_ptr(), self.weight._version, tuple(self.act16.shape))
+        if getattr(self, "_wprep_key", None) != key:
+            N, H, W, _ = self.act16.shape
+            self._wprep = ops.conv_filter_prepare(w16, N, H, W, self.stride, self.padding)
+            self._wprep_key = key
+        return self._wprep
+
     def _wgrad_workspace(self, err_in):
         from . import _lib
         N, H, W, C16 = self.act16.shape
         K, R, S, _ = self.weight.shape
         return ops.scratch(_lib.lib().niti_conv2d_i8_wgrad_workspace(N, H, W, C16, K, R, S, self.padding), err_in.device)
+
+    def _synced_filter(self):
+        """The forward filter copy if it matches the weights as they are now (then the update maintains it)."""
+        key = getattr(self, "_wprep_key", None)
+        if key is None or self._wprep is None or key[:2] != (self.weight.data_ptr(), self.weight._version):
+            self._wprep_key = None
+            return None
+        return self._wprep
 
     def _wgrad_update_fused(self, err_in, grad_rand):
         """Weight gradient, grad_calc and the weight update as one call into the library (no int32 gradient in
@@ -435,7 +454,7 @@ class TiConv2d(UpdateWeight):
             self.act16, err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE and not self.first_layer,
             mu=GRAD_BITWIDTH, method=method, div_mode=DIV_MODE, bw_mode=BW_MODE, want_grad=self.keep_grad,
             want_dw=KEEP_INT32_GRAD, exp_a=_exp_tensor(self.err_exp, dev), exp_b=_exp_tensor(self.act_in_exp, dev),
-            exp_out=self.grad_exp, workspace=self._wgrad_workspace(err_in))
+            exp_out=self.grad_exp, workspace=self._wgrad_workspace(err_in), prepared_filter=self._synced_filter())
         self.grad_int32acc = None if dw is None else (dw if dw.shape[3] == C else dw[..., :C].contiguous())
         return True
 

@@ -271,10 +271,16 @@ def test_conv_wgrad_update(dev, case, div_mode):
         assert int(sh.cpu()) == sh_ref and int(eo.cpu()) == sh_ref - 4
         assert torch.equal(g8.cpu(), g8_ref)
         assert torch.equal(wd.cpu(), w_ref)
-        # without the optional outputs
+        # without the optional outputs, and with a kernel-ready forward filter copy that has to follow the update
         wd2 = w.to(dev).clone()
-        ops.conv2d_wgrad_update(act16.to(dev).contiguous(), err.to(dev), wd2, mu=mu, method=method, div_mode=div_mode)
+        w16 = (F.pad(w, (0, 16 - C % 16)) if C % 16 else w).to(dev).contiguous()
+        wp = ops.conv_filter_prepare(w16, N, Q, Q)
+        ops.conv2d_wgrad_update(act16.to(dev).contiguous(), err.to(dev), wd2, mu=mu, method=method, div_mode=div_mode,
+                                prepared_filter=wp)
         assert torch.equal(wd2.cpu(), w_ref)
+        if wp is not None:
+            w16_ref = (F.pad(w_ref, (0, 16 - C % 16)) if C % 16 else w_ref).to(dev).contiguous()
+            assert torch.equal(wp.cpu(), ops.conv_filter_prepare(w16_ref, N, Q, Q).cpu())
 
 
 def test_conv_requant_rejects_what_it_does_not_cover(dev):
