@@ -150,20 +150,34 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
   const int wk = wave & 3;         // 32-output-channel quarter of the tile
   const int wc = wave >> 2;        // 32-input-channel half of the tile
   int a_base[2];     // [o]: error tile byte offset of this lane's 8-byte row, reduction step 0
-  int b_base[2][3];  // [o][s]: halo tile byte offset, reduction step 0, filter row 0
+  // Activation fragments: a lane holds 16 consecutive pixels (bytes) of one channel.  The three taps of a filter
+  // row read windows that start 0, 1 and 2 slots into the halo row, so only the window of the first tap is read
+  // from LDS, together with the 8 slots that follow it, and the other two are byte shifts of that sequence
+  // (v_alignbyte).  With 8-pixel image rows the two halves of a fragment lie in different rows and each half
+  // gets its own following slots.
+  constexpr int NB = Q >= 16 ? 3 : 4;
+  int b_base[NB];    // halo tile byte offsets of this lane's 8-byte rows, reduction step 0, filter row 0
 #pragma unroll
   for (int o = 0; o < 2; ++o) {
     const int lpix = 16 * lk + 8 * o + (j >> 1);  // pixel inside the 32-pixel step
-    {
-      const int cb = wk * 32 + gg * 16 + 8 * (j & 1);
-      a_base[o] = lpix * 128 + ((((cb >> 4) ^ ((lpix >> 1) & 7)) << 4) | (cb & 15));
-    }
-    const int lrow = lpix / Q, pw = lpix % Q;
+    const int cb = wk * 32 + gg * 16 + 8 * (j & 1);
+    a_base[o] = lpix * 128 + ((((cb >> 4) ^ ((lpix >> 1) & 7)) << 4) | (cb & 15));
+  }
+  {
     const int cb = wc * 32 + gg * 16 + 8 * (j & 1);
-#pragma unroll
-    for (int s = 0; s < 3; ++s) {
-      const int w = pw + s;
-      b_base[o][s] = G::ERR_BYTES + (lrow * G::RP + w) * 64 + ((((cb >> 4) ^ ((w >> 2) & 3)) << 4) | (cb & 15));
+    auto slot_addr = [&](int lrow, int w) {
+      return G::ERR_BYTES + (lrow * G::RP + w) * 64 + ((((cb >> 4) ^ ((w >> 2) & 3)) << 4) | (cb & 15));
+    };
+    const int p0 = 16 * lk + (j >> 1), p1 = p0 + 8;   // pixels of the two halves inside the 32-pixel step
+    if (Q >= 16) {
+      b_base[0] = slot_addr(p0 / Q, p0 % Q);
+      b_base[1] = slot_addr(p1 / Q, p1 % Q);
+      b_base[2] = slot_addr(p0 / Q, p0 % Q + 16);
+    } else {
+      b_base[0] = slot_addr(p0 / Q, p0 % Q);
+      b_base[1] = slot_addr(p0 / Q, p0 % Q + 8);
+      b_base[2] = slot_addr(p1 / Q, p1 % Q);
+      b_base[NB - 1] = slot_addr(p1 / Q, p1 % Q + 8);
     }
   }
 
@@ -192,20 +206,26 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
       const v2i_t ahi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
           (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[1] + ks * 4096));
       const v4i af = v4i{alo[0], alo[1], ahi[0], ahi[1]};
-      v4i bf[9];
 #pragma unroll
-      for (int r = 0; r < 3; ++r)
+      for (int r = 0; r < 3; ++r) {
+        const int roff = (hrow0 + r) * G::RP * 64;
+        v2i_t rd[NB];
 #pragma unroll
-        for (int s = 0; s < 3; ++s) {
-          const int roff = (hrow0 + r) * G::RP * 64;
-          const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-              (__attribute__((address_space(3))) v2i_t*)(sbase + b_base[0][s] + roff));
-          const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-              (__attribute__((address_space(3))) v2i_t*)(sbase + b_base[1][s] + roff));
-          bf[r * 3 + s] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        for (int q = 0; q < NB; ++q)
+          rd[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(sbase + b_base[q] + roff));
+        // the byte sequences the two 8-pixel halves are cut from: [d0 d1 d2] and [e0 e1 e2] (dwords)
+        const int d0 = rd[0][0], d1 = rd[0][1];
+        const int d2 = Q >= 16 ? rd[1][0] : rd[1][0];
+        const int e0 = Q >= 16 ? rd[1][0] : rd[2][0], e1 = Q >= 16 ? rd[1][1] : rd[2][1];
+        const int e2 = rd[NB - 1][0];
+        acc[r * 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{d0, d1, e0, e1}, acc[r * 3], 0, 0, 0);
+#pragma unroll
+        for (int s = 1; s < 3; ++s) {
+          const v4i bf = {static_cast<int>(__builtin_amdgcn_alignbyte(d1, d0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(d2, d1, s)),
+                          static_cast<int>(__builtin_amdgcn_alignbyte(e1, e0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(e2, e1, s))};
+          acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[r * 3 + s], 0, 0, 0);
         }
-#pragma unroll
-      for (int t = 0; t < 9; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf[t], acc[t], 0, 0, 0);
+      }
     }
   }
 
