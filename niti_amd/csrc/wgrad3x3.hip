@@ -245,6 +245,205 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
   }
 }
 
+// ---- the same computation with half the partial-sum traffic ------------------------------------------------
+// The kernel above leaves 128 x 64 x 9 partial sums (295 KB) per workgroup in memory; with about one workgroup
+// per compute unit that is almost 60 MB per launch, written and read again, whatever the layer - more time than
+// the matrix work.  Here a workgroup owns 128 x 32 x 9 sums: its 8 wavefronts are 4 output-channel quarters x 2
+// pixel halves, the two halves are added through LDS at the end, and 147 KB per workgroup go to memory.  The
+// error tile keeps its full 128-byte rows; the activation tile narrows to 32-byte slots (no swizzle needed: 8
+// pixels x 16 channels read by 16 lanes cover 32 distinct banks, the other 16 lanes the other 32).  A stage is
+// 256 output pixels.
+template <int Q, int BR, int NI>
+struct NGeom {
+  static constexpr int RP = Q + 2;
+  static constexpr int HR = BR + 2;
+  static constexpr int SLOTS = NI * HR * RP;
+  static constexpr int ACT_INSTR = (SLOTS + 31) / 32;       // an instruction fills 32 slots of 32 bytes
+  static constexpr int ACT_BYTES = ACT_INSTR * 1024;
+  static constexpr int ACT_LOADS = (ACT_INSTR + 7) / 8;
+  static constexpr int ERR_BYTES = 256 * 128;               // 32 instructions of 8 pixels x 128 bytes
+  static constexpr int STAGE_BYTES = ERR_BYTES + ACT_BYTES;
+  static constexpr int STAGES = 3;
+  static constexpr int NL = 4 + ACT_LOADS;                  // loads per wavefront per stage
+  static constexpr int REDUCE_BYTES = 4 * 9 * 16 * 64 * 4;  // four wavefronts park their accumulators
+  static constexpr int LDS_BYTES = (STAGES * STAGE_BYTES > REDUCE_BYTES ? STAGES * STAGE_BYTES : REDUCE_BYTES) + 1024;
+  static constexpr int HALF_ROWS = Q == 8 ? 2 * HR : 128 / Q;  // halo rows between the two pixel halves of a stage
+  static_assert(BR * NI * Q == 256, "a stage is 256 output pixels");
+  static_assert(NI == 1 || BR == Q, "several images per stage only as whole images");
+  static_assert(LDS_BYTES <= 160 * 1024, "stages must fit in LDS");
+};
+
+template <int Q, int BR, int NI>
+__global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs a) {
+  using G = NGeom<Q, BR, NI>;
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+  int8_t* const dump = smem + G::LDS_BYTES - 1024;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int k0 = blockIdx.x * 128;
+  const int c0 = blockIdx.y * 32;
+  const int band_begin = blockIdx.z * a.bands_per_split;   // bands of 256 pixels here
+  const int band_end = min(band_begin + a.bands_per_split, a.bands);
+  const int nb = band_end - band_begin;
+
+  const __amdgpu_buffer_rsrc_t ract = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.act), 0, a.act_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rerr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.err), 0, a.err_bytes, 0x00020000);
+
+  // ---- staging.  Error tile: an instruction fills 8 pixels x 128 bytes; lane -> (pixel lane/8, piece lane%8)
+  int err_off[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int pix = (wave + 8 * i) * 8 + (lane >> 3);
+    const int piece = (lane & 7) ^ ((pix >> 1) & 7);
+    const int ch = k0 + piece * 16;
+    err_off[i] = ch < a.K ? pix * a.K + ch : kOob;
+  }
+  // Activation tile: NI images x HR rows x RP slots x 32 bytes, slots in a row; lane -> (slot lane/2, half lane%2)
+  int act_off[G::ACT_LOADS];   // relative to image n0, row p0 = 0
+  int act_hrow[G::ACT_LOADS];  // halo row, image index above bit 10
+#pragma unroll
+  for (int i = 0; i < G::ACT_LOADS; ++i) {
+    const int slot = (wave + 8 * i) * 32 + (lane >> 1);
+    const int row = slot / G::RP, col = slot - row * G::RP;
+    const int ni = row / G::HR, h = row - ni * G::HR;
+    const int ch = c0 + (lane & 1) * 16;
+    const int iw = col - 1;
+    int off = kOob;
+    if (slot < G::SLOTS && iw >= 0 && iw < Q && ch < a.C) off = ((ni * Q + (h - 1)) * Q + iw) * a.C + ch;
+    act_off[i] = off;
+    act_hrow[i] = h + ni * 1024;
+  }
+  auto issue = [&](int band, int st) {
+    int8_t* base = smem + st * G::STAGE_BYTES;
+    const int pixbase = band * 256;
+    const int n0 = pixbase / (Q * Q);
+    const int p0 = (pixbase - n0 * (Q * Q)) / Q;
+    const int eb = pixbase * a.K;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int off = err_off[i] == kOob ? kOob : eb + err_off[i];
+      int8_t* dst = base + (wave + 8 * i) * 1024;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rerr, NITI_LDS(dst), 16, off, 0, 0, 0);
+    }
+    const int ab = (n0 * Q + p0) * Q * a.C;
+#pragma unroll
+    for (int i = 0; i < G::ACT_LOADS; ++i) {
+      const int idx = wave + 8 * i;
+      const int ih = p0 + (act_hrow[i] & 1023) - 1;
+      const bool ok = act_off[i] != kOob && ih >= 0 && ih < Q && n0 + (act_hrow[i] >> 10) < a.N;
+      const int off = ok ? ab + act_off[i] : kOob;
+      int8_t* dst = idx < G::ACT_INSTR ? base + G::ERR_BYTES + idx * 1024 : dump;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(ract, NITI_LDS(dst), 16, off, 0, 0, 0);
+    }
+  };
+
+  // ---- fragment addressing (transposing LDS reads, see the kernel above)
+  const int j = lane & 15;
+  const int gg = (lane >> 4) & 1;
+  const int lk = lane >> 5;
+  const int wk = wave & 3;    // 32-output-channel quarter of the tile
+  const int ph = wave >> 2;   // 128-pixel half of a stage
+  int a_base[2];
+  constexpr int NB = Q >= 16 ? 3 : 4;
+  int b_base[NB];
+#pragma unroll
+  for (int o = 0; o < 2; ++o) {
+    const int lpix = 16 * lk + 8 * o + (j >> 1);
+    const int cb = wk * 32 + gg * 16 + 8 * (j & 1);
+    a_base[o] = (ph * 128 + lpix) * 128 + ((((cb >> 4) ^ ((lpix >> 1) & 7)) << 4) | (cb & 15));
+  }
+  {
+    const int cb = gg * 16 + 8 * (j & 1);
+    auto slot_addr = [&](int lrow, int w) { return G::ERR_BYTES + ((ph * G::HALF_ROWS + lrow) * G::RP + w) * 32 + cb; };
+    const int p0 = 16 * lk + (j >> 1), p1 = p0 + 8;
+    if (Q >= 16) {
+      b_base[0] = slot_addr(p0 / Q, p0 % Q);
+      b_base[1] = slot_addr(p1 / Q, p1 % Q);
+      b_base[2] = slot_addr(p0 / Q, p0 % Q + 16);
+    } else {
+      b_base[0] = slot_addr(p0 / Q, p0 % Q);
+      b_base[1] = slot_addr(p0 / Q, p0 % Q + 8);
+      b_base[2] = slot_addr(p1 / Q, p1 % Q);
+      b_base[NB - 1] = slot_addr(p1 / Q, p1 % Q + 8);
+    }
+  }
+
+  v16i acc[9];
+#pragma unroll
+  for (int t = 0; t < 9; ++t)
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[t][e] = 0;
+
+#pragma unroll
+  for (int s = 0; s < G::STAGES - 1; ++s)
+    if (s < nb) issue(band_begin + s, s);
+
+  for (int it = 0; it < nb; ++it) {
+    if (it + G::STAGES - 2 < nb) wg_wait_vmcnt<(G::STAGES - 2) * G::NL>();
+    else wg_wait_vmcnt<0>();
+    wg_sync();
+    if (it + G::STAGES - 1 < nb) issue(band_begin + it + G::STAGES - 1, (it + G::STAGES - 1) % G::STAGES);
+    const int8_t* sbase = smem + (it % G::STAGES) * G::STAGE_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      const int prow = ks * 32 / Q;                         // first output row of this step inside the pixel half
+      const int hrow0 = (prow / BR) * G::HR + (prow % BR);  // its halo row for filter row 0
+      const v2i_t alo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[0] + ks * 4096));
+      const v2i_t ahi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
+          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[1] + ks * 4096));
+      const v4i af = v4i{alo[0], alo[1], ahi[0], ahi[1]};
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+        const int roff = (hrow0 + r) * G::RP * 32;
+        v2i_t rd[NB];
+#pragma unroll
+        for (int q = 0; q < NB; ++q)
+          rd[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(sbase + b_base[q] + roff));
+        const int d0 = rd[0][0], d1 = rd[0][1], d2 = rd[1][0];
+        const int e0 = Q >= 16 ? rd[1][0] : rd[2][0], e1 = Q >= 16 ? rd[1][1] : rd[2][1];
+        const int e2 = rd[NB - 1][0];
+        acc[r * 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{d0, d1, e0, e1}, acc[r * 3], 0, 0, 0);
+#pragma unroll
+        for (int s = 1; s < 3; ++s) {
+          const v4i bf = {static_cast<int>(__builtin_amdgcn_alignbyte(d1, d0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(d2, d1, s)),
+                          static_cast<int>(__builtin_amdgcn_alignbyte(e1, e0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(e2, e1, s))};
+          acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[r * 3 + s], 0, 0, 0);
+        }
+      }
+    }
+  }
+
+  // ---- add the two pixel halves: half 1 -> LDS -> half 0 -> memory.  Slot layout [value][lane].
+  __syncthreads();  // all tiles consumed, no load in flight (the last stage was waited for with vmcnt(0))
+  int32_t* const park = reinterpret_cast<int32_t*>(smem) + wk * (9 * 16 * 64) + lane;
+  if (ph == 1) {
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+#pragma unroll
+      for (int e = 0; e < 16; ++e) park[(t * 16 + e) * 64] = acc[t][e];
+  }
+  __syncthreads();
+  if (ph == 0) {
+    // partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+(lane&31)]
+    int32_t* out = a.partial + static_cast<long long>(blockIdx.z) * a.slice_stride;
+    const int c = c0 + (lane & 31);
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int k = k0 + wk * 32 + g * 8 + lk * 4 + e;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+          const int v = acc[t][4 * g + e] + park[(t * 16 + 4 * g + e) * 64];
+          if (c < a.C && k < a.K) out[(static_cast<long long>(k) * 9 + t) * a.C + c] = v;
+        }
+      }
+  }
+}
+
 // dw[e] = sum_z partial[z][e]; optional fp32 round trip; max |dw| folded into *absmax.
 // A workgroup owns 64 int4 columns; its 4 wavefronts each add every 4th slice, then combine in LDS.
 __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const int32_t* __restrict__ partial, int32_t* __restrict__ dw,
@@ -448,20 +647,48 @@ long long slice_stride_for(int C, int K) {
   return (n + 1023) / 1024 * 1024 + 1088;
 }
 
+// The narrow-tile arrangement needs whole stages of 256 pixels.  NITI_WGRAD_NARROW=0/1 pins the choice (tests).
+bool use_narrow_arrangement(int N, int Q) {
+  const bool fits = (static_cast<long long>(N) * Q * Q) % 256 == 0;
+  const char* e = getenv("NITI_WGRAD_NARROW");
+  if (e != nullptr) return e[0] == '1' && fits;
+  return fits;
+}
+
 int pick_splits(int N, int Q, int C, int K) {
-  const int bands = N * Q * Q / 128;
-  const int tiles = ((K + 127) / 128) * ((C + 63) / 64);
-  static int target = -1;
-  if (target < 0) {
-    const char* e = getenv("NITI_WGRAD_BLOCKS");
-    target = e ? atoi(e) : 192;  // fewer, longer workgroups: less partial-sum traffic per MFMA
-    if (target < 1) target = 192;
+  const char* e = getenv("NITI_WGRAD_BLOCKS");
+  int target = e != nullptr ? atoi(e) : 0;
+  int bands, tiles;
+  if (use_narrow_arrangement(N, Q)) {
+    bands = N * Q * Q / 256;
+    tiles = ((K + 127) / 128) * ((C + 31) / 32);
+    if (target < 1) target = 224;
+  } else {
+    bands = N * Q * Q / 128;
+    tiles = ((K + 127) / 128) * ((C + 63) / 64);
+    if (target < 1) target = 192;  // fewer, longer workgroups: less partial-sum traffic per MFMA
   }
   int splits = (target + tiles - 1) / tiles;
   if (splits > bands) splits = bands;
   if (splits < 1) splits = 1;
   const int per = (bands + splits - 1) / splits;
   return (bands + per - 1) / per;
+}
+
+template <int Q, int BR, int NI>
+int launch_narrow_geom(const WgradArgs& a, int splits, hipStream_t stream) {
+  using G = NGeom<Q, BR, NI>;
+  constexpr size_t lds = G::LDS_BYTES;
+  auto k = wgrad3x3_narrow_kernel<Q, BR, NI>;
+  static bool attr_set = false;
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return fail(NITI_ERR_LAUNCH, "wgrad: cannot reserve %zu bytes of LDS", lds);
+    attr_set = true;
+  }
+  dim3 grid((a.K + 127) / 128, (a.C + 31) / 32, splits);
+  hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, a);
+  return check_launch("wgrad3x3_narrow");
 }
 
 template <int Q, int BR, int NI>
@@ -508,11 +735,17 @@ static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N,
   a.N = N;
   a.C = C;
   a.K = K;
-  a.bands = N * H * H / 128;
+  const bool narrow = use_narrow_arrangement(N, H);
+  a.bands = N * H * H / (narrow ? 256 : 128);
   splits = pick_splits(N, H, C, K);
   a.bands_per_split = (a.bands + splits - 1) / splits;
   a.act_bytes = static_cast<long long>(N) * H * H * C;
   a.err_bytes = static_cast<long long>(N) * H * H * K;
+  if (narrow) {
+    if (H == 32) return launch_narrow_geom<32, 8, 1>(a, splits, stream);
+    if (H == 16) return launch_narrow_geom<16, 16, 1>(a, splits, stream);
+    return launch_narrow_geom<8, 8, 4>(a, splits, stream);
+  }
   if (H == 32) return launch_geom<32, 4, 1>(a, splits, stream);
   if (H == 16) return launch_geom<16, 8, 1>(a, splits, stream);
   return launch_geom<8, 8, 2>(a, splits, stream);

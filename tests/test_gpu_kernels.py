@@ -240,6 +240,36 @@ def test_conv_dgrad_requant(dev, case):
         assert int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
 
 
+@pytest.fixture(params=["0", "1"])
+def wgrad_arrangement(request):
+    """Pin the native 3x3 weight-gradient kernel to its 128 x 64 tiles (0) or its 128 x 32 tiles with two pixel halves (1)."""
+    import os
+    old = os.environ.get("NITI_WGRAD_NARROW")
+    os.environ["NITI_WGRAD_NARROW"] = request.param
+    yield request.param
+    if old is None:
+        os.environ.pop("NITI_WGRAD_NARROW", None)
+    else:
+        os.environ["NITI_WGRAD_NARROW"] = old
+
+
+@pytest.mark.parametrize("case", [(4, 8, 16, 16), (8, 8, 80, 144), (1, 16, 64, 64), (5, 16, 48, 272), (1, 32, 32, 16), (3, 32, 16, 80),
+                                  (20, 8, 96, 32), (4, 16, 256, 64), (64, 8, 64, 256)])
+def test_conv_wgrad_arrangements(dev, case, wgrad_arrangement):
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_wgrad_arrangements", case, wgrad_arrangement)
+    g = torch.Generator().manual_seed(980 + C + K)
+    act, err = ri8(g, N, Q, Q, C), ri8(g, N, Q, Q, K)
+    ref = co.conv_wgrad(act, err, 3, 3, 1, 1)
+    am = ops.new_scalar_u32(dev)
+    dw = ops.conv2d_wgrad(act.to(dev), err.to(dev), 3, 3, 1, 1, absmax=am)
+    assert torch.equal(dw.cpu(), ref)
+    assert int(am.cpu()) == po.absmax(ref)
+
+
 @pytest.mark.parametrize("case", [(4, 32, 16, 32), (8, 16, 128, 64), (6, 8, 80, 144), (64, 8, 64, 256), (16, 16, 256, 128),
                                   (2, 8, 16, 16), (4, 8, 3, 16), (8, 32, 3, 128), (32, 8, 512, 512)])
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
