@@ -662,7 +662,7 @@ int pick_splits(int N, int Q, int C, int K) {
   if (use_narrow_arrangement(N, Q)) {
     bands = N * Q * Q / 256;
     tiles = ((K + 127) / 128) * ((C + 31) / 32);
-    if (target < 1) target = 224;
+    if (target < 1) target = 256;
   } else {
     bands = N * Q * Q / 128;
     tiles = ((K + 127) / 128) * ((C + 63) / 64);
