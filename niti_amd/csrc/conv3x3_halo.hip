@@ -93,7 +93,9 @@ struct HGeom {
   static constexpr int ACT_BYTES = ACT_INSTR * 1024;
   static constexpr int ACT_LOADS = (ACT_INSTR + 7) / 8;    // per wavefront per slice
   static constexpr int NWF = KT / 64;                      // 32-channel tiles per wavefront
-  static constexpr int W_BYTES = 3 * KT * 32;              // one filter stage: the three taps of a filter row
+  static constexpr int RPS = KT == 64 ? 3 : 1;             // filter rows per stage: the narrow tile takes a whole slice
+  static constexpr int W_BYTES = RPS * 3 * KT * 32;        // one filter stage: RPS filter rows of three taps
+  static constexpr int W_INSTR = W_BYTES / 1024;
   static constexpr int WSTAGES = 3;
   static constexpr int TILE_BYTES = 2 * ACT_BYTES + WSTAGES * W_BYTES;
   static constexpr int LDS_BYTES = TILE_BYTES + 1024;      // + dump slot / reduction words
@@ -148,30 +150,36 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, NITI_LDS(dst), 16, off, 0, 0, 0);
     }
   };
-  // ---- filter staging.  The copy is [64-channel group][slice][tap][64 rows][32 bytes], so the three taps of a
-  // filter row of one group are 6 KB in a row = 6 load instructions.  KT == 128: 12 instructions, wavefront w
-  // issues number w and, if w < 4, number 8 + w.  KT == 64: wavefronts 0-5 issue one each.  The number of loads
-  // therefore differs between wavefronts but never inside one (a lane-dependent condition around a load would
-  // let the compiler split it into two instructions and break the vmcnt bookkeeping below).
+  // ---- filter staging.  The copy is [64-channel group][slice][tap][64 rows][32 bytes]: the three taps of a
+  // filter row of one group are 6 KB in a row, the nine taps of a slice 18 KB.  A stage is W_INSTR load
+  // instructions of 1 KB (KT == 128: one filter row of two groups, 12; KT == 64: a whole slice, 18); wavefront w
+  // issues numbers w, w + 8, w + 16 as far as they exist.  The number of loads therefore differs between
+  // wavefronts but never inside one (a lane-dependent condition around a load would let the compiler split it
+  // into two instructions and break the vmcnt bookkeeping below).
   // A group beyond the last one (K not a multiple of 128) re-reads the last group instead of reading out of
   // range: its sums are never stored.
   const int ngroups = (a.K + 63) / 64;
-  const int wl = KT == 128 ? (wave < 4 ? 2 : 1) : (wave < 6 ? 1 : 0);   // filter loads of this wavefront per stage
+  const int wl = (G::W_INSTR - wave + 7) / 8;   // filter loads of this wavefront per stage
   auto w_src = [&](int q) {  // instruction q of a stage -> byte offset in the copy for slice 0, filter row 0
     const int g = min(KT == 128 ? kt * 2 + q / 6 : kt, ngroups - 1);
-    return g * a.cslices * (9 * 2048) + (q % 6) * 1024 + lane * 16;
+    return g * a.cslices * (9 * 2048) + (KT == 128 ? q % 6 : q) * 1024 + lane * 16;
   };
-  const int wsrc_a = w_src(wave), wsrc_b = w_src(wave + 8);
+  const int wsrc_a = w_src(wave), wsrc_b = w_src(wave + 8), wsrc_c = w_src(wave + 16);
   auto issue_w = [&](int cs, int r, int st) {
     const int rel = (cs * 9 + r * 3) * 2048;
-    if (KT == 128 || wave < 6) {
+    {
       int8_t* dst = w_buf + st * G::W_BYTES + wave * 1024;
       const int off = wsrc_a + rel;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
     }
-    if (KT == 128 && wave < 4) {
+    if (wave + 8 < G::W_INSTR) {
       int8_t* dst = w_buf + st * G::W_BYTES + (wave + 8) * 1024;
       const int off = wsrc_b + rel;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
+    }
+    if (wave + 16 < G::W_INSTR) {
+      int8_t* dst = w_buf + st * G::W_BYTES + (wave + 16) * 1024;
+      const int off = wsrc_c + rel;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
     }
   };
@@ -207,64 +215,87 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
-  // ---- pipeline.  Stage t = 3 * slice + filter row.  Per-wavefront load order: act(0), W(0), W(1); inside
-  // stage t after its barrier: W(t+2), then - in the first stage of a slice - act(next slice).  Stage t needs
-  // W(t) (issued in stage t-2) and, in the first stage of a slice, that slice's activations (issued three
-  // stages earlier, so older than W(t)).  Younger than W(t) are W(t+1) and the activation loads issued in
-  // stage t-2 or t-1.
-  const int nst = a.cslices * 3;
-  issue_act(0, 0);
-  issue_w(0, 0, 0);
-  issue_w(0, 1, 1);
-  for (int ci = 0; ci < a.cslices; ++ci) {
-    const int8_t* sa = act_buf + (ci & 1) * G::ACT_BYTES;
-    const bool more = ci + 1 < a.cslices;
+  // one filter row: 12 (6) MFMAs from the activation tile sa and the three taps at sw
+  auto filter_row = [&](const int8_t* sa, const int8_t* sw, int r) {
+    const int roff = r * G::RP * 32;
+    // pixels under the centre column of this filter row; the fragment layout is lane -> (pixel lane % 32,
+    // 16 channels lane / 32), so the pixel to the left is one lane down and the one to the right one lane up
+    v4i pc[2];
 #pragma unroll
-    for (int r = 0; r < 3; ++r) {
-      const int t = ci * 3 + r;
-      int young = t + 1 < nst ? wl : 0;
-      if (r >= 1 && more) young += G::ACT_LOADS;   // issued in the first stage of this slice, after W(t) went out
-      hc_wait_vmcnt_dyn(young);
-      hc_sync();
-      if (t + 2 < nst) {
-        const int c2 = r == 0 ? ci : ci + 1, r2 = r == 0 ? 2 : r - 1;
-        issue_w(c2, r2, (t + 2) % G::WSTAGES);
+    for (int j = 0; j < 2; ++j) pc[j] = *reinterpret_cast<const v4i*>(sa + ((p_addr[j] + roff) ^ ((r & 1) << 4)));
+    v4i wf[3][NWF];
+#pragma unroll
+    for (int s = 0; s < 3; ++s)
+#pragma unroll
+      for (int i = 0; i < NWF; ++i) wf[s][i] = *reinterpret_cast<const v4i*>(sw + w_addr[i] + ((s + 1) % 3) * 2048);
+    // order: centre tap (needs no shifting) first, then right, then left; wf[0] = tap s=1, wf[1] = s=2, wf[2] = s=0
+#pragma unroll
+    for (int i = 0; i < NWF; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
+    v4i ps[2];
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
+#pragma unroll
+    for (int i = 0; i < NWF; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
+#pragma unroll
+    for (int i = 0; i < NWF; ++i)
+#pragma unroll
+      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
+  };
+
+  if constexpr (G::RPS == 1) {
+    // ---- pipeline, one filter row per stage.  Stage t = 3 * slice + filter row.  Per-wavefront load order: act(0),
+    // W(0), W(1); inside stage t after its barrier: W(t+2), then - in the first stage of a slice - act(next slice).
+    // Stage t needs W(t) (issued in stage t-2) and, in the first stage of a slice, that slice's activations
+    // (issued three stages earlier, so older than W(t)).  Younger than W(t) are W(t+1) and the activation loads
+    // issued in stage t-2 or t-1.
+    const int nst = a.cslices * 3;
+    issue_act(0, 0);
+    issue_w(0, 0, 0);
+    issue_w(0, 1, 1);
+    for (int ci = 0; ci < a.cslices; ++ci) {
+      const int8_t* sa = act_buf + (ci & 1) * G::ACT_BYTES;
+      const bool more = ci + 1 < a.cslices;
+#pragma unroll
+      for (int r = 0; r < 3; ++r) {
+        const int t = ci * 3 + r;
+        int young = t + 1 < nst ? wl : 0;
+        if (r >= 1 && more) young += G::ACT_LOADS;   // issued in the first stage of this slice, after W(t) went out
+        hc_wait_vmcnt_dyn(young);
+        hc_sync();
+        if (t + 2 < nst) {
+          const int c2 = r == 0 ? ci : ci + 1, r2 = r == 0 ? 2 : r - 1;
+          issue_w(c2, r2, (t + 2) % G::WSTAGES);
+        }
+        if (r == 0 && more) issue_act(ci + 1, (ci + 1) & 1);
+        filter_row(sa, w_buf + (t % G::WSTAGES) * G::W_BYTES, r);
       }
-      if (r == 0 && more) issue_act(ci + 1, (ci + 1) & 1);
-      const int8_t* sw = w_buf + (t % G::WSTAGES) * G::W_BYTES;
-      const int roff = r * G::RP * 32;
-      // pixels under the centre column of this filter row; the fragment layout is lane -> (pixel lane % 32,
-      // 16 channels lane / 32), so the pixel to the left is one lane down and the one to the right one lane up
-      v4i pc[2];
+    }
+  } else {
+    // ---- pipeline, one slice per stage (a barrier every 18 MFMAs instead of every 6).  Per-wavefront load order:
+    // act(0), W(0), W(1); inside stage ci after its barrier: act(ci+1), then W(ci+2).  Stage ci needs W(ci) and
+    // act(ci); the only loads younger than both are those of W(ci+1).
+    issue_act(0, 0);
+    issue_w(0, 0, 0);
+    if (a.cslices > 1) issue_w(1, 0, 1);
+    for (int ci = 0; ci < a.cslices; ++ci) {
+      const int8_t* sa = act_buf + (ci & 1) * G::ACT_BYTES;
+      hc_wait_vmcnt_dyn(ci + 1 < a.cslices ? wl : 0);
+      hc_sync();
+      if (ci + 1 < a.cslices) issue_act(ci + 1, (ci + 1) & 1);
+      if (ci + 2 < a.cslices) issue_w(ci + 2, 0, (ci + 2) % G::WSTAGES);
+      const int8_t* sw = w_buf + (ci % G::WSTAGES) * G::W_BYTES;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) pc[j] = *reinterpret_cast<const v4i*>(sa + ((p_addr[j] + roff) ^ ((r & 1) << 4)));
-      v4i wf[3][NWF];
-#pragma unroll
-      for (int s = 0; s < 3; ++s)
-#pragma unroll
-        for (int i = 0; i < NWF; ++i) wf[s][i] = *reinterpret_cast<const v4i*>(sw + w_addr[i] + ((s + 1) % 3) * 2048);
-      // order: centre tap (needs no shifting) first, then left, then right; wf[0] = tap s=1, wf[1] = s=2, wf[2] = s=0
-#pragma unroll
-      for (int i = 0; i < NWF; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
-      v4i ps[2];
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
-#pragma unroll
-      for (int i = 0; i < NWF; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
-#pragma unroll
-      for (int j = 0; j < 2; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
-#pragma unroll
-      for (int i = 0; i < NWF; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
+      for (int r = 0; r < 3; ++r) filter_row(sa, sw + r * 3 * 2048, r);
     }
   }
 
