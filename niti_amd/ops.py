@@ -206,6 +206,7 @@ class _SyncArena:
     def __init__(self):
         self.buf = {}
         self.off = {}
+        self.taken = {}
 
     def reset(self, device):
         key = str(device)
@@ -214,6 +215,7 @@ class _SyncArena:
         else:
             self.buf[key].zero_()
         self.off[key] = 0
+        self.taken[key] = []
 
     def take(self, words, device):
         key = str(device)
@@ -222,7 +224,19 @@ class _SyncArena:
             self.off[key] = None
             return None
         self.off[key] = off + (words + 31) // 32 * 32
+        self.taken.setdefault(key, []).append(off)
         return self.buf[key][off:off + words]
+
+    def timed_out(self, device) -> bool:
+        """True if a single-launch kernel that used a slice since the last reset flagged that its grid-wide wait ran
+        into the time limit (its output is then invalid).  Copies the flags to the host: for the end of a step or an
+        epoch, not for the inner loop."""
+        key = str(device)
+        offs = self.taken.get(key)
+        if not offs:
+            return False
+        idx = torch.tensor([o + 1 for o in offs], dtype=torch.long, device=self.buf[key].device)
+        return bool(self.buf[key][idx].ne(0).any().item())
 
 
 sync_arena = _SyncArena()

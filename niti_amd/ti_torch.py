@@ -449,7 +449,20 @@ class TiConv2d(UpdateWeight):
         if ops.wgrad_update_sync_words(N, H, W, C16, K, R, S, self.stride, self.padding) == 0:
             return False
         dev = err_in.device
+        key = ("wgrad_update", tuple(self.act16.shape), tuple(self.weight.shape))
+        if key in _fused_refused:
+            return False
+        from ._lib import NitiError
         self.grad_exp = torch.empty(1, dtype=torch.int32, device=dev)
+        try:
+            return self._wgrad_update_call(err_in, method, dev, C)
+        except NitiError as e:
+            if "do not fit" not in str(e):
+                raise
+            _fused_refused.add(key)     # a device too small for the finishing kernel's grid: separate steps from now on
+            return False
+
+    def _wgrad_update_call(self, err_in, method, dev, C):
         self.grad, dw, self.grad_shift, _ = ops.conv2d_wgrad_update(
             self.act16, err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE and not self.first_layer,
             mu=GRAD_BITWIDTH, method=method, div_mode=DIV_MODE, bw_mode=BW_MODE, want_grad=self.keep_grad,

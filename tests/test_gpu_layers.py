@@ -171,6 +171,8 @@ def test_training_step(tt, name, cfg_list, N):
     yo, eo = onet.forward_int8(x, 0)
     y, e = net.forward_int8(x.to(dev), 0)
     assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+    from niti_amd import ops
+    assert not ops.sync_arena.timed_out(dev), "a single-launch kernel gave up waiting for its workgroups"
 
 
 def test_ti_loss_matches_oracle_on_typical_logits(tt):
