@@ -113,14 +113,15 @@ class ConvTriple:
                 ops.requant(acc, am[0:1], 7, "round", exp_a=self.exp0, exp_b=self.exp0, exp_out=torch.empty_like(self.exp0))
             # data gradient + error requantisation
             if i > 0:
-                wt = ops.conv_filter_prepare(L["w"], BATCH, hw, hw, dgrad=True)
+                # the single-launch kernel reads the forward pass's filter copy; the two-pass path makes its own
+                so, sn = L["sync_d"]
+                wt = None if sn else ops.conv_filter_prepare(L["w"], BATCH, hw, hw, dgrad=True)
                 if record:
                     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
                     e0.record()
-                so, sn = L["sync_d"]
                 if sn:
                     ops.conv2d_dgrad_requant(L["err"], L["w"], 1, 1, f32_epilogue=True, sync=self.sync[so:so + sn],
-                                             prepared_filter=wt)
+                                             forward_filter=wp)
                 else:
                     dx = ops.conv2d_dgrad(L["err"], L["w"], 1, 1, f32_epilogue=True, absmax=am[1:2], prepared_filter=wt)
                 if record:

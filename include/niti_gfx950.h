@@ -36,6 +36,9 @@ enum {
                                      (pytorch/cutlass-extension/cutlassconv_kernel.cu:78-85) */
 #define NITI_CONV_FILTER_PREPARED 2u /* fprop / dgrad: `w` already is the kernel-ready filter copy written
                                         by niti_conv2d_i8_filter_prepare for the same shape; no workspace */
+#define NITI_CONV_FILTER_FORWARD_COPY 4u /* data gradient only, with NITI_CONV_FILTER_PREPARED: `w` is the
+                                            copy that niti_conv2d_i8_filter_prepare(.., dgrad = 0) made of
+                                            the same filter (the one the forward pass reads) */
 /* requant flags */
 #define NITI_RQ_RELU 1u /* clamp the int8 result at 0 (TiReLU.forward, ti_torch.py:272-279) */
 

@@ -13,6 +13,7 @@ SO_PATH = os.path.join(_HERE, "libniti_gfx950.so")
 OK = 0
 EPI_F32_ROUNDTRIP = 1
 CONV_FILTER_PREPARED = 2
+CONV_FILTER_FORWARD_COPY = 4
 RQ_RELU = 1
 ROUND = {"round": 0, "sto": 1, "psto": 2}
 DIV = {"floor": 0, "trunc": 1}

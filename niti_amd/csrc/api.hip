@@ -98,6 +98,19 @@ static int filter_copy_kind(int N, int H, int W, int C, int K, int R, int S, int
   return (!halo_off() && conv3x3_halo_supported(N, P, Q, K, C, R, S, 1, R - 1 - pad)) ? 3 : 1;
 }
 
+// NITI_CONV_FILTER_FORWARD_COPY is for a data gradient whose forward pass and whose own launch both run the halo
+// kernel (the copy of kind 2 is then read in place of the copy of kind 3); anything else is a caller error
+static int check_forward_copy_flag(const char* who, int dgrad, unsigned flags, int N, int H, int W, int C, int K, int R, int S,
+                                   int stride, int pad) {
+  if (!(flags & NITI_CONV_FILTER_FORWARD_COPY)) return NITI_OK;
+  if (!dgrad) return fail(NITI_ERR_INVALID_ARG, "%s: NITI_CONV_FILTER_FORWARD_COPY is a data-gradient flag", who);
+  if (!(flags & NITI_CONV_FILTER_PREPARED))
+    return fail(NITI_ERR_INVALID_ARG, "%s: NITI_CONV_FILTER_FORWARD_COPY needs NITI_CONV_FILTER_PREPARED", who);
+  if (filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 0) != 2 || filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 1) != 3)
+    return fail(NITI_ERR_UNSUPPORTED, "%s: the forward filter copy serves the data gradient only where both run the 3x3 kernel", who);
+  return NITI_OK;
+}
+
 extern "C" size_t niti_conv2d_i8_filter_workspace(int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                                                   int dgrad) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0) return 0;
@@ -136,6 +149,8 @@ extern "C" int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y
   if (x == nullptr || w == nullptr || y == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: null pointer");
   if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: pointers must be 16-byte aligned");
   if (C % 16 != 0) return fail(NITI_ERR_UNSUPPORTED, "conv: C=%d must be a multiple of 16", C);
+  st = check_forward_copy_flag("conv_fprop", 0, flags, N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int kind = filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 0);
   if (kind == 2) {
@@ -168,6 +183,8 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
     return fail(NITI_ERR_UNSUPPORTED, "conv_dgrad: needs stride 1, square filter, pad <= R-1 (stride=%d R=%d S=%d pad=%d)", stride, R, S, pad);
   if (K % 16 != 0) return fail(NITI_ERR_UNSUPPORTED, "conv_dgrad: K=%d must be a multiple of 16", K);
   if (!aligned16(err) || !aligned16(dx)) return fail(NITI_ERR_INVALID_ARG, "conv_dgrad: pointers must be 16-byte aligned");
+  st = check_forward_copy_flag("conv_dgrad", 1, flags, N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
   hipStream_t s = static_cast<hipStream_t>(stream);
   const int kind = filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 1);
   const int8_t* wt = w;
@@ -234,6 +251,8 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
   if (bw_mode != NITI_BW_INT && bw_mode != NITI_BW_F32) return fail(NITI_ERR_INVALID_ARG, "%s: bw_mode=%d", who, bw_mode);
   const int nb = fused_blocks(N, H, W, C, K, R, S, stride, pad, dgrad);
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "%s: shape not covered by the single-launch path; use the two-pass path", who);
+  st = check_forward_copy_flag(who, dgrad, flags, N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
   if (sync_words < conv3x3_halo_sync_words(nb))
     return fail(NITI_ERR_WORKSPACE, "%s: needs %zu zeroed sync words, got %zu", who, conv3x3_halo_sync_words(nb), sync_words);
   hipStream_t s = static_cast<hipStream_t>(stream);

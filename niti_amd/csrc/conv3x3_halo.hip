@@ -60,6 +60,7 @@ struct HaloArgs {
   uint32_t* absmax;
   int N, C, K;
   int cslices;        // ceil(C / 32)
+  int src_cslices;    // kWT only: 32-channel slices of the forward filter copy read as the data gradient's filter
   long long x_bytes, wp_bytes, y_bytes;
   unsigned flags;
   // requantising variant only
@@ -104,7 +105,10 @@ struct HGeom {
   static_assert(NI == 1 || BR == Q, "several images per workgroup only as whole images");
 };
 
-template <int Q, int BR, int NI, int KT, bool kFused>
+// kWT: the filter operand is the FORWARD copy of the filter of the convolution whose data gradient this launch
+// computes (input channels of this launch = that filter's output channels and vice versa, taps flipped); its
+// 32 x 32 byte blocks are staged as they are and transposed by ds_read_b64_tr_b8 when the fragments are read.
+template <int Q, int BR, int NI, int KT, bool kFused, bool kWT>
 __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) {
   using G = HGeom<Q, BR, NI, KT>;
   constexpr int NWF = G::NWF;
@@ -161,12 +165,19 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const int ngroups = (a.K + 63) / 64;
   const int wl = (G::W_INSTR - wave + 7) / 8;   // filter loads of this wavefront per stage
   auto w_src = [&](int q) {  // instruction q of a stage -> byte offset in the copy for slice 0, filter row 0
+    if (kWT) {
+      // KB q of a stage holds tap q / (KT/32) of the stage and 32-channel slice q % (KT/32) of this tile's output
+      // channels: rows = 32 reduction channels (half a 64-row group of the forward copy), 32 bytes = 32 outputs
+      const int cs = min(kt * (KT / 32) + q % (KT / 32), a.src_cslices - 1);
+      return (cs * 9 + 8 - q / (KT / 32)) * 2048 + lane * 16;
+    }
     const int g = min(KT == 128 ? kt * 2 + q / 6 : kt, ngroups - 1);
     return g * a.cslices * (9 * 2048) + (KT == 128 ? q % 6 : q) * 1024 + lane * 16;
   };
   const int wsrc_a = w_src(wave), wsrc_b = w_src(wave + 8), wsrc_c = w_src(wave + 16);
   auto issue_w = [&](int cs, int r, int st) {
-    const int rel = (cs * 9 + r * 3) * 2048;
+    // kWT: reduction slice cs = rows (cs & 1) * 32.. of group cs >> 1; a later filter row is an earlier forward tap
+    const int rel = kWT ? (cs >> 1) * a.src_cslices * (9 * 2048) + (cs & 1) * 1024 - r * 3 * 2048 : (cs * 9 + r * 3) * 2048;
     {
       int8_t* dst = w_buf + st * G::W_BYTES + wave * 1024;
       const int off = wsrc_a + rel;
@@ -188,12 +199,24 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const int wp_ = wave & 3;   // 64-pixel group
   const int wc = wave >> 2;   // channel group of KT/2
   const int lr = lane & 31, lk = lane >> 5;
-  int w_addr[NWF];            // this lane's filter row inside a stage, tap 0
+  constexpr int TAPB = kWT ? (KT / 32) * 1024 : 2048;   // bytes between consecutive taps inside a stage
+  int w_addr[NWF][kWT ? 2 : 1];   // this lane's filter row(s) inside a stage, tap 0
 #pragma unroll
   for (int i = 0; i < NWF; ++i) {
-    // row inside the 64-channel group the stage holds at (KT == 128 ? wc * 6144 : 0)
-    const int grow = KT == 128 ? i * 32 + lr : wc * 32 + lr;
-    w_addr[i] = (KT == 128 ? wc * 6144 : 0) + grow * 32 + ((lk ^ ((grow >> 3) & 1)) << 4);
+    if (kWT) {
+      // block (tap, slice j) = [32 reduction rows][32 output bytes]; two transposing reads of 8 rows x 16 outputs
+      const int j16 = lane & 15, gg = (lane >> 4) & 1;
+      const int jslice = KT == 128 ? wc * 2 + i : wc;
+#pragma unroll
+      for (int o = 0; o < (kWT ? 2 : 1); ++o) {
+        const int krow = 16 * lk + 8 * o + (j16 >> 1);
+        w_addr[i][o] = jslice * 1024 + krow * 32 + ((gg ^ ((krow >> 3) & 1)) << 4) + 8 * (j16 & 1);
+      }
+    } else {
+      // row inside the 64-channel group the stage holds at (KT == 128 ? wc * 6144 : 0)
+      const int grow = KT == 128 ? i * 32 + lr : wc * 32 + lr;
+      w_addr[i][0] = (KT == 128 ? wc * 6144 : 0) + grow * 32 + ((lk ^ ((grow >> 3) & 1)) << 4);
+    }
   }
   int p_addr[2];              // [pixel tile]: halo slot of this lane's pixel, filter row 0
 #pragma unroll
@@ -227,7 +250,17 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
     for (int s = 0; s < 3; ++s)
 #pragma unroll
-      for (int i = 0; i < NWF; ++i) wf[s][i] = *reinterpret_cast<const v4i*>(sw + w_addr[i] + ((s + 1) % 3) * 2048);
+      for (int i = 0; i < NWF; ++i) {
+        const int8_t* src = sw + ((s + 1) % 3) * TAPB;
+        if (kWT) {
+          typedef int v2i_t __attribute__((ext_vector_type(2)));
+          const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(src + w_addr[i][0]));
+          const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(src + w_addr[i][kWT ? 1 : 0]));
+          wf[s][i] = v4i{lo[0], lo[1], hi[0], hi[1]};
+        } else {
+          wf[s][i] = *reinterpret_cast<const v4i*>(src + w_addr[i][0]);
+        }
+      }
     // order: centre tap (needs no shifting) first, then right, then left; wf[0] = tap s=1, wf[1] = s=2, wf[2] = s=0
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
@@ -295,7 +328,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (ci + 2 < a.cslices) issue_w(ci + 2, 0, (ci + 2) % G::WSTAGES);
       const int8_t* sw = w_buf + (ci % G::WSTAGES) * G::W_BYTES;
 #pragma unroll
-      for (int r = 0; r < 3; ++r) filter_row(sa, sw + r * 3 * 2048, r);
+      for (int r = 0; r < 3; ++r) filter_row(sa, sw + r * 3 * TAPB, r);
     }
   }
 
@@ -504,14 +537,14 @@ int halo_ktile(long long pix, int K) {
   return (b128 < 2LL * cus && K > 64) ? 64 : 128;
 }
 
-template <int Q, int BR, int NI, int KT, bool kFused>
+template <int Q, int BR, int NI, int KT, bool kFused, bool kWT>
 int launch_halo(const HaloArgs& a, hipStream_t stream) {
   using G = HGeom<Q, BR, NI, KT>;
   constexpr size_t lds = G::LDS_BYTES;
   static_assert(8 * 32 * (32 * 4 + 16) <= G::TILE_BYTES, "int32 patches must stay clear of the reduction words");
   static_assert(8 * 64 * (G::NWF * 32 + 16) <= G::TILE_BYTES, "int8 patches must stay clear of the reduction words");
   static_assert(2 * lds <= 160 * 1024, "two workgroups per compute unit");
-  auto k = conv3x3_halo_kernel<Q, BR, NI, KT, kFused>;
+  auto k = conv3x3_halo_kernel<Q, BR, NI, KT, kFused, kWT>;
   static bool attr_set = false;
   static int resident = 0;  // workgroups the device holds at once
   if (!attr_set) {
@@ -534,20 +567,26 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
   return check_launch("conv3x3_halo");
 }
 
-template <bool kFused>
-int launch_halo_any(const HaloArgs& a, int H, hipStream_t stream) {
+template <bool kFused, bool kWT>
+int launch_halo_tiles(const HaloArgs& a, int H, hipStream_t stream) {
   const int ktile = halo_ktile(static_cast<long long>(a.N) * H * H, a.K);
   if (ktile == 128) {
-    if (H == 32) return launch_halo<32, 8, 1, 128, kFused>(a, stream);
-    if (H == 16) return launch_halo<16, 16, 1, 128, kFused>(a, stream);
-    return launch_halo<8, 8, 4, 128, kFused>(a, stream);
+    if (H == 32) return launch_halo<32, 8, 1, 128, kFused, kWT>(a, stream);
+    if (H == 16) return launch_halo<16, 16, 1, 128, kFused, kWT>(a, stream);
+    return launch_halo<8, 8, 4, 128, kFused, kWT>(a, stream);
   }
-  if (H == 32) return launch_halo<32, 8, 1, 64, kFused>(a, stream);
-  if (H == 16) return launch_halo<16, 16, 1, 64, kFused>(a, stream);
-  return launch_halo<8, 8, 4, 64, kFused>(a, stream);
+  if (H == 32) return launch_halo<32, 8, 1, 64, kFused, kWT>(a, stream);
+  if (H == 16) return launch_halo<16, 16, 1, 64, kFused, kWT>(a, stream);
+  return launch_halo<8, 8, 4, 64, kFused, kWT>(a, stream);
+}
+
+template <bool kFused>
+int launch_halo_any(const HaloArgs& a, int H, hipStream_t stream) {
+  return a.src_cslices > 0 ? launch_halo_tiles<kFused, true>(a, H, stream) : launch_halo_tiles<kFused, false>(a, H, stream);
 }
 
 void fill_common(HaloArgs& a, const int8_t* x, const int8_t* wp, int N, int H, int C, int K, unsigned flags) {
+  // NITI_CONV_FILTER_FORWARD_COPY: wp is the forward copy of the [C][3][3][K] filter whose data gradient this is
   a = HaloArgs{};
   a.x = x;
   a.wp = wp;
@@ -556,7 +595,9 @@ void fill_common(HaloArgs& a, const int8_t* x, const int8_t* wp, int N, int H, i
   a.K = K;
   a.cslices = (C + 31) / 32;
   a.x_bytes = static_cast<long long>(N) * H * H * C;
-  a.wp_bytes = static_cast<long long>(conv3x3_halo_filter_bytes(C, K));
+  const bool wt = (flags & NITI_CONV_FILTER_FORWARD_COPY) != 0;
+  a.src_cslices = wt ? (K + 31) / 32 : 0;
+  a.wp_bytes = static_cast<long long>(wt ? conv3x3_halo_filter_bytes(K, C) : conv3x3_halo_filter_bytes(C, K));
   a.flags = flags;
 }
 

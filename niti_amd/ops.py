@@ -79,10 +79,11 @@ def conv2d_fprop(x, w, stride=1, padding=1, f32_epilogue=False, absmax: Optional
     return y
 
 
-def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None, prepared_filter=None):
+def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None, prepared_filter=None, forward_filter=None):
     """err [N,P,Q,K] int8, w [K,R,S,C] int8 -> dx [N,H,W,C] int32 (stride 1).  ``prepared_filter``:
-    the output of conv_filter_prepare(w, N, H, W, stride, padding, dgrad=True)."""
-    _chk_dev(err, w, absmax, prepared_filter)
+    the output of conv_filter_prepare(w, N, H, W, stride, padding, dgrad=True).  ``forward_filter``: the copy the
+    FORWARD pass reads (conv_filter_prepare(.., dgrad=False)), for shapes where both passes run the 3x3 kernel."""
+    _chk_dev(err, w, absmax, prepared_filter, forward_filter)
     N, P, Q, K = err.shape
     K2, R, S, C = w.shape
     if K2 != K:
@@ -91,6 +92,8 @@ def conv2d_dgrad(err, w, stride=1, padding=1, f32_epilogue=False, absmax=None, p
     W = Q - 2 * padding + S - 1
     dx = torch.empty((N, H, W, C), dtype=torch.int32, device=err.device)
     flags = _flags(f32_epilogue)
+    if forward_filter is not None:
+        prepared_filter, flags = forward_filter, flags | L.CONV_FILTER_FORWARD_COPY
     if prepared_filter is not None:
         st = L.lib().niti_conv2d_i8_dgrad(_ptr(err), _ptr(prepared_filter), _ptr(dx), N, H, W, C, K, R, S, stride, padding,
                                           flags | L.CONV_FILTER_PREPARED, _ptr(absmax), None, 0, _stream(err))
@@ -110,8 +113,8 @@ def conv_requant_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1, dgrad=
 
 
 def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epilogue, target_bits, method, div_mode,
-                  bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None):
-    _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask)
+                  bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None, forward_filter=None):
+    _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask, forward_filter)
     if relu_mask is not None and (relu_mask.dtype != torch.int8 or tuple(relu_mask.shape) != tuple(out_shape)):
         raise RuntimeError("%s: relu_mask must be int8 and shaped like the output" % entry)
     if x.dtype != torch.int8 or w.dtype != torch.int8:
@@ -130,6 +133,8 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
     if shift_out is None:
         shift_out = torch.empty(1, dtype=torch.int32, device=x.device)
     flags = _flags(f32_epilogue)
+    if forward_filter is not None:
+        prepared_filter, flags = forward_filter, flags | L.CONV_FILTER_FORWARD_COPY
     if prepared_filter is not None:
         wptr, ws, nbytes, flags = _ptr(prepared_filter), None, 0, flags | L.CONV_FILTER_PREPARED
     else:
@@ -163,10 +168,11 @@ def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_b
 
 def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None, relu_mask=None):
+                         prepared_filter=None, relu_mask=None, forward_filter=None):
     """conv2d_dgrad + requant as one launch: err [N,P,Q,K] int8, w [K,R,S,C] int8 -> ([N,H,W,C] int8, shift, sync).
     ``relu_mask`` (int8 [N,H,W,C]): results whose mask element is not positive are stored as zero, after range
-    and rounding were taken from the unmasked sums (the backward pass of a ReLU in front of the layer)."""
+    and rounding were taken from the unmasked sums (the backward pass of a ReLU in front of the layer).
+    ``forward_filter``: the copy the forward pass reads, in place of ``prepared_filter`` (see conv2d_dgrad)."""
     N, P, Q, K = err.shape
     K2, R, S, C = w.shape
     if K2 != K:
@@ -175,7 +181,7 @@ def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target
     W = Q - 2 * padding + S - 1
     return _conv_requant("niti_conv2d_i8_dgrad_requant", True, err, w, (N, H, W, C), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, False, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter, relu_mask)
+                         prepared_filter, relu_mask, forward_filter)
 
 
 _scratch = {}

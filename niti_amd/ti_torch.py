@@ -189,7 +189,8 @@ KEEP_INT32_GRAD = False      # also store layer.grad_int32acc when the weight gr
 _fused_refused = set()       # (dgrad, input shape, filter shape, stride, padding) the device turned out too small for
 
 
-def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None, prepared_filter=None):
+def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None, prepared_filter=None,
+                        forward_filter=None):
     """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
     exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
     single-launch kernel, or more workgroups than the device holds at once."""
@@ -208,7 +209,7 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
     from ._lib import NitiError
     exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
     call = ops.conv2d_dgrad_requant if dgrad else ops.conv2d_fprop_requant
-    kw = dict(relu=relu, prepared_filter=prepared_filter) if not dgrad else dict(relu_mask=relu_mask)
+    kw = dict(relu=relu, prepared_filter=prepared_filter) if not dgrad else dict(relu_mask=relu_mask, forward_filter=forward_filter)
     try:
         y, shift, _ = call(x, w, stride, padding, f32_epilogue=F32_EPILOGUE, target_bits=BITWIDTH, method=method,
                            div_mode=DIV_MODE, bw_mode=BW_MODE, exp_a=exp_a, exp_b=exp_b, exp_out=exp_out, **kw)
@@ -386,18 +387,15 @@ class TiConv2d(UpdateWeight):
             # data gradient with the weights as they were in the forward pass
             # relu_below: the ReLU in front of this layer (possibly with a max-pool in between) leaves its backward
             # pass to this layer, whose input is that ReLU's (pooled) output
+            from ._lib import NitiError
             mask = self.act.contiguous() if self.relu_below else None
-            fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
-                                        False, self.err_exp_in, self._wexp(), relu_mask=mask)
-            if fused is not None:
-                err_out, _, new_exp = fused
-            else:
-                am = ops.new_scalar_u32(dev)
-                dx = ops.conv2d_dgrad(err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
-                err_out, _, new_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
-                                               exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
-                if mask is not None:
-                    err_out = ops.relu_bwd(mask, err_out)
+            try:
+                err_out, new_exp = self._data_gradient(err_in, rand, mask, self._dgrad_filter())
+            except NitiError as e:
+                if "forward filter copy" not in str(e):
+                    raise
+                self._dgrad_own_copy = True     # this shape's data gradient runs a kernel that needs its own copy
+                err_out, new_exp = self._data_gradient(err_in, rand, mask, None)
             self.err_exp = new_exp
         K, R, S, C = self.weight.shape
         if self._wgrad_update_fused(err_in, grad_rand):
@@ -413,6 +411,29 @@ class TiConv2d(UpdateWeight):
         self.weight_update(amg, grad_rand)
         if not self.first_layer:
             return err_out, self.err_exp
+
+    def _dgrad_filter(self):
+        """The forward pass's kernel-ready filter copy, which the data gradient can read in place of a copy of its
+        own while it matches the weights, or None."""
+        if getattr(self, "_dgrad_own_copy", False) or self.act16.shape[3] != self.weight.shape[3]:
+            return None
+        return self._synced_filter()
+
+    def _data_gradient(self, err_in, rand, mask, forward_filter):
+        """err_calc(conv_dgrad(err_in, weight)) (ti_torch.py:422-427), the ReLU mask applied; -> (int8 error, exponent)."""
+        fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
+                                    False, self.err_exp_in, self._wexp(), relu_mask=mask, forward_filter=forward_filter)
+        if fused is not None:
+            err_out, _, new_exp = fused
+            return err_out, new_exp
+        am = ops.new_scalar_u32(err_in.device)
+        dx = ops.conv2d_dgrad(err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am,
+                              forward_filter=forward_filter)
+        err_out, _, new_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
+                                       exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
+        if mask is not None:
+            err_out = ops.relu_bwd(mask, err_out)
+        return err_out, new_exp
 
     def _forward_filter(self, w16):
         """Kernel-ready copy of the (channel-padded) filter for the forward pass.  Made when the weight tensor was

@@ -149,6 +149,12 @@ def test_conv_halo_tiles(dev, case, halo_tile):
         assert torch.equal(dx.cpu(), dref)
         dx8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev))
         assert int(sync.cpu()[1]) == 0 and torch.equal(dx8.cpu(), d8) and int(sh.cpu()) == dsh
+        # the data gradient reading the copy of the filter that the forward pass uses
+        wf = ops.conv_filter_prepare(w.to(dev), N, Q, Q)
+        dx = ops.conv2d_dgrad(e.to(dev), w.to(dev), 1, 1, forward_filter=wf)
+        assert torch.equal(dx.cpu(), dref)
+        dx8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), forward_filter=wf)
+        assert int(sync.cpu()[1]) == 0 and torch.equal(dx8.cpu(), d8) and int(sh.cpu()) == dsh
 
 
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
@@ -232,6 +238,10 @@ def test_conv_dgrad_requant(dev, case):
             y, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), 1, 1, method=method, prepared_filter=prepared)
             assert int(sync.cpu()[1]) == 0
             assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
+        y, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), 1, 1, method=method,
+                                               forward_filter=ops.conv_filter_prepare(w.to(dev), N, Q, Q))
+        assert int(sync.cpu()[1]) == 0
+        assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
         # ReLU backward of the layer below folded in: zero where the mask is not positive, range from the unmasked sums
         mask = ri8(g, N, Q, Q, C)
         mask[0, 0, 0, :4] = torch.tensor([0, -128, 1, 127], dtype=torch.int8)
@@ -324,6 +334,10 @@ def test_conv_requant_rejects_what_it_does_not_cover(dev):
     w = torch.zeros((16, 3, 3, 16), dtype=torch.int8, device=dev)
     with pytest.raises(NitiError):
         ops.conv2d_fprop_requant(x, w)
+    # the forward filter copy stands in for the data gradient's own only where both passes run the 3x3 kernel
+    e = torch.zeros((3, 7, 9, 32), dtype=torch.int8, device=dev)
+    with pytest.raises(NitiError):
+        ops.conv2d_dgrad(e, torch.zeros((32, 3, 3, 16), dtype=torch.int8, device=dev), forward_filter=torch.zeros(64, dtype=torch.int8, device=dev))
     # a launch that would not be resident at once is refused by the library, not started
     N = 2048                                                          # 2048 workgroups of 256 pixels
     assert ops.conv_requant_sync_words(N, 16, 16, 16, 16) > 0
