@@ -250,6 +250,16 @@ int niti_maxpool_i8_bwd(const int8_t* y, const int8_t* dy, const int8_t* x, int8
                         int ks, int stride, int pad, int ties, void* stream);
 
 /*
+ * Integer cross-entropy gradient, TiLoss.forward (ti_loss.py:5-36), as one launch: out_val [n][classes] int8 logits
+ * with exponent *out_exp (device scalar), target [n] int64 class indices, rand [n][classes] int32 random integers
+ * (the low four bits stand in for the reference's torch.randint(0, 16)) -> grad [n][classes] int8 with exponent 0.
+ * Every float32 operation of the reference's sequence is kept in order (base-2 soft-max for out_exp > -7, the
+ * quadratic 1 + x + x^2/2 form below), the int64 truncating sums included; the last step is StoShift(.., 4).
+ */
+int niti_loss_grad_i8(const int8_t* out_val, const int32_t* out_exp, const int64_t* target, const int32_t* rand,
+                      int8_t* grad, int n, int classes, int div_mode, void* stream);
+
+/*
  * Grouped int8 convolution with float32 output, replaces int8conv_cuda.group_conv
  * (pytorch/int8conv-extension/int8conv.cpp:35-44, int8conv_kernel.cu:248-334):
  * x: [N,H,W,G*Cg] int8, w: [K,R,S,Cg] int8 (K % G == 0, filter k belongs to group k/(K/G)),

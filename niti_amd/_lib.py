@@ -51,6 +51,7 @@ SIGNATURES = {
     "niti_relu_i8_bwd": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "niti_maxpool_i8_fwd": (_i, [_vp, _vp] + [_i] * 7 + [_vp]),
     "niti_maxpool_i8_bwd": (_i, [_vp, _vp, _vp, _vp] + [_i] * 8 + [_vp]),
+    "niti_loss_grad_i8": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "niti_group_conv_i8_f32": (_i, [_vp, _vp, _vp] + [_i] * 12 + [_vp]),
 }
 

@@ -1,0 +1,88 @@
+// NITI's integer cross-entropy gradient (ti_loss.py:5-36) as one launch: one lane per sample.
+//
+// The reference evaluates a base-2 soft-max of the int8 logits in float32 tensor operations, truncates to
+// integers twice on the way and rounds the result to int8 with StoShift(.., 4).  Every float32 operation
+// of that sequence is kept, in the same order and with the same intermediate types (int64 sums of truncated
+// values, float32 products and quotients), so that the result only depends on the device's powf.
+#include "common.h"
+#include "requant_math.h"
+
+namespace niti {
+namespace {
+
+struct LossArgs {
+  const int8_t* out;       // [n][classes] logits
+  const int32_t* out_exp;  // exponent of the logits (device scalar)
+  const int64_t* target;   // [n]
+  const int32_t* rand;     // [n][classes], low four bits used
+  int8_t* grad;            // [n][classes]
+  int n, classes, trunc;
+};
+
+// no fused multiply-add: the reference runs every operation as a kernel of its own
+#pragma clang fp contract(off)
+
+// ti_loss.py:10-24 for one logit: 2^max(s - offset, 0) - 1 with s = v * 47274 / 2^15 * 2^e
+__device__ inline float scaled_logit(int v, float p2, bool up) {
+  const float s = static_cast<float>(static_cast<long long>(v) * 47274) / 32768.0f;
+  return up ? s * p2 : s / p2;
+}
+
+__global__ __launch_bounds__(64) void loss_grad_kernel(const LossArgs a) {
+  const int row = blockIdx.x * 64 + threadIdx.x;
+  if (row >= a.n) return;
+  const int8_t* v = a.out + static_cast<long long>(row) * a.classes;
+  const int e = *a.out_exp;
+  const bool big = e > -7;
+  const bool up = e >= 0;
+  const float p2 = exp2f(static_cast<float>(up ? e : -e));   // exact power of two
+  float off = 0.0f;
+  // small exponents (ti_loss.py:26-30): 2^(1-2e) + v 2^(1-e) + v^2 in 64-bit integers that wrap like the tensor's
+  const int sh2 = 1 - 2 * e, sh1 = 1 - e;
+  const unsigned long long c2 = (!big && sh2 < 64) ? 1ULL << sh2 : 0ULL;
+  auto small_term = [&](int x) {
+    const unsigned long long lin = sh1 < 64 ? static_cast<unsigned long long>(static_cast<long long>(x)) << sh1 : 0ULL;
+    return static_cast<long long>(c2 + lin + static_cast<unsigned long long>(static_cast<long long>(x) * x));
+  };
+  if (big) {
+    float m = scaled_logit(v[0], p2, up);
+    for (int j = 1; j < a.classes; ++j) m = fmaxf(m, scaled_logit(v[j], p2, up));
+    off = m - 10.0f;
+  }
+  auto numer = [&](int j) -> float {   // out_grad before the normalisation, as float32
+    if (!big) return static_cast<float>(small_term(v[j]));
+    const float s = fmaxf(scaled_logit(v[j], p2, up) - off, 0.0f);
+    return powf(2.0f, s) - 1.0f;
+  };
+  long long sum = 0;   // out_grad.sum(1, dtype=int64): truncation of every term (ti_loss.py:31)
+  for (int j = 0; j < a.classes; ++j) sum += big ? static_cast<long long>(numer(j)) : small_term(v[j]);
+  const float fsum = static_cast<float>(sum);
+  long long tsum = 0;  // ti_loss.py:34: int64 sum of the truncated normalised values
+  for (int j = 0; j < a.classes; ++j) tsum += static_cast<long long>(numer(j) * 2048.0f / fsum);
+  const long long t = a.target[row];
+  const bool trunc = a.trunc != 0;
+  for (int j = 0; j < a.classes; ++j) {
+    float g = numer(j) * 2048.0f / fsum;
+    if (j == t) g = g - static_cast<float>(tsum);
+    const int x = static_cast<int>(g);   // .type(torch.int32)
+    const long long idx = static_cast<long long>(row) * a.classes + j;
+    a.grad[idx] = static_cast<int8_t>(round_one<NITI_ROUND_STOCHASTIC>(x, 4, trunc, a.rand[idx] & 15));
+  }
+}
+
+}  // namespace
+}  // namespace niti
+
+using namespace niti;
+
+extern "C" int niti_loss_grad_i8(const int8_t* out_val, const int32_t* out_exp, const int64_t* target, const int32_t* rand,
+                                 int8_t* grad, int n, int classes, int div_mode, void* stream) {
+  clear_error();
+  if (out_val == nullptr || out_exp == nullptr || target == nullptr || rand == nullptr || grad == nullptr)
+    return fail(NITI_ERR_INVALID_ARG, "loss_grad: null pointer");
+  if (n <= 0 || classes <= 0) return fail(NITI_ERR_INVALID_ARG, "loss_grad: n=%d classes=%d", n, classes);
+  if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "loss_grad: div_mode=%d", div_mode);
+  const LossArgs a{out_val, out_exp, target, rand, grad, n, classes, div_mode == NITI_DIV_TRUNC ? 1 : 0};
+  hipLaunchKernelGGL(loss_grad_kernel, dim3((n + 63) / 64), dim3(64), 0, static_cast<hipStream_t>(stream), a);
+  return check_launch("loss_grad");
+}

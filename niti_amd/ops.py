@@ -392,6 +392,24 @@ def relu_bwd(act, dy):
     return dx
 
 
+def loss_grad(out_val, out_exp, target, rand, div_mode="floor"):
+    """TiLoss.forward (ti_loss.py:5-36) as one launch: int8 logits [n, classes] with exponent ``out_exp`` (1-element
+    int32 device tensor), int64 targets [n], int32 random integers [n, classes] -> int8 gradient (exponent 0)."""
+    _chk_dev(out_val, out_exp, target, rand)
+    if out_val.dtype != torch.int8 or out_val.dim() != 2 or not out_val.is_contiguous():
+        raise RuntimeError("loss_grad: contiguous int8 [n, classes] logits expected")
+    if out_exp.dtype != torch.int32 or target.dtype != torch.int64 or rand.dtype != torch.int32:
+        raise RuntimeError("loss_grad: int32 exponent, int64 targets and int32 random integers expected")
+    n, classes = out_val.shape
+    if target.numel() != n or tuple(rand.shape) != (n, classes) or not rand.is_contiguous() or not target.is_contiguous():
+        raise RuntimeError("loss_grad: shape mismatch")
+    grad = torch.empty_like(out_val)
+    st = L.lib().niti_loss_grad_i8(_ptr(out_val), _ptr(out_exp), _ptr(target), _ptr(rand), _ptr(grad), n, classes,
+                                   L.DIV[div_mode], _stream(out_val))
+    L.check(st, "niti_loss_grad_i8")
+    return grad
+
+
 def maxpool_fwd(x, kernel_size=2, stride=2, padding=0):
     _chk_dev(x)
     if x.dtype != torch.int8:

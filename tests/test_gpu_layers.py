@@ -176,23 +176,41 @@ def test_training_step(tt, name, cfg_list, N):
 
 
 def test_ti_loss_matches_oracle_on_typical_logits(tt):
-    """TiLoss runs float32 ops on the device; on these inputs the result equals the CPU evaluation."""
-    from niti_amd.ti_loss import TiLoss
+    """TiLoss is one kernel that keeps the reference's float32 operation sequence; only powf can differ between
+    host and device (one int8 step, rarely), and the integer branch (out_exp <= -7) is exact."""
+    from niti_amd.ti_loss import TiLoss, loss_grad_tensor_ops
     from oracle import niti_oracle as po
     dev = torch.device("cuda:0")
     g = torch.Generator().manual_seed(3000)
-    for e in (-9, -7, -6, -3, 0):
-        _say("ti_loss", e)
-        out = ri8(g, 64, 10)
-        tgt = torch.randint(0, 10, (64,), generator=g)
-        u = torch.randint(0, 16, (64, 10), generator=g, dtype=torch.int32)
-        ref, _ = po.ti_loss(out, e, tgt, u)
-        got, ge = TiLoss()(out.to(dev), e, tgt.to(dev), u.to(dev))
-        assert ge == 0
-        diff = (got.cpu().to(torch.int16) - ref.to(torch.int16)).abs()
-        # float32 pow may differ in the last ulp between host and device: allow one int8 step
-        assert int(diff.max()) <= 1
-        assert float((diff != 0).float().mean()) < 0.01
+    for div_mode in ("floor", "trunc"):
+        tt.DIV_MODE = div_mode
+        for e in (-12, -9, -7, -6, -3, 0, 2):
+            _say("ti_loss", e, div_mode)
+            n = 64 if e != -3 else 257          # more than one workgroup, ragged
+            out = ri8(g, n, 10)
+            tgt = torch.randint(0, 10, (n,), generator=g)
+            u = torch.randint(0, 16, (n, 10), generator=g, dtype=torch.int32)
+            ref, _ = po.ti_loss(out, e, tgt, u, div_mode)
+            got, ge = TiLoss()(out.to(dev), e, tgt.to(dev), u.to(dev))
+            assert ge == 0 and got.dtype == torch.int8 and tuple(got.shape) == (n, 10)
+            diff = (got.cpu().to(torch.int16) - ref.to(torch.int16)).abs()
+            if e <= -7:
+                assert int(diff.max()) == 0
+            assert int(diff.max()) <= 1
+            assert float((diff != 0).float().mean()) < 0.01
+            # the same sequence as device tensor operations
+            alt = loss_grad_tensor_ops(out.to(dev), e, tgt.to(dev), u.to(dev))
+            d2 = (got.to(torch.int16) - alt.to(torch.int16)).abs()
+            assert int(d2.max()) <= 1 and float((d2 != 0).float().mean()) < 0.01
+    tt.DIV_MODE = "floor"
+    # drawing the random integers on the device (no ``rand``): same distribution, values within one rounding step
+    out = ri8(g, 64, 10)
+    tgt = torch.randint(0, 10, (64,), generator=g)
+    lo, _ = po.ti_loss(out, -3, tgt, torch.full((64, 10), 15, dtype=torch.int32))
+    hi, _ = po.ti_loss(out, -3, tgt, torch.zeros((64, 10), dtype=torch.int32))
+    got, _ = TiLoss()(out.to(dev), -3, tgt.to(dev))
+    gc = got.cpu().to(torch.int16)
+    assert bool(((gc >= torch.minimum(lo, hi).to(torch.int16) - 1) & (gc <= torch.maximum(lo, hi).to(torch.int16) + 1)).all())
 
 
 def test_shims_match_reference_conventions():
