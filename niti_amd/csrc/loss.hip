@@ -1,4 +1,4 @@
-// NITI's integer cross-entropy gradient (ti_loss.py:5-36) as one launch: one lane per sample.
+// NITI's integer cross-entropy gradient (ti_loss.py:5-36) as one launch: one wavefront per sample.
 //
 // The reference evaluates a base-2 soft-max of the int8 logits in float32 tensor operations, truncates to
 // integers twice on the way and rounds the result to int8 with StoShift(.., 4).  Every float32 operation
@@ -28,8 +28,21 @@ __device__ inline float scaled_logit(int v, float p2, bool up) {
   return up ? s * p2 : s / p2;
 }
 
-__global__ __launch_bounds__(64) void loss_grad_kernel(const LossArgs a) {
-  const int row = blockIdx.x * 64 + threadIdx.x;
+__device__ inline long long wave_sum_i64(long long v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const int lo = __shfl_xor(static_cast<int>(v & 0xFFFFFFFFLL), off, 64);
+    const int hi = __shfl_xor(static_cast<int>(v >> 32), off, 64);
+    v += (static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo);
+  }
+  return v;
+}
+
+// One wavefront per sample, lanes over the classes.  The per-class terms are functions of the logit alone, so
+// recomputing them in each of the three passes gives the same bits as the reference's stored tensors.
+__global__ __launch_bounds__(256) void loss_grad_kernel(const LossArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.n) return;
   const int8_t* v = a.out + static_cast<long long>(row) * a.classes;
   const int e = *a.out_exp;
@@ -45,8 +58,10 @@ __global__ __launch_bounds__(64) void loss_grad_kernel(const LossArgs a) {
     return static_cast<long long>(c2 + lin + static_cast<unsigned long long>(static_cast<long long>(x) * x));
   };
   if (big) {
-    float m = scaled_logit(v[0], p2, up);
-    for (int j = 1; j < a.classes; ++j) m = fmaxf(m, scaled_logit(v[j], p2, up));
+    float m = -INFINITY;
+    for (int j = lane; j < a.classes; j += 64) m = fmaxf(m, scaled_logit(v[j], p2, up));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
     off = m - 10.0f;
   }
   auto numer = [&](int j) -> float {   // out_grad before the normalisation, as float32
@@ -55,13 +70,14 @@ __global__ __launch_bounds__(64) void loss_grad_kernel(const LossArgs a) {
     return powf(2.0f, s) - 1.0f;
   };
   long long sum = 0;   // out_grad.sum(1, dtype=int64): truncation of every term (ti_loss.py:31)
-  for (int j = 0; j < a.classes; ++j) sum += big ? static_cast<long long>(numer(j)) : small_term(v[j]);
-  const float fsum = static_cast<float>(sum);
+  for (int j = lane; j < a.classes; j += 64) sum += big ? static_cast<long long>(numer(j)) : small_term(v[j]);
+  const float fsum = static_cast<float>(wave_sum_i64(sum));
   long long tsum = 0;  // ti_loss.py:34: int64 sum of the truncated normalised values
-  for (int j = 0; j < a.classes; ++j) tsum += static_cast<long long>(numer(j) * 2048.0f / fsum);
+  for (int j = lane; j < a.classes; j += 64) tsum += static_cast<long long>(numer(j) * 2048.0f / fsum);
+  tsum = wave_sum_i64(tsum);
   const long long t = a.target[row];
   const bool trunc = a.trunc != 0;
-  for (int j = 0; j < a.classes; ++j) {
+  for (int j = lane; j < a.classes; j += 64) {
     float g = numer(j) * 2048.0f / fsum;
     if (j == t) g = g - static_cast<float>(tsum);
     const int x = static_cast<int>(g);   // .type(torch.int32)
@@ -83,6 +99,6 @@ extern "C" int niti_loss_grad_i8(const int8_t* out_val, const int32_t* out_exp, 
   if (n <= 0 || classes <= 0) return fail(NITI_ERR_INVALID_ARG, "loss_grad: n=%d classes=%d", n, classes);
   if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "loss_grad: div_mode=%d", div_mode);
   const LossArgs a{out_val, out_exp, target, rand, grad, n, classes, div_mode == NITI_DIV_TRUNC ? 1 : 0};
-  hipLaunchKernelGGL(loss_grad_kernel, dim3((n + 63) / 64), dim3(64), 0, static_cast<hipStream_t>(stream), a);
+  hipLaunchKernelGGL(loss_grad_kernel, dim3((n + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), a);
   return check_launch("loss_grad");
 }

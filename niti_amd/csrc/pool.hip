@@ -145,6 +145,52 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const PoolArgs a) {
   }
 }
 
+// 0xFF in every byte where a and b agree
+__device__ inline uint32_t equal_bytes(uint32_t a, uint32_t b) {
+  const uint32_t z = a ^ b;
+  const uint32_t nz = (((z & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | z) & 0x80808080u;   // bit 7 of the bytes that differ
+  return ((nz ^ 0x80808080u) >> 7) * 0xFFu;
+}
+
+// The layers' case: 2 x 2 windows, stride 2, no padding, even H and W, C % 16 == 0.  Windows do not overlap, so a
+// lane owns one window x 16 channels: six 16-byte loads, byte-parallel compares, four 16-byte stores.
+template <bool kAll>
+__global__ __launch_bounds__(256) void maxpool2x2_bwd_kernel(const PoolArgs a) {
+  const int CV = a.C >> 4;
+  const int64_t total = static_cast<int64_t>(a.N) * a.P * a.Q * CV;
+  const int64_t gstride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t rowb = static_cast<int64_t>(a.W) * a.C;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < total; i += gstride) {
+    const uint32_t pix = static_cast<uint32_t>(i / CV);           // (n * P + p) * Q + q < 2^31 (checked on the host)
+    const uint32_t cv = static_cast<uint32_t>(i - static_cast<int64_t>(pix) * CV);
+    const uint32_t q = pix % static_cast<uint32_t>(a.Q);
+    const uint32_t np = pix / static_cast<uint32_t>(a.Q);         // n * P + p; input row 2 * np since H = 2 P
+    const int64_t x0 = (static_cast<int64_t>(np) * 2 * a.W + 2 * q) * a.C + cv * 16;
+    const v4i y = *reinterpret_cast<const v4i*>(a.y + i * 16);
+    const v4i d = *reinterpret_cast<const v4i*>(a.dy + i * 16);
+    v4i x[4];
+    x[0] = *reinterpret_cast<const v4i*>(a.x + x0);
+    x[1] = *reinterpret_cast<const v4i*>(a.x + x0 + a.C);
+    x[2] = *reinterpret_cast<const v4i*>(a.x + x0 + rowb);
+    x[3] = *reinterpret_cast<const v4i*>(a.x + x0 + rowb + a.C);
+    v4i o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      uint32_t taken = 0;   // bytes whose gradient an earlier position of the window (scan order) already received
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t eq = equal_bytes(static_cast<uint32_t>(x[k][e]), static_cast<uint32_t>(y[e]));
+        o[k][e] = static_cast<int>(static_cast<uint32_t>(d[e]) & (kAll ? eq : eq & ~taken));
+        taken |= eq;
+      }
+    }
+    *reinterpret_cast<v4i*>(a.out + x0) = o[0];
+    *reinterpret_cast<v4i*>(a.out + x0 + a.C) = o[1];
+    *reinterpret_cast<v4i*>(a.out + x0 + rowb) = o[2];
+    *reinterpret_cast<v4i*>(a.out + x0 + rowb + a.C) = o[3];
+  }
+}
+
 struct GroupConvArgs {
   const int8_t* x;
   const int8_t* w;
@@ -232,6 +278,13 @@ extern "C" int niti_maxpool_i8_bwd(const int8_t* y, const int8_t* dy, const int8
   if (ties != NITI_TIES_FIRST && ties != NITI_TIES_ALL) return fail(NITI_ERR_INVALID_ARG, "maxpool_bwd: ties=%d", ties);
   PoolArgs a{x, y, dy, dx, N, H, W, C, P, Q, ks, stride, pad, ties == NITI_TIES_ALL};
   const bool vec = C % 16 == 0 && aligned16(x) && aligned16(y) && aligned16(dy) && aligned16(dx);
+  if (vec && ks == 2 && stride == 2 && pad == 0 && H % 2 == 0 && W % 2 == 0 && static_cast<int64_t>(N) * P * Q < 0x7fffffffLL) {
+    const int64_t windows = static_cast<int64_t>(N) * P * Q * (C / 16);
+    const dim3 grid(grid_for(windows, 256, 1 << 20));
+    if (ties == NITI_TIES_ALL) hipLaunchKernelGGL(maxpool2x2_bwd_kernel<true>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    else hipLaunchKernelGGL(maxpool2x2_bwd_kernel<false>, grid, dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    return check_launch("maxpool2x2_bwd");
+  }
   const int64_t total = static_cast<int64_t>(N) * H * W * (vec ? C / 16 : C);
   if (vec) hipLaunchKernelGGL(maxpool_bwd_kernel<16>, dim3(grid_for(total, 256)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
   else hipLaunchKernelGGL(maxpool_bwd_kernel<1>, dim3(grid_for(total, 256)), dim3(256), 0, static_cast<hipStream_t>(stream), a);

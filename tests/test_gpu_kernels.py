@@ -477,7 +477,7 @@ def test_relu(dev):
 
 
 POOL_CASES = [(2, 8, 8, 16, 2, 2, 0), (1, 6, 6, 5, 2, 2, 0), (2, 7, 7, 32, 3, 2, 1), (1, 5, 5, 3, 2, 1, 0),
-              (1, 9, 9, 16, 3, 3, 0), (8, 32, 32, 128, 2, 2, 0), (3, 7, 7, 16, 2, 2, 0)]
+              (1, 9, 9, 16, 3, 3, 0), (8, 32, 32, 128, 2, 2, 0), (3, 7, 7, 16, 2, 2, 0), (5, 4, 6, 48, 2, 2, 0), (2, 2, 2, 16, 2, 2, 0)]
 
 
 @pytest.mark.parametrize("case", POOL_CASES)
