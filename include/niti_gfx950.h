@@ -250,6 +250,29 @@ int niti_maxpool_i8_bwd(const int8_t* y, const int8_t* dy, const int8_t* x, int8
                         int ks, int stride, int pad, int ties, void* stream);
 
 /*
+ * TiLinear with at most 16 output features (the classifier), each pass as one launch with its requantisation
+ * folded in (ti_torch.py:241-266); operands as the layer stores them: act [M][F], w [O][F], err [M][O], int8.
+ *   fwd_requant:   out8 [M][O] = act_calc(act * w^T)            (ti_torch.py:245-249)
+ *   dgrad_requant: dx8 [M][F]  = err_calc(err * w)              (ti_torch.py:256-261)
+ *   wgrad_update:  g = grad_calc(err^T * act), w = clip(w - g)  (ti_torch.py:263-265, 16-21); g8_out optional
+ * `which` names the pass for the sync query, which returns 0 for shapes these kernels do not cover (then use
+ * niti_gemm_i8 + niti_requant_i32_i8 / niti_grad_update_i8).  sync: zeroed uint32 words as for the convolutions
+ * (word 0 range out, word 1 time-out flag; the forward pass accumulates its int32 sums in the words from 16 on).
+ * Rounding NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC; shift_out / exp_* as in niti_requant_i32_i8.
+ */
+enum { NITI_FC_FORWARD = 0, NITI_FC_DGRAD = 1, NITI_FC_WGRAD = 2 };
+size_t niti_fc_i8_sync_words(int which, int M, int O, int F);
+int niti_fc_i8_fwd_requant(const int8_t* act, const int8_t* w, int8_t* out8, int M, int O, int F, int target_bits, int method,
+                           int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
+                           const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
+int niti_fc_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int M, int O, int F, int target_bits, int method,
+                             int div_mode, int bw_mode, uint32_t* sync, size_t sync_words, int32_t* shift_out,
+                             const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
+int niti_fc_i8_wgrad_update(const int8_t* err, const int8_t* act, int8_t* w, int M, int O, int F, int mu, int method,
+                            int div_mode, int bw_mode, uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* shift_out,
+                            const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
+
+/*
  * Integer cross-entropy gradient, TiLoss.forward (ti_loss.py:5-36), as one launch: out_val [n][classes] int8 logits
  * with exponent *out_exp (device scalar), target [n] int64 class indices, rand [n][classes] int32 random integers
  * (the low four bits stand in for the reference's torch.randint(0, 16)) -> grad [n][classes] int8 with exponent 0.

@@ -51,6 +51,10 @@ SIGNATURES = {
     "niti_relu_i8_bwd": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "niti_maxpool_i8_fwd": (_i, [_vp, _vp] + [_i] * 7 + [_vp]),
     "niti_maxpool_i8_bwd": (_i, [_vp, _vp, _vp, _vp] + [_i] * 8 + [_vp]),
+    "niti_fc_i8_sync_words": (_sz, [_i] * 4),
+    "niti_fc_i8_fwd_requant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _u, _vp, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "niti_fc_i8_dgrad_requant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp, _vp, _vp]),
+    "niti_fc_i8_wgrad_update": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "niti_loss_grad_i8": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
     "niti_group_conv_i8_f32": (_i, [_vp, _vp, _vp] + [_i] * 12 + [_vp]),
 }

@@ -209,7 +209,7 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
 
 // ---- convolution + requantisation in one launch -------------------------------------------------------
 // wall-clock ticks (100 MHz) a grid-wide wait may last; NITI_SYNC_TIMEOUT_MS overrides the 10 s default
-static long long sync_spin_limit() {
+long long niti::sync_spin_limit() {
   static long long spin_limit = -1;
   if (spin_limit < 0) {
     const char* e = getenv("NITI_SYNC_TIMEOUT_MS");

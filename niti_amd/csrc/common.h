@@ -133,6 +133,8 @@ struct RequantSpec {
   int32_t* exp_out;
   const int8_t* mask;      // conv + requantisation only: optional ReLU-backward mask, laid out like the output
 };
+// wall-clock ticks (100 MHz) a grid-wide wait may last (api.hip)
+long long sync_spin_limit();
 int wgrad3x3_finish_blocks(int C, int K);
 size_t wgrad3x3_sync_words(int blocks);
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,

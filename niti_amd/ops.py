@@ -392,6 +392,87 @@ def relu_bwd(act, dy):
     return dx
 
 
+FC_PASS = {"forward": 0, "dgrad": 1, "wgrad": 2}
+
+
+def fc_sync_words(which, M, O, F) -> int:
+    """uint32 sync words the one-launch TiLinear kernels need for act [M,F], weight [O,F]; 0 when the shape is
+    outside them (more than 16 output features, ...) and the GEMM entry point has to be used."""
+    return int(L.lib().niti_fc_i8_sync_words(FC_PASS[which], M, O, F))
+
+
+def _fc_sync(which, M, O, F, sync, device, who):
+    words = fc_sync_words(which, M, O, F)
+    if words == 0:
+        raise L.NitiError("%s: shape not covered by the few-output-features kernels" % who)
+    if sync is None:
+        sync = sync_arena.take(words, device)
+    if sync is None:
+        sync = torch.zeros(words, dtype=torch.int32, device=device)
+    elif sync.dtype != torch.int32 or sync.numel() < words:
+        raise RuntimeError("%s: sync must be a zeroed int32 tensor of at least %d words" % (who, words))
+    return sync
+
+
+def fc_fwd_requant(act, w, target_bits=7, method="round", div_mode="floor", bw_mode="int", relu=False, sync=None,
+                   shift_out=None, exp_a=None, exp_b=None, exp_out=None):
+    """act_calc(act @ w^T) as one launch: act [M,F] int8, w [O,F] int8 (O <= 16) -> ([M,O] int8, shift, sync)."""
+    _chk_dev(act, w, sync, shift_out, exp_a, exp_b, exp_out)
+    if act.dtype != torch.int8 or w.dtype != torch.int8 or act.dim() != 2 or w.dim() != 2 or act.shape[1] != w.shape[1]:
+        raise RuntimeError("fc_fwd_requant: int8 act [M,F] and w [O,F] expected")
+    M, F = act.shape
+    O = w.shape[0]
+    sync = _fc_sync("forward", M, O, F, sync, act.device, "fc_fwd_requant")
+    out = torch.empty((M, O), dtype=torch.int8, device=act.device)
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=act.device)
+    st = L.lib().niti_fc_i8_fwd_requant(_ptr(act), _ptr(w), _ptr(out), M, O, F, target_bits, L.ROUND[method], L.DIV[div_mode],
+                                        L.BW[bw_mode], L.RQ_RELU if relu else 0, _ptr(sync), sync.numel(), _ptr(shift_out),
+                                        _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _stream(act))
+    L.check(st, "niti_fc_i8_fwd_requant")
+    return out, shift_out, sync
+
+
+def fc_dgrad_requant(err, w, target_bits=7, method="round", div_mode="floor", bw_mode="int", sync=None, shift_out=None,
+                     exp_a=None, exp_b=None, exp_out=None):
+    """err_calc(err @ w) as one launch: err [M,O] int8, w [O,F] int8 (O <= 16) -> ([M,F] int8, shift, sync)."""
+    _chk_dev(err, w, sync, shift_out, exp_a, exp_b, exp_out)
+    if err.dtype != torch.int8 or w.dtype != torch.int8 or err.dim() != 2 or w.dim() != 2 or err.shape[1] != w.shape[0]:
+        raise RuntimeError("fc_dgrad_requant: int8 err [M,O] and w [O,F] expected")
+    M, O = err.shape
+    F = w.shape[1]
+    sync = _fc_sync("dgrad", M, O, F, sync, err.device, "fc_dgrad_requant")
+    dx = torch.empty((M, F), dtype=torch.int8, device=err.device)
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=err.device)
+    st = L.lib().niti_fc_i8_dgrad_requant(_ptr(err), _ptr(w), _ptr(dx), M, O, F, target_bits, L.ROUND[method], L.DIV[div_mode],
+                                          L.BW[bw_mode], _ptr(sync), sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b),
+                                          _ptr(exp_out), _stream(err))
+    L.check(st, "niti_fc_i8_dgrad_requant")
+    return dx, shift_out, sync
+
+
+def fc_wgrad_update(err, act, w, mu=5, method="psto", div_mode="floor", bw_mode="int", sync=None, want_grad=False,
+                    shift_out=None, exp_a=None, exp_b=None, exp_out=None):
+    """g = grad_calc(err^T @ act, mu); w = clip(w - g) in place, as one launch: err [M,O], act [M,F], w [O,F] int8
+    (O <= 16, M <= 512) -> (g as int8 [O,F] if want_grad else None, shift, sync)."""
+    _chk_dev(err, act, w, sync, shift_out, exp_a, exp_b, exp_out)
+    if err.dtype != torch.int8 or act.dtype != torch.int8 or w.dtype != torch.int8 or err.dim() != 2 or act.dim() != 2 \
+            or tuple(w.shape) != (err.shape[1], act.shape[1]) or err.shape[0] != act.shape[0]:
+        raise RuntimeError("fc_wgrad_update: int8 err [M,O], act [M,F] and w [O,F] expected")
+    M, O = err.shape
+    F = act.shape[1]
+    sync = _fc_sync("wgrad", M, O, F, sync, err.device, "fc_wgrad_update")
+    g8 = torch.empty_like(w) if want_grad else None
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=err.device)
+    st = L.lib().niti_fc_i8_wgrad_update(_ptr(err), _ptr(act), _ptr(w), M, O, F, mu, L.ROUND[method], L.DIV[div_mode],
+                                         L.BW[bw_mode], _ptr(sync), sync.numel(), _ptr(g8), _ptr(shift_out), _ptr(exp_a),
+                                         _ptr(exp_b), _ptr(exp_out), _stream(err))
+    L.check(st, "niti_fc_i8_wgrad_update")
+    return g8, shift_out, sync
+
+
 def loss_grad(out_val, out_exp, target, rand, div_mode="floor"):
     """TiLoss.forward (ti_loss.py:5-36) as one launch: int8 logits [n, classes] with exponent ``out_exp`` (1-element
     int32 device tensor), int64 targets [n], int32 random integers [n, classes] -> int8 gradient (exponent 0)."""

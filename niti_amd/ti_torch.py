@@ -501,11 +501,34 @@ class TiLinear(UpdateWeight):
         self._init_weight(torch.Size([out_features, in_features]))
         self.last_layer = last_layer
 
+    def _one_launch(self, which, M, fn, rand):
+        """The pass runs as one of the library's kernels for few output features (operands read as stored,
+        requantisation folded in) when the shape is inside them and the rounding needs no random input."""
+        O, F = self.weight.shape
+        return (FUSE_CONV_REQUANT and rand is None and _method_name(fn) != "sto" and self.weight.is_contiguous()
+                and (which, M, O, F) not in _fused_refused and ops.fc_sync_words(which, M, O, F) > 0)
+
+    def _try(self, which, M, call):
+        """``call()``, or None when the device turned out too small to hold the kernel's grid at once."""
+        from ._lib import NitiError
+        try:
+            return call()
+        except NitiError as e:
+            if "do not fit" not in str(e):
+                raise
+            _fused_refused.add((which, M) + tuple(self.weight.shape))
+            return None
+
     def forward(self, input, rand=None):
         self.act_in = input
         act_in, exp_in = input
         act_in = act_in.contiguous()
         dev = act_in.device
+        if self._one_launch("forward", act_in.shape[0], ACT_ROUND_METHOD, rand):
+            exp_out = torch.empty(1, dtype=torch.int32, device=dev)
+            act_out, _, _ = ops.fc_fwd_requant(act_in, self.weight, BITWIDTH, _method_name(ACT_ROUND_METHOD), DIV_MODE, BW_MODE,
+                                               exp_a=_exp_tensor(exp_in, dev), exp_b=self._wexp(), exp_out=exp_out)
+            return act_out, exp_out
         am = ops.new_scalar_u32(dev)
         acc = ops.gemm(act_in, self.weight, trans_b=True, absmax=am)            # act @ W^T, W read as stored
         act_out, _, exp_out = _requant(acc, BITWIDTH, ACT_ROUND_METHOD, am, rand,
@@ -517,14 +540,35 @@ class TiLinear(UpdateWeight):
         err_in = err_in.contiguous()
         dev = err_in.device
         act, self.act_in_exp = self.act_in
+        act = act.contiguous()
+        M = err_in.shape[0]
         self.err_exp_in = _exp_tensor(err_exp, dev)
-        am = ops.new_scalar_u32(dev)
-        dx = ops.gemm(err_in, self.weight, absmax=am)                             # err @ W
-        err_out, _, self.err_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
-                                            exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
-        amg = ops.new_scalar_u32(dev)
-        self.grad_int32acc = ops.gemm(err_in, act.contiguous(), trans_a=True, absmax=amg)   # err^T @ act
-        self.weight_update(amg, grad_rand)
+        done = None
+        if self._one_launch("dgrad", M, ERROR_ROUND_METHOD, rand):
+            new_exp = torch.empty(1, dtype=torch.int32, device=dev)
+            done = self._try("dgrad", M, lambda: ops.fc_dgrad_requant(
+                err_in, self.weight, BITWIDTH, _method_name(ERROR_ROUND_METHOD), DIV_MODE, BW_MODE,
+                exp_a=self.err_exp_in, exp_b=self._wexp(), exp_out=new_exp))
+        if done is not None:
+            err_out, self.err_exp = done[0], new_exp
+        else:
+            am = ops.new_scalar_u32(dev)
+            dx = ops.gemm(err_in, self.weight, absmax=am)                             # err @ W
+            err_out, _, self.err_exp = _requant(dx, BITWIDTH, ERROR_ROUND_METHOD, am, rand,
+                                                exp_a=self.err_exp_in, exp_b=self._wexp(), want_exp=True)
+        done = None
+        if not KEEP_INT32_GRAD and self._one_launch("wgrad", M, GRAD_ROUND_METHOD, grad_rand):
+            self.grad_exp = torch.empty(1, dtype=torch.int32, device=dev)
+            done = self._try("wgrad", M, lambda: ops.fc_wgrad_update(
+                err_in, act, self.weight, GRAD_BITWIDTH, _method_name(GRAD_ROUND_METHOD), DIV_MODE, BW_MODE,
+                want_grad=self.keep_grad, exp_a=_exp_tensor(self.err_exp, dev), exp_b=_exp_tensor(self.act_in_exp, dev),
+                exp_out=self.grad_exp))
+        if done is not None:
+            self.grad, self.grad_shift, self.grad_int32acc = done[0], done[1], None
+        else:
+            amg = ops.new_scalar_u32(dev)
+            self.grad_int32acc = ops.gemm(err_in, act, trans_a=True, absmax=amg)     # err^T @ act
+            self.weight_update(amg, grad_rand)
         return err_out, self.err_exp
 
 

@@ -323,6 +323,55 @@ def test_conv_wgrad_update(dev, case, div_mode):
             assert torch.equal(wp.cpu(), ops.conv_filter_prepare(w16_ref, N, Q, Q).cpu())
 
 
+@pytest.mark.parametrize("case", [(128, 10, 8192), (5, 3, 64), (33, 16, 272), (512, 10, 1024), (1, 1, 16), (100, 7, 4000)])
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+def test_fc_few_outputs(dev, case, div_mode):
+    """TiLinear's three passes as one launch each (few output features) against GEMM + requantisation of the oracle."""
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    M, O, F = case
+    _say("fc_few_outputs", case, div_mode)
+    g = torch.Generator().manual_seed(4100 + M + O + F)
+    act, w, err = ri8(g, M, F), ri8(g, O, F), ri8(g, M, O, lo=-40, hi=40)
+    ea = torch.tensor([-3], dtype=torch.int32, device=dev)
+    eb = torch.tensor([-5], dtype=torch.int32, device=dev)
+    # forward: act_calc(act @ w^T)
+    acc = po.int8mm(act, w.t().contiguous())
+    for method in ("round", "psto"):
+        ref, sh_ref = po.act_calc(acc, 0, method, div_mode)
+        eo = torch.zeros(1, dtype=torch.int32, device=dev)
+        y, sh, sync = ops.fc_fwd_requant(act.to(dev), w.to(dev), 7, method, div_mode, exp_a=ea, exp_b=eb, exp_out=eo)
+        sync = sync.cpu()
+        assert int(sync[0]) == po.absmax(acc) and int(sync[1]) == 0
+        assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(eo.cpu()) == sh_ref - 8
+        # data gradient: err_calc(err @ w)
+        dacc = po.int8mm(err, w)
+        dref, dsh = po.err_calc(dacc, method, div_mode)
+        dx, sh, sync = ops.fc_dgrad_requant(err.to(dev), w.to(dev), 7, method, div_mode, exp_a=ea, exp_out=eo)
+        sync = sync.cpu()
+        assert int(sync[0]) == po.absmax(dacc) and int(sync[1]) == 0
+        assert torch.equal(dx.cpu(), dref) and int(sh.cpu()) == dsh and int(eo.cpu()) == dsh - 3
+        # weight gradient, grad_calc, update
+        if M <= 512:
+            gacc = po.int8mm(err.t().contiguous(), act)
+            for mu in (5, 3):
+                g8_ref, gsh = po.grad_calc(gacc, mu, method, div_mode)
+                w_ref = po.weight_update(w, g8_ref)
+                wd = w.to(dev).clone()
+                g8, sh, sync = ops.fc_wgrad_update(err.to(dev), act.to(dev), wd, mu, method, div_mode, want_grad=True,
+                                                   exp_a=ea, exp_b=eb, exp_out=eo)
+                sync = sync.cpu()
+                assert int(sync[0]) == po.absmax(gacc) and int(sync[1]) == 0
+                assert torch.equal(g8.cpu(), g8_ref) and int(sh.cpu()) == gsh and int(eo.cpu()) == gsh - 8
+                assert torch.equal(wd.cpu(), w_ref)
+                wd2 = w.to(dev).clone()
+                ops.fc_wgrad_update(err.to(dev), act.to(dev), wd2, mu, method, div_mode)
+                assert torch.equal(wd2.cpu(), w_ref)
+    # shapes outside the kernels are reported, not run
+    assert ops.fc_sync_words("forward", 128, 17, 8192) == 0 and ops.fc_sync_words("wgrad", 513, 10, 64) == 0
+    assert ops.fc_sync_words("dgrad", 8, 10, 24) == 0
+
+
 def test_conv_requant_rejects_what_it_does_not_cover(dev):
     from niti_amd import ops
     from niti_amd._lib import NitiError
