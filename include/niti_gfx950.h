@@ -47,6 +47,8 @@ enum { NITI_ROUND_NEAREST = 0, NITI_ROUND_STOCHASTIC = 1, NITI_ROUND_PSEUDO_STOC
 enum { NITI_DIV_FLOOR = 0, NITI_DIV_TRUNC = 1 };
 enum { NITI_BW_INT = 0, NITI_BW_F32 = 1 };
 enum { NITI_TIES_FIRST = 0, NITI_TIES_ALL = 1 };
+#define NITI_POOL_BWD_RELU 2 /* or-ed into `ties` of niti_maxpool_i8_bwd: also zero dx where x <= 0, the backward pass
+                                of a ReLU whose output is the pooling's input (TiReLU.backward, ti_torch.py:289) */
 
 int niti_version(void);
 const char* niti_status_string(int status);
@@ -230,6 +232,10 @@ int niti_grad_update_i8(const int32_t* g, int8_t* w, int64_t n, const uint32_t* 
                         int div_mode, int bw_mode, const int32_t* rand, int8_t* g8_out, int32_t* shift_out,
                         const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
 
+/* dst [rows][kpad] = src [rows][k] with zeros appended to every row: the zero padding of the channel dimension to a
+   multiple of 16 that conv2d_int8 applies to input and filter (ti_torch.py:182-187), as one launch */
+int niti_pad_rows_i8(const int8_t* src, int8_t* dst, int64_t rows, int k, int kpad, void* stream);
+
 /* w = clip(int16(w) - int16(g), +-127)  (ti_torch.py:21) */
 int niti_weight_update_i8(int8_t* w, const int8_t* g, int64_t n, void* stream);
 
@@ -242,7 +248,8 @@ int niti_relu_i8_bwd(const int8_t* act, const int8_t* dy, int8_t* dx, int64_t n,
  * (pytorch/int8pool-extension/int8pool.cpp:37-57, int8pool_kernel.cu:28-138).
  * x: [N,H,W,C], y/dy: [N,P,Q,C], dx: [N,H,W,C], P=(H+2*pad-ks)/stride+1.
  * Backward routes dy to the position(s) of x equal to y: the first in (kh,kw) scan order
- * (NITI_TIES_FIRST) or all of them (NITI_TIES_ALL); overlapping windows add.
+ * (NITI_TIES_FIRST) or all of them (NITI_TIES_ALL); overlapping windows add.  NITI_POOL_BWD_RELU or-ed into
+ * `ties` folds the backward pass of a ReLU in front of the pooling into the same launch.
  */
 int niti_maxpool_i8_fwd(const int8_t* x, int8_t* y, int N, int H, int W, int C, int ks, int stride, int pad,
                         void* stream);
@@ -257,7 +264,7 @@ int niti_maxpool_i8_bwd(const int8_t* y, const int8_t* dy, const int8_t* x, int8
  *   wgrad_update:  g = grad_calc(err^T * act), w = clip(w - g)  (ti_torch.py:263-265, 16-21); g8_out optional
  * `which` names the pass for the sync query, which returns 0 for shapes these kernels do not cover (then use
  * niti_gemm_i8 + niti_requant_i32_i8 / niti_grad_update_i8).  sync: zeroed uint32 words as for the convolutions
- * (word 0 range out, word 1 time-out flag; the forward pass accumulates its int32 sums in the words from 16 on).
+ * (word 0 range out, word 1 time-out flag, one slot per workgroup from word 16).
  * Rounding NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC; shift_out / exp_* as in niti_requant_i32_i8.
  */
 enum { NITI_FC_FORWARD = 0, NITI_FC_DGRAD = 1, NITI_FC_WGRAD = 2 };

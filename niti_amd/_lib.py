@@ -19,6 +19,7 @@ ROUND = {"round": 0, "sto": 1, "psto": 2}
 DIV = {"floor": 0, "trunc": 1}
 BW = {"int": 0, "f32": 1}
 TIES = {"first": 0, "all": 1}
+POOL_BWD_RELU = 2
 
 _vp, _i, _u, _i64, _sz = C.c_void_p, C.c_int, C.c_uint, C.c_int64, C.c_size_t
 
@@ -46,6 +47,7 @@ SIGNATURES = {
     "niti_absmax_i32": (_i, [_vp, _i64, _vp, _vp]),
     "niti_requant_i32_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _u, _vp, _vp, _vp, _vp, _vp]),
     "niti_grad_update_i8": (_i, [_vp, _vp, _i64, _vp, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "niti_pad_rows_i8": (_i, [_vp, _vp, _i64, _i, _i, _vp]),
     "niti_weight_update_i8": (_i, [_vp, _vp, _i64, _vp]),
     "niti_relu_i8_fwd": (_i, [_vp, _vp, _i64, _vp]),
     "niti_relu_i8_bwd": (_i, [_vp, _vp, _vp, _i64, _vp]),

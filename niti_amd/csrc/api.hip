@@ -111,6 +111,16 @@ static int check_forward_copy_flag(const char* who, int dgrad, unsigned flags, i
   return NITI_OK;
 }
 
+extern "C" int niti_pad_rows_i8(const int8_t* src, int8_t* dst, int64_t rows, int k, int kpad, void* stream) {
+  clear_error();
+  if (src == nullptr || dst == nullptr) return fail(NITI_ERR_INVALID_ARG, "pad_rows: null pointer");
+  if (rows <= 0 || k <= 0 || kpad < k) return fail(NITI_ERR_INVALID_ARG, "pad_rows: rows=%lld k=%d kpad=%d", static_cast<long long>(rows), k, kpad);
+  int64_t g = (rows * kpad + 255) / 256;
+  if (g > 4096) g = 4096;
+  hipLaunchKernelGGL(pad_rows_i8_kernel, dim3(static_cast<unsigned>(g)), dim3(256), 0, static_cast<hipStream_t>(stream), src, dst, rows, k, kpad);
+  return check_launch("pad_rows");
+}
+
 extern "C" size_t niti_conv2d_i8_filter_workspace(int N, int H, int W, int C, int K, int R, int S, int stride, int pad,
                                                   int dgrad) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0) return 0;

@@ -3,14 +3,13 @@
 // kernels one ragged tile and two operand re-layouts; written for the shape, all three passes read their
 // operands as stored:
 //   forward   out[m][o] = sum_f act[m][f] w[o][f]   -> act_calc: both operands are reduction-contiguous, which is
-//             the register layout of v_mfma_i32_16x16x64_i8; the reduction is split over many wavefronts whose
-//             partial tiles meet in zeroed int32 words by atomic adds, and the wavefront that arrives last
-//             (a counter) owns the range, the rounding and the int8 store - nobody waits.
+//             the register layout of v_mfma_i32_16x16x64_i8; a workgroup owns 16 samples, its 16 wavefronts split
+//             the reduction and are added through LDS.
 //   dgrad     dx[m][f] = sum_o err[m][o] w[o][f]    -> err_calc: a lane owns 16 consecutive f of one sample.
 //   wgrad     g[o][f]  = sum_m err[m][o] act[m][f]  -> grad_calc -> w = clip(w - g): a lane owns 4 consecutive f,
 //             the four wavefronts of a workgroup each take a quarter of the samples (four at a time through
 //             v_dot4_i32_i8 after a 4 x 4 byte transposition) and are added through LDS.
-// dgrad and wgrad keep their int32 sums in registers across the tensor-wide range: every workgroup publishes its
+// All three keep their int32 sums in registers across the tensor-wide range: every workgroup publishes its
 // largest magnitude in a slot of its own and reads all slots (all workgroups resident - checked by the host - and
 // the wait bounded by a wall-clock limit), as the convolution kernels do.
 #include "common.h"
@@ -19,7 +18,7 @@
 namespace niti {
 namespace {
 
-constexpr int kSlot0 = 16;      // sync words: 0 range out, 1 wait gave up, 2 arrival counter, 16.. slots / accumulators
+constexpr int kSlot0 = 16;      // sync words: 0 range out, 1 wait gave up, 16.. one slot per workgroup
 constexpr int kMaxOut = 16;     // output features these kernels handle
 constexpr int kWgradMaxM = 512;
 
@@ -30,8 +29,7 @@ struct FcArgs {
   int8_t* out8;        // forward: [M][O]; dgrad: [M][F]; wgrad: optional rounded gradient [O][F]
   uint32_t* sync;
   int M, O, F;
-  int ksplit, kchunk;  // forward: wavefronts per 16-sample tile, reduction elements per wavefront
-  int total_waves;
+  int kchunk;          // forward: reduction elements per wavefront
   int target_bits, method, trunc, bw_mode;
   unsigned rq_flags;
   long long spin_limit;
@@ -81,59 +79,63 @@ __device__ inline uint32_t exchange_range(const FcArgs& a, uint32_t bmax) {
 }
 
 // ---- forward ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void fc_fwd_requant_kernel(const FcArgs a) {
+// One workgroup of 16 wavefronts per tile of 16 samples; wavefront w reduces over features [w * kchunk, (w+1) * kchunk).
+__global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
+  __shared__ int part[16][256];
+  __shared__ uint32_t gshare;
   const int lane = threadIdx.x & 63;
-  const int wid = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (wid >= a.total_waves) return;
-  const int mt = wid / a.ksplit, ks = wid - mt * a.ksplit;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int mt = blockIdx.x;
   const int row = lane & 15, kg = lane >> 4;           // operand row (sample / output feature), 16-byte piece of a 64-step
   const int m = mt * 16 + row;
-  const int k0 = ks * a.kchunk;
+  const int k0 = wave * a.kchunk;
   const int k1 = min(k0 + a.kchunk, a.F);
   const int8_t* pa = a.act + static_cast<long long>(m) * a.F;
   const int8_t* pw = a.w + static_cast<long long>(row) * a.F;
   const bool va = m < a.M, vw = row < a.O;
   v4i acc = {0, 0, 0, 0};
   const v4i zero = {0, 0, 0, 0};
-  for (int k = k0 + kg * 16; k < k1 + kg * 16; k += 64) {   // every lane runs the same number of steps
-    const bool in = k < k1;                                   // F is a multiple of 16: a piece is inside or outside
-    const v4i fa = (va && in) ? *reinterpret_cast<const v4i*>(pa + k) : zero;
-    const v4i fw = (vw && in) ? *reinterpret_cast<const v4i*>(pw + k) : zero;
-    acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa, fw, acc, 0, 0, 0);
+  for (int kb = k0; kb < k1; kb += 256) {                 // four 64-steps at a time, their loads in flight together
+    v4i fa[4], fw[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int k = kb + u * 64 + kg * 16;
+      const bool in = k < k1;                             // F is a multiple of 16: a piece is inside or outside
+      fa[u] = (va && in) ? *reinterpret_cast<const v4i*>(pa + k) : zero;
+      fw[u] = (vw && in) ? *reinterpret_cast<const v4i*>(pw + k) : zero;
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fw[u], acc, 0, 0, 0);
   }
   // acc[i]: sample mt*16 + 4*(lane/16) + i, output feature lane%16
-  int* const sums = reinterpret_cast<int*>(a.sync + kSlot0);
-  const int o = lane & 15;
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int mm = mt * 16 + 4 * (lane >> 4) + i;
-    if (mm < a.M && o < a.O && acc[i] != 0) atomicAdd(&sums[mm * kMaxOut + o], acc[i]);
-  }
-  __threadfence();
-  uint32_t arrived = 0;
-  if (lane == 0) arrived = atomicAdd(&a.sync[2], 1u);
-  arrived = __builtin_amdgcn_readfirstlane(arrived);
-  if (arrived != static_cast<uint32_t>(a.total_waves - 1)) return;
-  // the last wavefront to arrive: every partial tile is in; range, shift, rounding, store
-  __threadfence();
-  const int n = a.M * a.O;
-  uint32_t lmax = 0;
-  for (int i = lane; i < n; i += 64) {
-    const int mm = i / a.O, oo = i - mm * a.O;
-    const int v = __hip_atomic_load(&sums[mm * kMaxOut + oo], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint32_t u = uabs(v);
-    lmax = u > lmax ? u : lmax;
-  }
-  const uint32_t gmax = wave_max_u32(lmax);
-  const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
-  if (lane == 0) write_scalars(a, gmax, shift);
-  const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC, trunc = a.trunc != 0, relu = (a.rq_flags & NITI_RQ_RELU) != 0;
-  for (int i = lane; i < n; i += 64) {
-    const int mm = i / a.O, oo = i - mm * a.O;
-    const int v = __hip_atomic_load(&sums[mm * kMaxOut + oo], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    int r = round_to_i8(v, shift, psto, trunc);
-    if (relu && r < 0) r = 0;
-    a.out8[i] = static_cast<int8_t>(r);
+  for (int i = 0; i < 4; ++i) part[wave][i * 64 + lane] = acc[i];
+  __syncthreads();
+  if (wave == 0) {
+    uint32_t lmax = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int sum = 0;
+#pragma unroll
+      for (int w = 0; w < 16; ++w) sum += part[w][i * 64 + lane];
+      acc[i] = sum;
+      const uint32_t u = uabs(sum);     // rows beyond M and columns beyond O are sums of zeros
+      lmax = u > lmax ? u : lmax;
+    }
+    const uint32_t gmax = exchange_range(a, wave_max_u32(lmax));
+    const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
+    if (blockIdx.x == 0 && lane == 0) write_scalars(a, gmax, shift);
+    const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC, trunc = a.trunc != 0, relu = (a.rq_flags & NITI_RQ_RELU) != 0;
+    const int o = lane & 15;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int mm = mt * 16 + 4 * (lane >> 4) + i;
+      if (mm < a.M && o < a.O) {
+        int r = round_to_i8(acc[i], shift, psto, trunc);
+        if (relu && r < 0) r = 0;
+        a.out8[static_cast<long long>(mm) * a.O + o] = static_cast<int8_t>(r);
+      }
+    }
   }
 }
 
@@ -150,15 +152,22 @@ __global__ __launch_bounds__(256) void fc_dgrad_requant_kernel(const FcArgs a) {
   int acc[16];
 #pragma unroll
   for (int i = 0; i < 16; ++i) acc[i] = 0;
-  if (valid) {
-    for (int o = 0; o < a.O; ++o) {
-      const int e = a.err[static_cast<long long>(m) * a.O + o];
-      const v4i wv = *reinterpret_cast<const v4i*>(a.w + static_cast<long long>(o) * a.F + f);
+  {
+    // all rows of w at once (rows beyond O repeat the last one with a zero factor): sixteen loads in flight
+    v4i wv[kMaxOut];
+    int e[kMaxOut];
+#pragma unroll
+    for (int o = 0; o < kMaxOut; ++o) {
+      const int oo = min(o, a.O - 1);
+      wv[o] = *reinterpret_cast<const v4i*>(a.w + static_cast<long long>(oo) * a.F + f);
+      e[o] = (valid && o < a.O) ? static_cast<int>(a.err[static_cast<long long>(m) * a.O + oo]) : 0;
+    }
+#pragma unroll
+    for (int o = 0; o < kMaxOut; ++o)
 #pragma unroll
       for (int d = 0; d < 4; ++d)
 #pragma unroll
-        for (int b = 0; b < 4; ++b) acc[4 * d + b] += e * static_cast<int>(static_cast<int8_t>((static_cast<uint32_t>(wv[d]) >> (8 * b)) & 0xFFu));
-    }
+        for (int b = 0; b < 4; ++b) acc[4 * d + b] += e[o] * static_cast<int>(static_cast<int8_t>((static_cast<uint32_t>(wv[o][d]) >> (8 * b)) & 0xFFu));
   }
   uint32_t lmax = 0;
 #pragma unroll
@@ -196,6 +205,23 @@ __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int groups = (a.M + 3) >> 2;                      // groups of four samples
+  const int f = (blockIdx.x * 64 + lane) * 4;
+  const bool valid = f < a.F;                              // F is a multiple of 4
+  const int per = (groups + 3) >> 2;
+  const int g0 = wave * per, g1 = min(g0 + per, groups);
+  const int8_t* pa = a.act + f;
+  constexpr int kAhead = 4;   // groups of four samples whose loads are in flight together
+  auto load = [&](int gb, uint32_t (&r)[kAhead][4]) {
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int m = 4 * (gb + u) + j;
+        r[u][j] = (valid && gb + u < g1 && m < a.M) ? *reinterpret_cast<const uint32_t*>(pa + static_cast<long long>(m) * a.F) : 0u;
+      }
+  };
+  uint32_t ra[kAhead][4], rb[kAhead][4];
+  load(g0, ra);                                             // in flight while the error words are put together
   for (int i = threadIdx.x; i < kMaxOut * groups; i += 256) {
     const int o = i / groups, g = i - o * groups;
     uint32_t word = 0;
@@ -209,39 +235,38 @@ __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
     err_t[o][g] = word;
   }
   __syncthreads();
-  const int f = (blockIdx.x * 64 + lane) * 4;
-  const bool valid = f < a.F;                              // F is a multiple of 4
   int acc[kMaxOut][4];
 #pragma unroll
   for (int o = 0; o < kMaxOut; ++o)
 #pragma unroll
     for (int b = 0; b < 4; ++b) acc[o][b] = 0;
-  const int per = (groups + 3) >> 2;
-  const int g0 = wave * per, g1 = min(g0 + per, groups);
-  const int8_t* pa = a.act + f;
-  for (int g = g0; g < g1; ++g) {
-    uint32_t r[4];
+  auto mac = [&](int gb, const uint32_t (&r)[kAhead][4]) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int m = 4 * g + j;
-      r[j] = (valid && m < a.M) ? *reinterpret_cast<const uint32_t*>(pa + static_cast<long long>(m) * a.F) : 0u;
-    }
-    // 4 x 4 byte transposition: c[b] = byte b (feature f + b) of the four samples
-    const uint32_t lo01 = __builtin_amdgcn_perm(r[1], r[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(r[1], r[0], 0x07030602u);
-    const uint32_t lo23 = __builtin_amdgcn_perm(r[3], r[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(r[3], r[2], 0x07030602u);
-    uint32_t c[4];
-    c[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
-    c[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
-    c[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
-    c[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+    for (int u = 0; u < kAhead; ++u) {
+      const int g = min(gb + u, groups - 1);   // beyond g1 the loaded activations are zero
+      // 4 x 4 byte transposition: c[b] = byte b (feature f + b) of the four samples
+      const uint32_t lo01 = __builtin_amdgcn_perm(r[u][1], r[u][0], 0x05010400u), hi01 = __builtin_amdgcn_perm(r[u][1], r[u][0], 0x07030602u);
+      const uint32_t lo23 = __builtin_amdgcn_perm(r[u][3], r[u][2], 0x05010400u), hi23 = __builtin_amdgcn_perm(r[u][3], r[u][2], 0x07030602u);
+      uint32_t c[4];
+      c[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+      c[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+      c[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+      c[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
 #pragma unroll
-    for (int o = 0; o < kMaxOut; ++o) {
-      if (o < a.O) {
-        const int ew = static_cast<int>(err_t[o][g]);
+      for (int o = 0; o < kMaxOut; ++o) {
+        if (o < a.O) {
+          const int ew = static_cast<int>(err_t[o][g]);
 #pragma unroll
-        for (int b = 0; b < 4; ++b) acc[o][b] = __builtin_amdgcn_sdot4(static_cast<int>(c[b]), ew, acc[o][b], false);
+          for (int b = 0; b < 4; ++b) acc[o][b] = __builtin_amdgcn_sdot4(static_cast<int>(c[b]), ew, acc[o][b], false);
+        }
       }
     }
+  };
+  for (int gb = g0; gb < g1; gb += 2 * kAhead) {
+    load(gb + kAhead, rb);
+    mac(gb, ra);
+    load(gb + 2 * kAhead, ra);
+    mac(gb + kAhead, rb);
   }
   if (wave > 0) {
 #pragma unroll
@@ -260,6 +285,10 @@ __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
       const uint32_t u = uabs(acc[o][b]);
       lmax = u > lmax ? u : lmax;
     }
+  uint32_t wcur[kMaxOut];   // the weights this lane updates, fetched while the ranges are exchanged
+#pragma unroll
+  for (int o = 0; o < kMaxOut; ++o)
+    wcur[o] = (valid && o < a.O) ? *reinterpret_cast<const uint32_t*>(a.w + static_cast<long long>(o) * a.F + f) : 0u;
   const uint32_t gmax = exchange_range(a, wave_max_u32(lmax));
   const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
   if (blockIdx.x == 0 && lane == 0) write_scalars(a, gmax, shift);
@@ -269,7 +298,7 @@ __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
   for (int o = 0; o < kMaxOut; ++o) {
     if (o < a.O) {
       uint32_t* pw = reinterpret_cast<uint32_t*>(a.w + static_cast<long long>(o) * a.F + f);
-      const uint32_t wold = *pw;
+      const uint32_t wold = wcur[o];
       int r[4];
       uint32_t wnew = 0;
 #pragma unroll
@@ -284,33 +313,23 @@ __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
   }
 }
 
-int resident_blocks(const void* kernel) {
+int resident_blocks(const void* kernel, int threads = 256) {
   int dev = 0, cus = 0, per_cu = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess)
+      hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, threads, 0) != hipSuccess)
     return 0;
   return cus * per_cu;
 }
 
-// forward: reduction elements per wavefront (a multiple of 64) and wavefronts per 16-sample tile
-void fwd_split(int M, int F, int* ksplit, int* kchunk) {
-  const int tiles = (M + 15) / 16;
-  const int steps = (F + 63) / 64;
-  int want = 1024 / tiles;                 // about four wavefronts per compute unit
-  if (want < 1) want = 1;
-  int per = (steps + want - 1) / want;
-  if (per < 4) per = 4;
-  *kchunk = per * 64;
-  *ksplit = (F + *kchunk - 1) / *kchunk;
-}
+// forward: reduction elements per wavefront (a multiple of 256), sixteen wavefronts per 16-sample tile
+int fwd_chunk(int F) { return ((F + 15) / 16 + 255) / 256 * 256; }
 
 long long blocks_of(int which, int M, int O, int F) {
   if (M <= 0 || O <= 0 || F <= 0 || O > kMaxOut) return 0;
   if (which == NITI_FC_FORWARD) {
-    if (F % 16 != 0 || static_cast<long long>(M) * kMaxOut > (1 << 22)) return 0;
-    int ksplit, kchunk;
-    fwd_split(M, F, &ksplit, &kchunk);
-    return (static_cast<long long>((M + 15) / 16) * ksplit + 3) / 4;
+    if (F % 16 != 0) return 0;
+    const long long nb = (M + 15) / 16;
+    return nb <= 4096 ? nb : 0;
   }
   if (which == NITI_FC_DGRAD) {
     if (F % 16 != 0) return 0;
@@ -333,7 +352,6 @@ using namespace niti;
 extern "C" size_t niti_fc_i8_sync_words(int which, int M, int O, int F) {
   const long long nb = blocks_of(which, M, O, F);
   if (nb == 0) return 0;
-  if (which == NITI_FC_FORWARD) return static_cast<size_t>(kSlot0) + static_cast<size_t>(M) * kMaxOut;
   return static_cast<size_t>(kSlot0 + (nb + 15) / 16 * 16);
 }
 
@@ -383,9 +401,11 @@ extern "C" int niti_fc_i8_fwd_requant(const int8_t* act, const int8_t* w, int8_t
   a.w = const_cast<int8_t*>(w);
   a.out8 = out8;
   a.rq_flags = rq_flags;
-  fwd_split(M, F, &a.ksplit, &a.kchunk);
-  a.total_waves = ((M + 15) / 16) * a.ksplit;
-  hipLaunchKernelGGL(fc_fwd_requant_kernel, dim3(static_cast<unsigned>(nb)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+  static int resident = 0;
+  if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_fwd_requant_kernel), 1024);
+  if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "fc_fwd_requant: %lld workgroups do not fit on the device at once (%d)", nb, resident);
+  a.kchunk = fwd_chunk(F);
+  hipLaunchKernelGGL(fc_fwd_requant_kernel, dim3(static_cast<unsigned>(nb)), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
   return check_launch("fc_fwd_requant");
 }
 

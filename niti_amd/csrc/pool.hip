@@ -3,6 +3,7 @@
 // Pooling threads own 16 consecutive channels of one pixel (one 16-byte load/store) when
 // C % 16 == 0, one channel otherwise.
 #include "common.h"
+#include "requant_math.h"
 
 namespace niti {
 namespace {
@@ -47,6 +48,7 @@ struct PoolArgs {
   const int8_t* dy;
   int8_t* out;
   int N, H, W, C, P, Q, ks, stride, pad, ties_all;
+  int relu;   // backward: also zero the positions whose input is not positive (a ReLU in front of the pooling)
 };
 
 template <int V>
@@ -141,6 +143,10 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const PoolArgs a) {
         for (int e = 0; e < V; ++e) acc[e] += hit[e] ? ds.get(e) : 0;
       }
     }
+    if (a.relu) {
+#pragma unroll
+      for (int e = 0; e < V; ++e) acc[e] = xs.get(e) > 0 ? acc[e] : 0;
+    }
     pack_store<V>(a.out + i * V, acc);
   }
 }
@@ -180,7 +186,9 @@ __global__ __launch_bounds__(256) void maxpool2x2_bwd_kernel(const PoolArgs a) {
 #pragma unroll
       for (int k = 0; k < 4; ++k) {
         const uint32_t eq = equal_bytes(static_cast<uint32_t>(x[k][e]), static_cast<uint32_t>(y[e]));
-        o[k][e] = static_cast<int>(static_cast<uint32_t>(d[e]) & (kAll ? eq : eq & ~taken));
+        uint32_t keep = kAll ? eq : eq & ~taken;
+        if (a.relu) keep &= positive_bytes(static_cast<uint32_t>(x[k][e]));
+        o[k][e] = static_cast<int>(static_cast<uint32_t>(d[e]) & keep);
         taken |= eq;
       }
     }
@@ -260,7 +268,7 @@ extern "C" int niti_maxpool_i8_fwd(const int8_t* x, int8_t* y, int N, int H, int
   int st = check_pool("maxpool_fwd", N, H, W, C, ks, stride, pad, &P, &Q);
   if (st != NITI_OK) return st;
   if (x == nullptr || y == nullptr) return fail(NITI_ERR_INVALID_ARG, "maxpool_fwd: null pointer");
-  PoolArgs a{x, nullptr, nullptr, y, N, H, W, C, P, Q, ks, stride, pad, 0};
+  PoolArgs a{x, nullptr, nullptr, y, N, H, W, C, P, Q, ks, stride, pad, 0, 0};
   const bool vec = C % 16 == 0 && aligned16(x) && aligned16(y);
   const int64_t total = static_cast<int64_t>(N) * P * Q * (vec ? C / 16 : C);
   if (vec) hipLaunchKernelGGL(maxpool_fwd_kernel<16>, dim3(grid_for(total, 256)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
@@ -275,8 +283,10 @@ extern "C" int niti_maxpool_i8_bwd(const int8_t* y, const int8_t* dy, const int8
   int st = check_pool("maxpool_bwd", N, H, W, C, ks, stride, pad, &P, &Q);
   if (st != NITI_OK) return st;
   if (x == nullptr || y == nullptr || dy == nullptr || dx == nullptr) return fail(NITI_ERR_INVALID_ARG, "maxpool_bwd: null pointer");
+  const int relu = (ties & NITI_POOL_BWD_RELU) != 0;
+  ties &= ~NITI_POOL_BWD_RELU;
   if (ties != NITI_TIES_FIRST && ties != NITI_TIES_ALL) return fail(NITI_ERR_INVALID_ARG, "maxpool_bwd: ties=%d", ties);
-  PoolArgs a{x, y, dy, dx, N, H, W, C, P, Q, ks, stride, pad, ties == NITI_TIES_ALL};
+  PoolArgs a{x, y, dy, dx, N, H, W, C, P, Q, ks, stride, pad, ties == NITI_TIES_ALL, relu};
   const bool vec = C % 16 == 0 && aligned16(x) && aligned16(y) && aligned16(dy) && aligned16(dx);
   if (vec && ks == 2 && stride == 2 && pad == 0 && H % 2 == 0 && W % 2 == 0 && static_cast<int64_t>(N) * P * Q < 0x7fffffffLL) {
     const int64_t windows = static_cast<int64_t>(N) * P * Q * (C / 16);

@@ -473,6 +473,21 @@ def fc_wgrad_update(err, act, w, mu=5, method="psto", div_mode="floor", bw_mode=
     return g8, shift_out, sync
 
 
+def pad_last_dim(t, multiple=16):
+    """``t`` with zeros appended along its last dimension up to a multiple of ``multiple`` (``t`` itself when it
+    already is one): the channel padding of conv2d_int8 (ti_torch.py:182-187) as one launch."""
+    c = t.shape[-1]
+    if c % multiple == 0:
+        return t
+    _chk_dev(t)
+    if t.dtype != torch.int8:
+        raise RuntimeError("pad_last_dim: int8 tensor expected")
+    cp = (c + multiple - 1) // multiple * multiple
+    out = torch.empty(tuple(t.shape[:-1]) + (cp,), dtype=torch.int8, device=t.device)
+    L.check(L.lib().niti_pad_rows_i8(_ptr(t), _ptr(out), t.numel() // c, c, cp, _stream(t)), "niti_pad_rows_i8")
+    return out
+
+
 def loss_grad(out_val, out_exp, target, rand, div_mode="floor"):
     """TiLoss.forward (ti_loss.py:5-36) as one launch: int8 logits [n, classes] with exponent ``out_exp`` (1-element
     int32 device tensor), int64 targets [n], int32 random integers [n, classes] -> int8 gradient (exponent 0)."""
@@ -504,12 +519,13 @@ def maxpool_fwd(x, kernel_size=2, stride=2, padding=0):
     return y
 
 
-def maxpool_bwd(y, dy, x, kernel_size=2, stride=2, padding=0, ties="first"):
+def maxpool_bwd(y, dy, x, kernel_size=2, stride=2, padding=0, ties="first", relu=False):
+    """``relu``: also zero the gradient where x <= 0 (the backward pass of a ReLU whose output x is)."""
     _chk_dev(y, dy, x)
     N, H, W, C = x.shape
     dx = torch.empty_like(x)
     st = L.lib().niti_maxpool_i8_bwd(_ptr(y), _ptr(dy), _ptr(x), _ptr(dx), N, H, W, C, kernel_size, stride, padding,
-                                     L.TIES[ties], _stream(x))
+                                     L.TIES[ties] | (L.POOL_BWD_RELU if relu else 0), _stream(x))
     L.check(st, "niti_maxpool_i8_bwd")
     return dx
 

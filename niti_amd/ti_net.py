@@ -32,6 +32,10 @@ class TiNet(Module):
             if j < len(layers) and isinstance(layers[j], ti_torch.TiConv2d) and not layers[j].first_layer:
                 layers[j].relu_below = True
                 l.bwd_folded = True
+            elif j == i + 2:
+                # ReLU -> max-pool -> anything else: the pooling's backward pass applies the mask to its own output
+                layers[i + 1].relu_below = True
+                l.bwd_folded = True
         return self
 
     def forward(self, x):

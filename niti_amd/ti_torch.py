@@ -230,8 +230,11 @@ def int8mm(lhs, rhs):
 
 
 def _pad_channels16(t):
-    c = t.size(3)
-    return t if c % 16 == 0 else F.pad(t, (0, 16 - c % 16), "constant", 0)
+    if t.size(3) % 16 == 0:
+        return t
+    if t.is_cuda and t.dtype == torch.int8:
+        return ops.pad_last_dim(t.contiguous(), 16)
+    return F.pad(t, (0, 16 - t.size(3) % 16), "constant", 0)
 
 
 def conv2d_int8(input, weight, stride=1, padding=1, absmax=None):
@@ -589,7 +592,7 @@ class TiReLU(Module):
         return ops.relu_fwd(act_in.contiguous()), exp_in
 
     def backward(self, input):
-        if self.bwd_folded:      # the convolution above this layer masked its data gradient already
+        if self.bwd_folded:      # the convolution or pooling above this layer masked its data gradient already
             return input
         err_in, err_exp = input
         act, _ = self.act_in
@@ -604,6 +607,7 @@ class TiMaxpool2d(Module):
         self.kernel_size = kernel_size
         self.stride = stride
         self.padding = padding
+        self.relu_below = False     # the ReLU in front of this layer leaves its backward pass to this layer
 
     def forward(self, input):
         self.act_in, exp_in = input
@@ -614,7 +618,7 @@ class TiMaxpool2d(Module):
     def backward(self, input):
         err_in, err_exp = input
         err_out = ops.maxpool_bwd(self.act_out, err_in.contiguous(), self.act_in, self.kernel_size, self.stride,
-                                  self.padding, POOL_TIES)
+                                  self.padding, POOL_TIES, relu=self.relu_below)
         return err_out, err_exp
 
 

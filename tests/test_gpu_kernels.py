@@ -546,6 +546,22 @@ def test_maxpool(dev, case):
             ref = co.maxpool_bwd(yref, dy, x, ks, st, pad, ties)
             dx = ops.maxpool_bwd(y, dy.to(dev), x.to(dev), ks, st, pad, ties)
             assert torch.equal(dx.cpu(), ref), ties
+            # with the backward pass of a ReLU in front of the pooling folded in
+            dxr = ops.maxpool_bwd(y, dy.to(dev), x.to(dev), ks, st, pad, ties, relu=True)
+            assert torch.equal(dxr.cpu(), torch.where(x > 0, ref, torch.zeros_like(ref))), ties
+
+
+def test_pad_last_dim(dev):
+    import torch.nn.functional as F
+    from niti_amd import ops
+    g = torch.Generator().manual_seed(77)
+    for shape in ((128, 32, 32, 3), (7, 3, 3, 3), (5, 40), (2, 2, 2, 16), (3, 1, 1, 17)):
+        _say("pad_last_dim", shape)
+        x = ri8(g, *shape)
+        y = ops.pad_last_dim(x.to(dev), 16)
+        c = shape[-1]
+        ref = F.pad(x, (0, (16 - c % 16) % 16))
+        assert y.dtype == torch.int8 and torch.equal(y.cpu(), ref)
 
 
 def test_group_conv_first_layer_wgrad(dev):
