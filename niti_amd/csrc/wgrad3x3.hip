@@ -482,11 +482,13 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const int32_t* __rest
 }
 
 // Partial sums -> rounded gradient -> updated weights in one launch (the int32 gradient is not stored unless
-// asked for).  A workgroup owns kFinishV x 64 int4 columns at a grid-wide stride; its 4 wavefronts each add every
-// 4th slice and combine in LDS, wavefront 0 keeps the sums in registers, publishes the workgroup's largest
-// magnitude in its slot, waits for the slots of all workgroups (all resident: the host sizes the grid for that;
-// the wait is bounded by a wall-clock limit), derives the shift from the maximum over the slots and applies
-// w = clip(w - round(sum >> shift)).
+// asked for).  A workgroup owns kFinishV x 64 int4 columns at a grid-wide stride; its NW wavefronts each add every
+// NW-th slice of every column (no barrier in between, so all those loads are in flight together), column v is
+// then completed through LDS by wavefront v % NW, which keeps the sums in registers.  The workgroup publishes its
+// largest magnitude in its slot and waits for the slots of all workgroups (all resident: the host sizes the grid
+// for that; the wait is bounded by a wall-clock limit), derives the shift from the maximum over the slots, and
+// every wavefront applies w = clip(w - round(sum >> shift)) to its columns.  NW = 16 serves the launches with
+// many slices and few columns, NW = 4 the others.
 constexpr int kFinishV = 16;
 constexpr int kFinishSlot0 = 16;
 struct FinishArgs {
@@ -508,51 +510,61 @@ struct FinishArgs {
   int32_t* exp_out;
 };
 
-__global__ __launch_bounds__(256) void wgrad_finish_kernel(const FinishArgs a) {
-  __shared__ v4i part[3][64];
+template <int NW>
+__global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishArgs a) {
+  constexpr int OWN = kFinishV / NW > 0 ? kFinishV / NW : 1;   // columns a wavefront completes
+  __shared__ v4i part[2][NW][64];
+  __shared__ uint32_t wmax[NW];
   __shared__ uint32_t gshare;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   v4i sum[kFinishV];
-  uint32_t lmax = 0;
-  // phase 1: every wavefront adds its share of the slices for all of the workgroup's columns; no barrier in
-  // here, so the loads of all columns are in flight together
+  // phase 1: every wavefront adds its share of the slices for all of the workgroup's columns
 #pragma unroll
   for (int v = 0; v < kFinishV; ++v) {
     const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
     v4i s = {0, 0, 0, 0};
     if (col < a.nv) {
       int z = wave;
-      for (; z + 12 < a.splits; z += 16) {
-        const v4i v0 = reinterpret_cast<const v4i*>(a.partial + (z + 0) * a.slice_stride)[col];
-        const v4i v1 = reinterpret_cast<const v4i*>(a.partial + (z + 4) * a.slice_stride)[col];
-        const v4i v2 = reinterpret_cast<const v4i*>(a.partial + (z + 8) * a.slice_stride)[col];
-        const v4i v3 = reinterpret_cast<const v4i*>(a.partial + (z + 12) * a.slice_stride)[col];
+      for (; z + 3 * NW < a.splits; z += 4 * NW) {
+        const v4i v0 = reinterpret_cast<const v4i*>(a.partial + (z + 0 * NW) * a.slice_stride)[col];
+        const v4i v1 = reinterpret_cast<const v4i*>(a.partial + (z + 1 * NW) * a.slice_stride)[col];
+        const v4i v2 = reinterpret_cast<const v4i*>(a.partial + (z + 2 * NW) * a.slice_stride)[col];
+        const v4i v3 = reinterpret_cast<const v4i*>(a.partial + (z + 3 * NW) * a.slice_stride)[col];
         s += (v0 + v1) + (v2 + v3);
       }
-      for (; z < a.splits; z += 4) s += reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
+      for (; z < a.splits; z += NW) s += reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
     }
     sum[v] = s;
   }
-  // phase 2: combine the four wavefronts' shares in LDS; wavefront 0 keeps the totals
+  // phase 2: column v is completed by wavefront v % NW (two LDS buffers in turn: one barrier per column)
+  v4i fin[OWN];
+  uint32_t lmax = 0;
 #pragma unroll
   for (int v = 0; v < kFinishV; ++v) {
     if (static_cast<long long>(v) * gridDim.x * 64 >= a.nv) continue;  // uniform over the grid: nothing at this stride
-    if (wave > 0) part[wave - 1][lane] = sum[v];
+    part[v & 1][wave][lane] = sum[v];
     __syncthreads();
-    if (wave == 0) {
-      v4i s = sum[v] + part[0][lane] + part[1][lane] + part[2][lane];
+    if (wave == v % NW) {
+      v4i s = part[v & 1][0][lane];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) s += part[v & 1][w][lane];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
         const uint32_t u = uabs(s[e]);
         lmax = u > lmax ? u : lmax;
       }
-      sum[v] = s;
+      fin[v / NW] = s;
     }
-    __syncthreads();
   }
+  lmax = wave_max_u32(lmax);
+  if (lane == 0) wmax[wave] = lmax;
+  __syncthreads();
   if (wave == 0) {
-    const uint32_t bmax = wave_max_u32(lmax);
+    uint32_t bmax = 0;
+    for (int w = lane; w < NW; w += 64) bmax = max(bmax, wmax[w]);
+    bmax = wave_max_u32(bmax);
     const int nb = gridDim.x;
     uint32_t* const slots = a.sync + kFinishSlot0;
     if (lane == 0) __hip_atomic_store(&slots[blockIdx.x], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -574,68 +586,71 @@ __global__ __launch_bounds__(256) void wgrad_finish_kernel(const FinishArgs a) {
       __builtin_amdgcn_s_sleep(4);
     }
     g = wave_max_u32(g);
-    const uint32_t gmax = g != 0u ? g - 1u : 0u;
-    const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
-    if (blockIdx.x == 0 && lane == 0) {
-      const int sh = shift > 0 ? shift : 0;
-      a.sync[0] = gmax;
-      if (a.shift_out != nullptr) *a.shift_out = sh;
-      if (a.exp_out != nullptr)
-        *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
-    }
-    const bool trunc = a.trunc != 0;
-    const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
-    const bool same_layout = a.Cw == a.C;
+    if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
+  }
+  __syncthreads();
+  const uint32_t gmax = gshare;
+  const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    const int sh = shift > 0 ? shift : 0;
+    a.sync[0] = gmax;
+    if (a.shift_out != nullptr) *a.shift_out = sh;
+    if (a.exp_out != nullptr)
+      *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+  }
+  // phase 3: every wavefront rounds its columns and updates their weights (element counts fit 31 bits: host check)
+  const bool trunc = a.trunc != 0;
+  const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
+  const bool same_layout = a.Cw == a.C;
+  const uint32_t C = static_cast<uint32_t>(a.C), Cw = static_cast<uint32_t>(a.Cw);
 #pragma unroll
-    for (int v = 0; v < kFinishV; ++v) {
-      const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
-      if (col >= a.nv) continue;
-      const v4i s = sum[v];
-      if (a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
-      int r[4];
+  for (int j = 0; j < OWN; ++j) {
+    const int v = j * NW + wave;
+    if (v >= kFinishV) continue;
+    const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
+    if (col >= a.nv) continue;
+    const v4i s = fin[j];
+    if (a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
+    int r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
+      else r[e] = wrap_to_i8(s[e]);
+    }
+    const uint32_t e0 = static_cast<uint32_t>(col) * 4u;
+    const uint32_t rt = e0 / C;               // k * 9 + tap
+    const uint32_t c0 = e0 - rt * C;
+    uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
+    if (same_layout) {
+      const uint32_t wold = reinterpret_cast<const uint32_t*>(a.w)[col];
+      uint32_t gp = 0;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
-        else r[e] = wrap_to_i8(s[e]);
+        const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * e)) & 0xFFu));
+        wnew |= (static_cast<uint32_t>(clip127(wo - r[e])) & 0xFFu) << (8 * e);
+        gp |= (static_cast<uint32_t>(r[e]) & 0xFFu) << (8 * e);
       }
-      uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
-      if (same_layout) {
-        const uint32_t wold = reinterpret_cast<const uint32_t*>(a.w)[col];
-        uint32_t gp = 0;
+      reinterpret_cast<uint32_t*>(a.w)[col] = wnew;
+      if (a.g8 != nullptr) reinterpret_cast<uint32_t*>(a.g8)[col] = gp;
+    } else {
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * e)) & 0xFFu));
-          wnew |= (static_cast<uint32_t>(clip127(wo - r[e])) & 0xFFu) << (8 * e);
-          gp |= (static_cast<uint32_t>(r[e]) & 0xFFu) << (8 * e);
-        }
-        reinterpret_cast<uint32_t*>(a.w)[col] = wnew;
-        if (a.g8 != nullptr) reinterpret_cast<uint32_t*>(a.g8)[col] = gp;
-      } else {
-        const long long e0 = col * 4;
-        const long long row = e0 / a.C;
-        const int c0 = static_cast<int>(e0 - row * a.C);
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (c0 + e < a.Cw) {
-            const long long wi = row * a.Cw + c0 + e;
-            const int wn = clip127(static_cast<int>(a.w[wi]) - r[e]);
-            a.w[wi] = static_cast<int8_t>(wn);
-            wnew |= (static_cast<uint32_t>(wn) & 0xFFu) << (8 * e);
-            if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
-          }
+      for (int e = 0; e < 4; ++e) {
+        if (c0 + e < Cw) {
+          const uint32_t wi = rt * Cw + c0 + e;
+          const int wn = clip127(static_cast<int>(a.w[wi]) - r[e]);
+          a.w[wi] = static_cast<int8_t>(wn);
+          wnew |= (static_cast<uint32_t>(wn) & 0xFFu) << (8 * e);
+          if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
         }
       }
-      if (a.wprep != nullptr) {
-        // [64-channel group][32-channel slice][tap][64 rows][32 bytes], 16-byte halves swapped where (row >> 3) is odd
-        const long long e0 = col * 4;
-        const long long rt = e0 / a.C;                  // k * 9 + tap
-        const int c0 = static_cast<int>(e0 - rt * a.C);
-        const int k = static_cast<int>(rt / 9), tap = static_cast<int>(rt - static_cast<long long>(k) * 9);
-        const int row = k & 63, cs = c0 >> 5;
-        const int half = ((c0 >> 4) & 1) ^ ((row >> 3) & 1);
-        const long long dst = ((((static_cast<long long>(k >> 6) * ((a.C + 31) >> 5) + cs) * 9 + tap) * 64 + row) << 5) + half * 16 + (c0 & 15);
-        *reinterpret_cast<uint32_t*>(a.wprep + dst) = wnew;
-      }
+    }
+    if (a.wprep != nullptr) {
+      // [64-channel group][32-channel slice][tap][64 rows][32 bytes], 16-byte halves swapped where (row >> 3) is odd
+      const uint32_t k = rt / 9u, tap = rt - k * 9u;
+      const uint32_t row = k & 63u, cs = c0 >> 5;
+      const uint32_t half = ((c0 >> 4) & 1u) ^ ((row >> 3) & 1u);
+      const uint32_t dst = (((((k >> 6) * ((C + 31u) >> 5) + cs) * 9u + tap) * 64u + row) << 5) + half * 16u + (c0 & 15u);
+      *reinterpret_cast<uint32_t*>(a.wprep + dst) = wnew;
     }
   }
 }
@@ -781,15 +796,18 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
                            void* workspace, hipStream_t stream) {
   const int nb = wgrad3x3_finish_blocks(C, K);
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large for the single-pass finish", K, C);
-  static int resident = 0;
-  if (resident == 0) {
-    int dev = 0, cus = 0, per_cu = 0;
+  if (static_cast<long long>(K) * 9 * C >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large", K, C);
+  static int resident[2] = {0, 0};   // workgroups of 4 / 16 wavefronts the device holds at once
+  if (resident[0] == 0) {
+    int dev = 0, cus = 0, per4 = 0, per16 = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
-        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(wgrad_finish_kernel), 256, 0) != hipSuccess)
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per4, reinterpret_cast<const void*>(wgrad_finish_kernel<4>), 256, 0) != hipSuccess ||
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per16, reinterpret_cast<const void*>(wgrad_finish_kernel<16>), 1024, 0) != hipSuccess)
       return fail(NITI_ERR_LAUNCH, "wgrad_update: cannot query occupancy");
-    resident = cus * per_cu;
+    resident[0] = cus * per4;
+    resident[1] = cus * per16;
   }
-  if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: %d workgroups do not fit on the device at once (%d)", nb, resident);
+  if (nb > resident[0]) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: %d workgroups do not fit on the device at once (%d)", nb, resident[0]);
   WgradArgs a;
   int splits = 1;
   const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, workspace, a, splits, stream);
@@ -816,7 +834,9 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   f.exp_a = rq.exp_a;
   f.exp_b = rq.exp_b;
   f.exp_out = rq.exp_out;
-  hipLaunchKernelGGL(wgrad_finish_kernel, dim3(nb), dim3(256), 0, stream, f);
+  // many slices and few columns per workgroup: sixteen wavefronts share the slices
+  if (splits >= 32 && nb <= resident[1]) hipLaunchKernelGGL(wgrad_finish_kernel<16>, dim3(nb), dim3(1024), 0, stream, f);
+  else hipLaunchKernelGGL(wgrad_finish_kernel<4>, dim3(nb), dim3(256), 0, stream, f);
   return check_launch("wgrad_finish");
 }
 
