@@ -487,7 +487,10 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
         for (int q = 0; q < 4; ++q) v[q] &= static_cast<int>(positive_bytes(static_cast<uint32_t>(mk[q])));
       }
-      __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0);
+      // the 128-channel tile writes 64 bytes per pixel and wavefront: streaming stores start the write-back of the
+      // 16 MiB result while the kernel still runs (measured 2 us per launch); the 32-byte pieces of the 64-channel
+      // tile are slower that way
+      __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, KT == 128 ? 2 : 0);
     }
   }
 }
