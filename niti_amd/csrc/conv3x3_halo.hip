@@ -401,96 +401,136 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     __syncthreads();  // the tiles are dead from here on
     if (lane == 0) red[wave] = wmax;
     __syncthreads();
+    // Results are stored before the range is final: a first look at the slots (those of the workgroups that finished
+    // earlier, at least this one's own) gives a shift that is the final one unless a later workgroup raises the bit
+    // width; the int8 stores of all workgroups then overlap the wait for the last slots instead of following it in
+    // one burst.  When the final shift differs, the sums (still in registers) are rounded and stored once more.
+    const int nb = gridDim.x * gridDim.y;
+    uint32_t* const slots = a.sync + kSyncSlot0;
+    auto look = [&](bool& all) {   // wavefront 0: largest slot value seen (0 for none), and whether all are filled
+      bool ok = true;
+      uint32_t g = 0;
+      for (int i = lane; i < nb; i += 64) {
+        const uint32_t v = __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ok = ok && v != 0u;
+        g = v > g ? v : g;
+      }
+      all = __all(ok);
+      return wave_max_u32(g);
+    };
     if (wave == 0) {
       uint32_t bmax = lane < 8 ? red[lane] : 0u;
       bmax = wave_max_u32(bmax);
-      const int nb = gridDim.x * gridDim.y;
       const int b = blockIdx.y * gridDim.x + blockIdx.x;
-      uint32_t* const slots = a.sync + kSyncSlot0;
       if (lane == 0) __hip_atomic_store(&slots[b], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const long long t0 = wall_clock64();
-      uint32_t g = 0;
-      for (;;) {
-        bool ok = true;
-        g = 0;
-        for (int i = lane; i < nb; i += 64) {
-          const uint32_t v = __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          ok = ok && v != 0u;
-          g = v > g ? v : g;
-        }
-        if (__all(ok)) break;
-        if (wall_clock64() - t0 > a.spin_limit) {  // not every workgroup showed up: flag it and leave anyway
-          if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          break;
-        }
-        __builtin_amdgcn_s_sleep(4);
+      bool all;
+      const uint32_t g = max(look(all), bmax + 1u);   // the own slot may not be visible yet
+      if (lane == 0) {
+        red[8] = g - 1u;
+        red[9] = all ? 1u : 0u;
       }
-      g = wave_max_u32(g);
-      if (lane == 0) red[8] = g != 0u ? g - 1u : 0u;
     }
     __syncthreads();
-    const uint32_t gmax = red[8];
-    const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
-    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
-      const int sh = shift > 0 ? shift : 0;
-      a.sync[0] = gmax;
-      if (a.shift_out != nullptr) *a.shift_out = sh;
-      if (a.exp_out != nullptr)
-        *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
-    }
-    // ---- round, pack four channels per dword, transpose through a per-wavefront patch, store 16-byte pieces
+    int shift = bitwidth_of(red[8], a.bw_mode) - a.target_bits;
+    bool final_range = red[9] != 0u;
     const bool trunc = a.trunc != 0;
     const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
     const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
     constexpr int PROW = NWF * 32 + 16;  // the wavefront's channels of one pixel, padded
     int8_t* patch = smem + wave * (64 * PROW);
-    // the vector ALU work of this block is what the whole device does at this moment (every workgroup is here
-    // at the same time), so the common rounding mode gets a short form
-    const bool fast = shift >= 1 && !trunc && !psto;
-    const int sm1 = shift - 1, lo = relu ? 0 : -127;
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int i = 0; i < NWF; ++i)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          int r[4];
-#pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            int x = acc[i][j][4 * g + e];
-            if (rt) x = f32_roundtrip(x);
-            if (fast) {
-              r[e] = round_nearest_floor_fast(x, sm1, lo);
-            } else {
-              if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
-              else r[e] = wrap_to_i8(x);
-              if (relu && r[e] < 0) r[e] = 0;
-            }
-          }
-          *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = pack4_i8(r[0], r[1], r[2], r[3]);
-        }
-    // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y8, 0, a.y8_bytes, 0x00020000);
     constexpr int LPP = NWF * 2;       // lanes (16-byte pieces) per pixel
     constexpr int PPI = 64 / LPP;      // pixels per store instruction
     const int prow = lane / LPP, piece = lane % LPP;
     const int ch = chbase + piece * 16;
+    if (rt) {   // once, in place: the values are rounded up to twice below
 #pragma unroll
-    for (int t = 0; t < 64 / PPI; ++t) {
-      const int pl = t * PPI + prow;
-      v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
-      const int m = pixbase + wp_ * 64 + pl;
-      const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
-      if (a.mask != nullptr) {  // ReLU backward of the layer below, folded in: its output is this layer's input
-        const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
-        const auto mk = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
+      for (int i = 0; i < NWF; ++i)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] &= static_cast<int>(positive_bytes(static_cast<uint32_t>(mk[q])));
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+          for (int e = 0; e < 16; ++e) acc[i][j][e] = f32_roundtrip(acc[i][j][e]);
+    }
+#pragma nounroll
+    for (int pass = 0; pass < 2; ++pass) {
+      // the sums look modified to the compiler in every pass: nothing derived from them (magnitudes, signs) is
+      // computed ahead of the loop and kept in 64 more registers
+#pragma unroll
+      for (int i = 0; i < NWF; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[i][j]));
+      // round, pack four channels per dword, transpose through a per-wavefront patch, store 16-byte pieces; the
+      // common rounding mode gets a short form
+      const bool fast = shift >= 1 && !trunc && !psto;
+      const int sm1 = shift - 1, lo = relu ? 0 : -127;
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int i = 0; i < NWF; ++i)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            int r[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              const int x = acc[i][j][4 * g + e];
+              if (fast) {
+                r[e] = round_nearest_floor_fast(x, sm1, lo);
+              } else {
+                if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
+                else r[e] = wrap_to_i8(x);
+                if (relu && r[e] < 0) r[e] = 0;
+              }
+            }
+            *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = pack4_i8(r[0], r[1], r[2], r[3]);
+          }
+      // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
+#pragma unroll
+      for (int t = 0; t < 64 / PPI; ++t) {
+        const int pl = t * PPI + prow;
+        v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
+        const int m = pixbase + wp_ * 64 + pl;
+        const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
+        if (a.mask != nullptr) {  // ReLU backward of the layer below, folded in: its output is this layer's input
+          const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
+          const auto mk = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) v[q] &= static_cast<int>(positive_bytes(static_cast<uint32_t>(mk[q])));
+        }
+        // the 128-channel tile writes 64 bytes per pixel and wavefront: streaming stores start the write-back of the
+        // 16 MiB result while the kernel still runs (measured 2 us per launch); the 32-byte pieces of the 64-channel
+        // tile are slower that way
+        __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, KT == 128 ? 2 : 0);
       }
-      // the 128-channel tile writes 64 bytes per pixel and wavefront: streaming stores start the write-back of the
-      // 16 MiB result while the kernel still runs (measured 2 us per launch); the 32-byte pieces of the 64-channel
-      // tile are slower that way
-      __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, KT == 128 ? 2 : 0);
+      if (final_range) break;
+      // ---- wait for the slots of all workgroups; the maximum over them is the tensor's range
+      if (wave == 0) {
+        const long long t0 = wall_clock64();
+        uint32_t g = 0;
+        for (;;) {
+          bool all;
+          g = look(all);
+          if (all) break;
+          if (wall_clock64() - t0 > a.spin_limit) {  // not every workgroup showed up: flag it and leave anyway
+            if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+          __builtin_amdgcn_s_sleep(4);
+        }
+        if (lane == 0) red[8] = g != 0u ? g - 1u : 0u;
+      }
+      __syncthreads();
+      final_range = true;
+      const int fshift = bitwidth_of(red[8], a.bw_mode) - a.target_bits;
+      if (fshift == shift) break;
+      shift = fshift;
+      __builtin_amdgcn_s_waitcnt(0);   // the stores of the first pass leave before those that replace them
+    }
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
+      const int sh = shift > 0 ? shift : 0;
+      a.sync[0] = red[8];
+      if (a.shift_out != nullptr) *a.shift_out = sh;
+      if (a.exp_out != nullptr)
+        *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
     }
   }
 }

@@ -221,6 +221,37 @@ def test_conv_fprop_requant_f32_epilogue(dev):
         assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(a)
 
 
+@pytest.mark.parametrize("hot", [0, 3, 7])
+def test_conv_requant_range_set_by_one_tile(dev, hot):
+    """The single-launch kernels store results with the range seen so far and store again when a later workgroup
+    raises it: one image with large values among images of tiny ones makes most workgroups take that second pass."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = 8, 32, 64, 128
+    _say("conv_requant_range_set_by_one_tile", hot)
+    g = torch.Generator().manual_seed(5150 + hot)
+    x = ri8(g, N, Q, Q, C, lo=-1, hi=1)
+    x[hot] = ri8(g, Q, Q, C)
+    w = ri8(g, K, 3, 3, C)
+    acc = po.conv2d_fprop_i32(x, w, 1, 1)
+    for method in ("round", "psto"):
+        ref, sh_ref = po.act_calc(acc, 0, method)
+        for rep in range(3):     # the order in which workgroups finish differs from launch to launch
+            y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), method=method)
+            assert int(sync.cpu()[1]) == 0 and int(sync.cpu()[0]) == po.absmax(acc)
+            assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref
+    e = ri8(g, N, Q, Q, K, lo=-1, hi=1)
+    e[hot] = ri8(g, Q, Q, K)
+    dacc = co.conv_dgrad(e, w, Q, Q, 1, 1)
+    dref, dsh = po.err_calc(dacc)
+    mask = ri8(g, N, Q, Q, C)
+    for rep in range(3):
+        d8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), relu_mask=mask.to(dev))
+        assert int(sync.cpu()[1]) == 0 and int(sh.cpu()) == dsh
+        assert torch.equal(d8.cpu(), torch.where(mask > 0, dref, torch.zeros_like(dref)))
+
+
 @pytest.mark.parametrize("case", [(4, 8, 96, 48), (1, 16, 32, 16), (2, 16, 256, 128), (8, 32, 128, 128), (4, 8, 16, 32)])
 def test_conv_dgrad_requant(dev, case):
     from niti_amd import ops
