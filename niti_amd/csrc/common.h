@@ -68,13 +68,49 @@ __device__ inline int f32_roundtrip(int v) {
 
 __device__ inline uint32_t uabs(int v) { return v < 0 ? 0u - static_cast<uint32_t>(v) : static_cast<uint32_t>(v); }
 
+// Largest value over the wavefront, in every lane.  A max-scan inside each row of 16 lanes (row_shr 1, 2, 4, 8: lanes
+// without a source keep the neutral 0), then the row totals carried into the following rows (row_bcast 15 and 31),
+// which leaves the wavefront's maximum in lane 63: six data-parallel moves instead of six trips through the LDS
+// crossbar.
 __device__ inline uint32_t wave_max_u32(uint32_t v) {
+  uint32_t o;
+  o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x111, 0xf, 0xf, false));
+  v = o > v ? o : v;
+  o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x112, 0xf, 0xf, false));
+  v = o > v ? o : v;
+  o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x114, 0xf, 0xf, false));
+  v = o > v ? o : v;
+  o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x118, 0xf, 0xf, false));
+  v = o > v ? o : v;
+  o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x142, 0xa, 0xf, false));
+  v = o > v ? o : v;
+  o = static_cast<uint32_t>(__builtin_amdgcn_update_dpp(0, static_cast<int>(v), 0x143, 0xc, 0xf, false));
+  v = o > v ? o : v;
+  return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63));
+}
+
+// Called by a whole wavefront: the largest of the nb slot words (0 when none is filled) and whether all are filled.
+// A lane reads eight slots per round with the loads in flight together, so a round costs one trip to memory.
+__device__ inline uint32_t read_slots(const uint32_t* slots, int nb, bool& all) {
+  constexpr int kLook = 8;
+  const int lane = threadIdx.x & 63;
+  bool ok = true;
+  uint32_t g = 0;
+  for (int base = 0; base < nb; base += 64 * kLook) {
+    uint32_t v[kLook];
 #pragma unroll
-  for (int off = 32; off > 0; off >>= 1) {
-    uint32_t o = __shfl_xor(v, off, 64);
-    v = o > v ? o : v;
+    for (int u = 0; u < kLook; ++u) {
+      const int i = base + u * 64 + lane;
+      v[u] = i < nb ? __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1u;
+    }
+#pragma unroll
+    for (int u = 0; u < kLook; ++u) {
+      ok = ok && v[u] != 0u;
+      g = v[u] > g ? v[u] : g;
+    }
   }
-  return v;
+  all = __all(ok);
+  return wave_max_u32(g);
 }
 
 // Folds a wavefront's max |value| into *dst.  Same-address atomics serialise in the memory

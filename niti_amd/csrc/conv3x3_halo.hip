@@ -396,38 +396,38 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (wave == 0) fold_absmax(a.absmax, lane < 8 ? red[lane] : 0u);
     }
   } else {
-    // ---- tensor-wide range: workgroup maximum -> own slot -> wait for all slots -> maximum over the slots
+    // ---- tensor-wide range: workgroup maximum -> own slot -> maximum over the slots of all workgroups.
+    // Results are stored before the range is final: the slots filled so far (read before this workgroup's own
+    // maximum is known, so the latency hides behind that reduction) and the own maximum give a shift that is the
+    // final one unless another workgroup raises the bit width; the int8 stores of all workgroups then overlap the
+    // wait for the last slots instead of following it in one burst.  When the final shift differs, the sums (still
+    // in registers) are rounded and stored once more.
+    const int nb = gridDim.x * gridDim.y;
+    uint32_t* const slots = a.sync + kSyncSlot0;
+    constexpr int kLook = 8;   // slots a lane reads with its loads in flight together
+    auto look = [&](bool& all) { return read_slots(slots, nb, all); };   // wavefront 0
+    uint32_t early[kLook];   // a hint: the first 64 * kLook slots as they are now
+#pragma unroll
+    for (int u = 0; u < kLook; ++u) {
+      const int i = u * 64 + lane;
+      early[u] = (wave == 0 && i < nb) ? __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+    }
     const uint32_t wmax = wave_max_u32(lmax);
     __syncthreads();  // the tiles are dead from here on
     if (lane == 0) red[wave] = wmax;
     __syncthreads();
-    // Results are stored before the range is final: a first look at the slots (those of the workgroups that finished
-    // earlier, at least this one's own) gives a shift that is the final one unless a later workgroup raises the bit
-    // width; the int8 stores of all workgroups then overlap the wait for the last slots instead of following it in
-    // one burst.  When the final shift differs, the sums (still in registers) are rounded and stored once more.
-    const int nb = gridDim.x * gridDim.y;
-    uint32_t* const slots = a.sync + kSyncSlot0;
-    auto look = [&](bool& all) {   // wavefront 0: largest slot value seen (0 for none), and whether all are filled
-      bool ok = true;
-      uint32_t g = 0;
-      for (int i = lane; i < nb; i += 64) {
-        const uint32_t v = __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ok = ok && v != 0u;
-        g = v > g ? v : g;
-      }
-      all = __all(ok);
-      return wave_max_u32(g);
-    };
     if (wave == 0) {
       uint32_t bmax = lane < 8 ? red[lane] : 0u;
       bmax = wave_max_u32(bmax);
       const int b = blockIdx.y * gridDim.x + blockIdx.x;
       if (lane == 0) __hip_atomic_store(&slots[b], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      bool all;
-      const uint32_t g = max(look(all), bmax + 1u);   // the own slot may not be visible yet
+      uint32_t g = bmax + 1u;
+#pragma unroll
+      for (int u = 0; u < kLook; ++u) g = early[u] > g ? early[u] : g;
+      g = wave_max_u32(g);
       if (lane == 0) {
         red[8] = g - 1u;
-        red[9] = all ? 1u : 0u;
+        red[9] = nb == 1 ? 1u : 0u;
       }
     }
     __syncthreads();

@@ -571,21 +571,15 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
     const long long t0 = wall_clock64();
     uint32_t g = 0;
     for (;;) {
-      bool ok = true;
-      g = 0;
-      for (int i = lane; i < nb; i += 64) {
-        const uint32_t v = __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        ok = ok && v != 0u;
-        g = v > g ? v : g;
-      }
-      if (__all(ok)) break;
+      bool all;
+      g = read_slots(slots, nb, all);
+      if (all) break;
       if (wall_clock64() - t0 > a.spin_limit) {
         if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         break;
       }
       __builtin_amdgcn_s_sleep(4);
     }
-    g = wave_max_u32(g);
     if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
   }
   __syncthreads();
