@@ -300,7 +300,7 @@ def main():
             traffic = json.load(f).get("bytes_per_launch")
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic,
-                "kernel": "conv3x3_halo_kernel<..., true> (convolution + requantisation)", "launches": n_launch,
+                "kernel": "conv3x3_halo_kernel<..., true, *> (convolution + requantisation)", "launches": n_launch,
                 "avg_launch_us": round(k_ms * 1e3 / max(n_launch, 1), 2), "event_pair_overhead_us": round(pair_ms * 1e3, 2),
                 "ops_per_launch_avg": k_ops / max(n_launch, 1),
                 "note": "int8 multiply-accumulate counted as 2 ops; unit is tera-ops/s"}
