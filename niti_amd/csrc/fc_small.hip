@@ -194,8 +194,13 @@ __global__ __launch_bounds__(256) void fc_dgrad_requant_kernel(const FcArgs a) {
 
 // ---- weight gradient + update ---------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
-  __shared__ uint32_t err_t[kMaxOut][kWgradMaxM / 4];   // [o][sample / 4]: four consecutive samples' errors per word
-  __shared__ int red[3][kMaxOut * 4][64];
+  // one buffer used twice: the error words during the loop, the four wavefronts' sums after it
+  __shared__ __attribute__((aligned(16))) int smem_raw[4 * kMaxOut * 4 * 64];
+  __shared__ uint32_t wmax[4];
+  __shared__ uint32_t gshare;
+  static_assert(sizeof(uint32_t) * kMaxOut * (kWgradMaxM / 4) <= sizeof(smem_raw), "error words fit the buffer");
+  uint32_t (*err_t)[kWgradMaxM / 4] = reinterpret_cast<uint32_t (*)[kWgradMaxM / 4]>(smem_raw);   // [o][sample / 4]
+  int (*red)[kMaxOut * 4][64] = reinterpret_cast<int (*)[kMaxOut * 4][64]>(smem_raw);              // [wavefront][o * 4 + b][lane]
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int groups = (a.M + 3) >> 2;                      // groups of four samples
@@ -262,46 +267,57 @@ __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
     load(gb + 2 * kAhead, ra);
     mac(gb + kAhead, rb);
   }
-  if (wave > 0) {
+  __syncthreads();   // every wavefront is done with the error words
 #pragma unroll
-    for (int o = 0; o < kMaxOut; ++o)
+  for (int o = 0; o < kMaxOut; ++o)
 #pragma unroll
-      for (int b = 0; b < 4; ++b) red[wave - 1][o * 4 + b][lane] = acc[o][b];
-  }
+    for (int b = 0; b < 4; ++b) red[wave][o * 4 + b][lane] = acc[o][b];
   __syncthreads();
-  if (wave != 0) return;
+  // wavefront w completes, rounds and applies the output features w, w + 4, w + 8, w + 12
+  int fin[4][4];
   uint32_t lmax = 0;
 #pragma unroll
-  for (int o = 0; o < kMaxOut; ++o)
+  for (int j = 0; j < 4; ++j)
 #pragma unroll
     for (int b = 0; b < 4; ++b) {
-      acc[o][b] += red[0][o * 4 + b][lane] + red[1][o * 4 + b][lane] + red[2][o * 4 + b][lane];
-      const uint32_t u = uabs(acc[o][b]);
+      const int row = (4 * j + wave) * 4 + b;
+      fin[j][b] = red[0][row][lane] + red[1][row][lane] + red[2][row][lane] + red[3][row][lane];
+      const uint32_t u = uabs(fin[j][b]);
       lmax = u > lmax ? u : lmax;
     }
-  uint32_t wcur[kMaxOut];   // the weights this lane updates, fetched while the ranges are exchanged
+  uint32_t wcur[4];   // the weights this lane updates, fetched while the ranges are exchanged
 #pragma unroll
-  for (int o = 0; o < kMaxOut; ++o)
-    wcur[o] = (valid && o < a.O) ? *reinterpret_cast<const uint32_t*>(a.w + static_cast<long long>(o) * a.F + f) : 0u;
-  const uint32_t gmax = exchange_range(a, wave_max_u32(lmax));
+  for (int j = 0; j < 4; ++j) {
+    const int o = 4 * j + wave;
+    wcur[j] = (valid && o < a.O) ? *reinterpret_cast<const uint32_t*>(a.w + static_cast<long long>(o) * a.F + f) : 0u;
+  }
+  lmax = wave_max_u32(lmax);
+  if (lane == 0) wmax[wave] = lmax;
+  __syncthreads();
+  if (wave == 0) {
+    const uint32_t g = exchange_range(a, max(max(wmax[0], wmax[1]), max(wmax[2], wmax[3])));
+    if (lane == 0) gshare = g;
+  }
+  __syncthreads();
+  const uint32_t gmax = gshare;
   const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
-  if (blockIdx.x == 0 && lane == 0) write_scalars(a, gmax, shift);
+  if (blockIdx.x == 0 && threadIdx.x == 0) write_scalars(a, gmax, shift);
   if (!valid) return;
   const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC, trunc = a.trunc != 0;
 #pragma unroll
-  for (int o = 0; o < kMaxOut; ++o) {
+  for (int j = 0; j < 4; ++j) {
+    const int o = 4 * j + wave;
     if (o < a.O) {
-      uint32_t* pw = reinterpret_cast<uint32_t*>(a.w + static_cast<long long>(o) * a.F + f);
-      const uint32_t wold = wcur[o];
+      const uint32_t wold = wcur[j];
       int r[4];
       uint32_t wnew = 0;
 #pragma unroll
       for (int b = 0; b < 4; ++b) {
-        r[b] = round_to_i8(acc[o][b], shift, psto, trunc);
+        r[b] = round_to_i8(fin[j][b], shift, psto, trunc);
         const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * b)) & 0xFFu));
         wnew |= (static_cast<uint32_t>(clip127(wo - r[b])) & 0xFFu) << (8 * b);
       }
-      *pw = wnew;
+      *reinterpret_cast<uint32_t*>(a.w + static_cast<long long>(o) * a.F + f) = wnew;
       if (a.out8 != nullptr) *reinterpret_cast<uint32_t*>(a.out8 + static_cast<long long>(o) * a.F + f) = pack4_i8(r[0], r[1], r[2], r[3]);
     }
   }
