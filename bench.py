@@ -293,11 +293,15 @@ def main():
     k_ops = sum(o for (_, _, o) in wl.events)
     n_launch = len(wl.events)
     achieved = k_ops / (k_ms * 1e-3) / 1e12
+    # HBM bytes per launch of this kernel as the counters of an earlier rocprofv3 run gave them (the summary states
+    # the figure on a line of its own); null when the summary is not there
     traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    tpath = os.path.join(ROOT, "profiles", "conv_triple_hbm_traffic.txt")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get("bytes_per_launch")
+            for line in f:
+                if line.startswith("traffic_bytes_per_launch:"):
+                    traffic = int(line.split(":", 1)[1].split()[0])
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic,
                 "kernel": "conv3x3_halo_kernel<..., true, *> (convolution + requantisation)", "launches": n_launch,
