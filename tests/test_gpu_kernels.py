@@ -221,6 +221,68 @@ def test_conv_fprop_requant_f32_epilogue(dev):
         assert torch.equal(y.cpu(), ref) and int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(a)
 
 
+VGG_LAYERS = [(3, 128, 32), (128, 128, 32), (128, 256, 16), (256, 256, 16), (256, 512, 8), (512, 512, 8)]
+
+
+@pytest.mark.parametrize("layer", VGG_LAYERS)
+def test_conv_triple_at_benchmark_size(dev, layer):
+    """The six layer shapes of the benchmark at batch 128, where the CPU oracle would take minutes: checked through
+    what does not depend on size - the oracle on a few images of the batch (convolutions are per sample), the
+    adjoint identities <fprop(x,w),e> = <x,dgrad(e,w)> = <w,wgrad(x,e)> in 64-bit integers, additivity of the
+    weight gradient over the batch, and the single-launch forms against convolution + requantisation as two
+    launches (that chain is checked against the oracle at small sizes)."""
+    import torch.nn.functional as F
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    C, K, Q = layer
+    N = 128
+    _say("conv_triple_at_benchmark_size", layer)
+    g = torch.Generator().manual_seed(7000 + C + K + Q)
+    x, w = ri8(g, N, Q, Q, C), ri8(g, K, 3, 3, C)
+    e = torch.clamp(torch.round(torch.distributions.Laplace(0.0, 16.0).sample((N, Q, Q, K))), -127, 127).to(torch.int8)
+    x16 = (F.pad(x, (0, 16 - C % 16)) if C % 16 else x).contiguous()
+    w16 = (F.pad(w, (0, 16 - C % 16)) if C % 16 else w).contiguous()
+    xd, wd, ed, x16d, w16d = x.to(dev), w.to(dev), e.to(dev), x16.to(dev), w16.to(dev)
+    sub = [0, 77, 127]
+    # forward
+    am = ops.new_scalar_u32(dev)
+    y = ops.conv2d_fprop(x16d, w16d, 1, 1, absmax=am)
+    assert torch.equal(y[sub].cpu(), co.conv_fprop(x[sub].contiguous(), w, 1, 1))
+    assert int(am.cpu()) == int(y.abs().max())
+    y8, sh, sync = ops.conv2d_fprop_requant(x16d, w16d)
+    r8, rsh = ops.requant(y, am, 7, "round")
+    assert int(sync.cpu()[1]) == 0 and int(sync.cpu()[0]) == int(am.cpu())
+    assert torch.equal(y8, r8) and int(sh.cpu()) == int(rsh.cpu())
+    lhs = int((y.to(torch.int64) * ed.to(torch.int64)).sum())
+    # weight gradient
+    amw = ops.new_scalar_u32(dev)
+    dw = ops.conv2d_wgrad(x16d, ed, 3, 3, 1, 1, absmax=amw)[..., :C]
+    assert int((dw.to(torch.int64) * wd.to(torch.int64)).sum()) == lhs
+    half = ops.conv2d_wgrad(x16d[:64].contiguous(), ed[:64].contiguous(), 3, 3, 1, 1)[..., :C] + \
+        ops.conv2d_wgrad(x16d[64:].contiguous(), ed[64:].contiguous(), 3, 3, 1, 1)[..., :C]
+    assert torch.equal(dw, half)
+    one = ops.conv2d_wgrad(x16d[5:7].contiguous(), ed[5:7].contiguous(), 3, 3, 1, 1)[..., :C]
+    assert torch.equal(one.cpu(), co.conv_wgrad(x[5:7].contiguous(), e[5:7].contiguous(), 3, 3, 1, 1))
+    if C % 16 == 0:
+        wnew, wtwo = wd.clone(), wd.clone()
+        g8, _, sh, sync = ops.conv2d_wgrad_update(x16d, ed, wnew, mu=5, method="psto", want_grad=True)
+        g8two, shtwo = ops.grad_update(dw.contiguous(), wtwo, amw, 5, "psto", want_grad=True)
+        assert int(sync.cpu()[1]) == 0 and int(sync.cpu()[0]) == int(amw.cpu())
+        assert torch.equal(g8, g8two) and int(sh.cpu()) == int(shtwo.cpu()) and torch.equal(wnew, wtwo)
+        assert torch.equal(wnew.cpu(), po.weight_update(w, g8.cpu()))
+    # data gradient (the first layer has none)
+    if C % 16 == 0:
+        amd = ops.new_scalar_u32(dev)
+        dx = ops.conv2d_dgrad(ed, wd, 1, 1, absmax=amd)
+        assert torch.equal(dx[sub].cpu(), co.conv_dgrad(e[sub].contiguous(), w, Q, Q, 1, 1))
+        assert int((dx.to(torch.int64) * xd.to(torch.int64)).sum()) == lhs
+        wf = ops.conv_filter_prepare(wd, N, Q, Q)
+        d8, sh, sync = ops.conv2d_dgrad_requant(ed, wd, forward_filter=wf)
+        r8, rsh = ops.requant(dx, amd, 7, "round")
+        assert int(sync.cpu()[1]) == 0 and torch.equal(d8, r8) and int(sh.cpu()) == int(rsh.cpu())
+
+
 @pytest.mark.parametrize("hot", [0, 3, 7])
 def test_conv_requant_range_set_by_one_tile(dev, hot):
     """The single-launch kernels store results with the range seen so far and store again when a later workgroup
