@@ -61,6 +61,9 @@ class ConvTriple:
             e = laplace_i8(g, (BATCH, hw, hw, k))
             L = dict(c=c, k=k, hw=hw, x=x.to(dev), w=w.to(dev), err=e.to(dev))
             L["x16"] = F.pad(L["x"], (0, 16 - c % 16)).contiguous() if c % 16 else L["x"]
+            # requantisation shifts of the layer's forward and data-gradient results, kept from step to step
+            L["shift_f"] = torch.zeros(1, dtype=torch.int32, device=dev)
+            L["shift_d"] = torch.zeros(1, dtype=torch.int32, device=dev)
             self.layers.append(L)
         self.absmax = torch.zeros(3 * len(LAYERS), dtype=torch.int32, device=dev)
         # zeroed words the single-launch conv + requantisation kernels exchange their tile ranges through
@@ -102,8 +105,10 @@ class ConvTriple:
                 e0.record()
             so, sn = L["sync_f"]
             if sn:
+                # the shift of the previous step is handed in as the prediction for this one
                 ops.conv2d_fprop_requant(L["x16"], w16, 1, 1, f32_epilogue=True, sync=self.sync[so:so + sn], exp_a=self.exp0,
-                                         exp_b=self.exp0, exp_out=torch.empty_like(self.exp0), prepared_filter=wp)
+                                         exp_b=self.exp0, exp_out=torch.empty_like(self.exp0), prepared_filter=wp,
+                                         shift_out=L["shift_f"], shift_hint=True)
             else:
                 acc = ops.conv2d_fprop(L["x16"], w16, 1, 1, f32_epilogue=True, absmax=am[0:1], prepared_filter=wp)
             if record:
@@ -121,7 +126,7 @@ class ConvTriple:
                     e0.record()
                 if sn:
                     ops.conv2d_dgrad_requant(L["err"], L["w"], 1, 1, f32_epilogue=True, sync=self.sync[so:so + sn],
-                                             forward_filter=wp)
+                                             forward_filter=wp, shift_out=L["shift_d"], shift_hint=True)
                 else:
                     dx = ops.conv2d_dgrad(L["err"], L["w"], 1, 1, f32_epilogue=True, absmax=am[1:2], prepared_filter=wt)
                 if record:

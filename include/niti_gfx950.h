@@ -41,6 +41,10 @@ enum {
                                             the same filter (the one the forward pass reads) */
 /* requant flags */
 #define NITI_RQ_RELU 1u /* clamp the int8 result at 0 (TiReLU.forward, ti_torch.py:272-279) */
+#define NITI_RQ_SHIFT_HINT 2u /* niti_conv2d_i8_*_requant: *shift_out holds a predicted shift on entry (the same
+                                 tensor's shift of the previous training step).  The kernels store results before the
+                                 tensor's range is final and store again if the shift turns out different; a good
+                                 prediction saves that second pass.  The results do not depend on it. */
 
 /* rounding method (ti_torch.py:23-69) / division meaning / bit-width evaluation / pool ties */
 enum { NITI_ROUND_NEAREST = 0, NITI_ROUND_STOCHASTIC = 1, NITI_ROUND_PSEUDO_STOCHASTIC = 2 };
@@ -124,7 +128,7 @@ int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N,
  * can only happen when other work keeps part of the device busy that long.  Launches that share a sync buffer
  * must not overlap.
  * flags: NITI_EPI_F32_ROUNDTRIP, NITI_CONV_FILTER_PREPARED (w is a copy made by niti_conv2d_i8_filter_prepare;
- * otherwise workspace must hold niti_conv2d_i8_filter_workspace bytes).  rq_flags: NITI_RQ_RELU.
+ * otherwise workspace must hold niti_conv2d_i8_filter_workspace bytes).  rq_flags: NITI_RQ_RELU, NITI_RQ_SHIFT_HINT.
  * shift_out / exp_a / exp_b / exp_out as in niti_requant_i32_i8 (each may be NULL).
  * relu_mask (data gradient only, may be NULL): int8 [N,H,W,C] like dx8; elements whose mask byte is not positive
  * are stored as zero AFTER the range and the rounding were taken from the unmasked sums.  Passing the layer's

@@ -15,6 +15,7 @@ EPI_F32_ROUNDTRIP = 1
 CONV_FILTER_PREPARED = 2
 CONV_FILTER_FORWARD_COPY = 4
 RQ_RELU = 1
+RQ_SHIFT_HINT = 2
 ROUND = {"round": 0, "sto": 1, "psto": 2}
 DIV = {"floor": 0, "trunc": 1}
 BW = {"int": 0, "f32": 1}

@@ -406,6 +406,10 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     uint32_t* const slots = a.sync + kSyncSlot0;
     constexpr int kLook = 8;   // slots a lane reads with its loads in flight together
     auto look = [&](bool& all) { return read_slots(slots, nb, all); };   // wavefront 0
+    // NITI_RQ_SHIFT_HINT: *shift_out holds the caller's prediction (the previous training step's shift of this
+    // tensor).  Read before this workgroup fills its slot: workgroup (0, 0) overwrites the word only after all slots
+    // are filled.
+    const int predicted = ((a.rq_flags & NITI_RQ_SHIFT_HINT) != 0 && a.shift_out != nullptr && wave == 0) ? *a.shift_out : 0;
     uint32_t early[kLook];   // a hint: the first 64 * kLook slots as they are now
 #pragma unroll
     for (int u = 0; u < kLook; ++u) {
@@ -428,11 +432,15 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (lane == 0) {
         red[8] = g - 1u;
         red[9] = nb == 1 ? 1u : 0u;
+        red[10] = static_cast<uint32_t>(predicted);
       }
     }
     __syncthreads();
-    int shift = bitwidth_of(red[8], a.bw_mode) - a.target_bits;
+    // a shift below 1 means "no shift" whatever its value; the prediction counts unless this workgroup's own sums or
+    // the slots seen so far already need more (or the range is final already)
+    int shift = max(bitwidth_of(red[8], a.bw_mode) - a.target_bits, 0);
     bool final_range = red[9] != 0u;
+    if (!final_range) shift = max(shift, static_cast<int>(red[10]));
     const bool trunc = a.trunc != 0;
     const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
     const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
@@ -520,7 +528,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       }
       __syncthreads();
       final_range = true;
-      const int fshift = bitwidth_of(red[8], a.bw_mode) - a.target_bits;
+      const int fshift = max(bitwidth_of(red[8], a.bw_mode) - a.target_bits, 0);
       if (fshift == shift) break;
       shift = fshift;
       __builtin_amdgcn_s_waitcnt(0);   // the stores of the first pass leave before those that replace them

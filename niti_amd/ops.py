@@ -113,7 +113,8 @@ def conv_requant_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1, dgrad=
 
 
 def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epilogue, target_bits, method, div_mode,
-                  bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None, forward_filter=None):
+                  bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None, forward_filter=None,
+                  shift_hint=False):
     _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask, forward_filter)
     if relu_mask is not None and (relu_mask.dtype != torch.int8 or tuple(relu_mask.shape) != tuple(out_shape)):
         raise RuntimeError("%s: relu_mask must be int8 and shaped like the output" % entry)
@@ -131,6 +132,8 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
         raise RuntimeError("%s: sync must be a zeroed int32 tensor of at least %d words" % (entry, words))
     y = torch.empty(out_shape, dtype=torch.int8, device=x.device)
     if shift_out is None:
+        if shift_hint:
+            raise RuntimeError("%s: shift_hint needs shift_out, holding the predicted shift" % entry)
         shift_out = torch.empty(1, dtype=torch.int32, device=x.device)
     flags = _flags(f32_epilogue)
     if forward_filter is not None:
@@ -142,7 +145,7 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
         ws = torch.empty(max(nbytes, 16), dtype=torch.int8, device=x.device)
         wptr = _ptr(w)
     head = (_ptr(x), wptr, _ptr(y), N, H, W, C, K, R, S, stride, padding, flags, target_bits, L.ROUND[method],
-            L.DIV[div_mode], L.BW[bw_mode], L.RQ_RELU if relu else 0)
+            L.DIV[div_mode], L.BW[bw_mode], (L.RQ_RELU if relu else 0) | (L.RQ_SHIFT_HINT if shift_hint else 0))
     tail = (_ptr(sync), sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes, _stream(x))
     st = getattr(L.lib(), entry)(*(head + ((_ptr(relu_mask),) if dgrad else ()) + tail))
     L.check(st, entry)
@@ -151,10 +154,12 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
 
 def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", relu=False, sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None):
+                         prepared_filter=None, shift_hint=False):
     """conv2d_fprop + requant as one launch: x [N,H,W,C] int8, w [K,R,S,C] int8 -> ([N,P,Q,K] int8, device shift,
     sync).  sync[0] holds max|sum| afterwards, sync[1] != 0 flags a timed-out wait (invalid output).  ``sync``, if
-    given, must hold conv_requant_sync_words(...) zeroed int32 words."""
+    given, must hold conv_requant_sync_words(...) zeroed int32 words.  ``shift_hint``: ``shift_out`` holds a
+    predicted shift on entry (e.g. this tensor's shift of the previous training step); a good prediction saves the
+    kernel a second store pass, the results do not depend on it."""
     N, H, W, C = x.shape
     K, R, S, C2 = w.shape
     if C2 != C:
@@ -163,12 +168,12 @@ def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_b
     Q = (W + 2 * padding - S) // stride + 1
     return _conv_requant("niti_conv2d_i8_fprop_requant", False, x, w, (N, P, Q, K), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter)
+                         prepared_filter, shift_hint=shift_hint)
 
 
 def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None, relu_mask=None, forward_filter=None):
+                         prepared_filter=None, relu_mask=None, forward_filter=None, shift_hint=False):
     """conv2d_dgrad + requant as one launch: err [N,P,Q,K] int8, w [K,R,S,C] int8 -> ([N,H,W,C] int8, shift, sync).
     ``relu_mask`` (int8 [N,H,W,C]): results whose mask element is not positive are stored as zero, after range
     and rounding were taken from the unmasked sums (the backward pass of a ReLU in front of the layer).
@@ -181,7 +186,7 @@ def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target
     W = Q - 2 * padding + S - 1
     return _conv_requant("niti_conv2d_i8_dgrad_requant", True, err, w, (N, H, W, C), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, False, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter, relu_mask, forward_filter)
+                         prepared_filter, relu_mask, forward_filter, shift_hint)
 
 
 _scratch = {}

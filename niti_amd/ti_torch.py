@@ -190,7 +190,7 @@ _fused_refused = set()       # (dgrad, input shape, filter shape, stride, paddin
 
 
 def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None, prepared_filter=None,
-                        forward_filter=None):
+                        forward_filter=None, shift_state=None):
     """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
     exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
     single-launch kernel, or more workgroups than the device holds at once."""
@@ -210,6 +210,8 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
     exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
     call = ops.conv2d_dgrad_requant if dgrad else ops.conv2d_fprop_requant
     kw = dict(relu=relu, prepared_filter=prepared_filter) if not dgrad else dict(relu_mask=relu_mask, forward_filter=forward_filter)
+    if shift_state is not None:     # the tensor's shift of the previous step: the kernel's prediction for this one
+        kw.update(shift_out=shift_state, shift_hint=True)
     try:
         y, shift, _ = call(x, w, stride, padding, f32_epilogue=F32_EPILOGUE, target_bits=BITWIDTH, method=method,
                            div_mode=DIV_MODE, bw_mode=BW_MODE, exp_a=exp_a, exp_b=exp_b, exp_out=exp_out, **kw)
@@ -371,7 +373,8 @@ class TiConv2d(UpdateWeight):
         w16 = _pad_channels16(self.weight).contiguous()
         exp_a, exp_b = _exp_tensor(self.act_in_exp, dev), self._wexp()
         fused = _conv_requant_fused(False, self.act16, w16, self.stride, self.padding, ACT_ROUND_METHOD, rand,
-                                    self.fuse_relu, exp_a, exp_b, prepared_filter=self._forward_filter(w16))
+                                    self.fuse_relu, exp_a, exp_b, prepared_filter=self._forward_filter(w16),
+                                    shift_state=self._shift_state("act", dev))
         if fused is not None:
             return fused[0], fused[2]
         am = ops.new_scalar_u32(dev)
@@ -415,6 +418,15 @@ class TiConv2d(UpdateWeight):
         if not self.first_layer:
             return err_out, self.err_exp
 
+    def _shift_state(self, which, device):
+        """1-element int32 device tensor that keeps the requantisation shift of this layer's activations ("act") or
+        errors ("err") from one step to the next; the single-launch kernels take it as their prediction."""
+        states = self.__dict__.setdefault("_shift_states", {})
+        key = (which, str(device))
+        if key not in states:
+            states[key] = torch.zeros(1, dtype=torch.int32, device=device)
+        return states[key]
+
     def _dgrad_filter(self):
         """The forward pass's kernel-ready filter copy, which the data gradient can read in place of a copy of its
         own while it matches the weights, or None."""
@@ -425,7 +437,8 @@ class TiConv2d(UpdateWeight):
     def _data_gradient(self, err_in, rand, mask, forward_filter):
         """err_calc(conv_dgrad(err_in, weight)) (ti_torch.py:422-427), the ReLU mask applied; -> (int8 error, exponent)."""
         fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
-                                    False, self.err_exp_in, self._wexp(), relu_mask=mask, forward_filter=forward_filter)
+                                    False, self.err_exp_in, self._wexp(), relu_mask=mask, forward_filter=forward_filter,
+                                    shift_state=self._shift_state("err", err_in.device))
         if fused is not None:
             err_out, _, new_exp = fused
             return err_out, new_exp

@@ -283,6 +283,34 @@ def test_conv_triple_at_benchmark_size(dev, layer):
         assert int(sync.cpu()[1]) == 0 and torch.equal(d8, r8) and int(sh.cpu()) == int(rsh.cpu())
 
 
+@pytest.mark.parametrize("case", [(8, 32, 64, 128), (16, 8, 256, 64), (4, 16, 32, 48)])
+def test_conv_requant_predicted_shift(dev, case):
+    """A predicted shift (right, too small, too large, absurd) changes how often the kernel stores, never what."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_requant_predicted_shift", case)
+    g = torch.Generator().manual_seed(8200 + C + K)
+    x, w, e = ri8(g, N, Q, Q, C), ri8(g, K, 3, 3, C), ri8(g, N, Q, Q, K)
+    acc = po.conv2d_fprop_i32(x, w, 1, 1)
+    ref, sh_ref = po.act_calc(acc, 0)
+    dacc = co.conv_dgrad(e, w, Q, Q, 1, 1)
+    dref, dsh = po.err_calc(dacc)
+    for guess in (sh_ref, sh_ref - 1, sh_ref + 1, 0, 31):
+        so = torch.tensor([max(guess, 0)], dtype=torch.int32, device=dev)
+        y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), shift_out=so, shift_hint=True)
+        assert sh is so and int(sync.cpu()[1]) == 0
+        assert torch.equal(y.cpu(), ref) and int(so.cpu()) == sh_ref
+        so = torch.tensor([max(guess, 0)], dtype=torch.int32, device=dev)
+        d8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), shift_out=so, shift_hint=True)
+        assert torch.equal(d8.cpu(), dref) and int(so.cpu()) == dsh
+    # all-zero input: no shift at all, whatever was predicted
+    so = torch.tensor([5], dtype=torch.int32, device=dev)
+    y, sh, sync = ops.conv2d_fprop_requant(torch.zeros_like(x).to(dev), w.to(dev), shift_out=so, shift_hint=True)
+    assert int(y.abs().max()) == 0 and int(so.cpu()) == 0
+
+
 @pytest.mark.parametrize("hot", [0, 3, 7])
 def test_conv_requant_range_set_by_one_tile(dev, hot):
     """The single-launch kernels store results with the range seen so far and store again when a later workgroup
