@@ -268,7 +268,7 @@ int niti_maxpool_i8_bwd(const int8_t* y, const int8_t* dy, const int8_t* x, int8
  *   wgrad_update:  g = grad_calc(err^T * act), w = clip(w - g)  (ti_torch.py:263-265, 16-21); g8_out optional
  * `which` names the pass for the sync query, which returns 0 for shapes these kernels do not cover (then use
  * niti_gemm_i8 + niti_requant_i32_i8 / niti_grad_update_i8).  sync: zeroed uint32 words as for the convolutions
- * (word 0 range out, word 1 time-out flag, one slot per workgroup from word 16).
+ * (word 0 range out, word 1 time-out flag, one slot per workgroup from word 16, four words apart).
  * Rounding NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC; shift_out / exp_* as in niti_requant_i32_i8.
  */
 enum { NITI_FC_FORWARD = 0, NITI_FC_DGRAD = 1, NITI_FC_WGRAD = 2 };

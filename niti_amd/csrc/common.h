@@ -6,6 +6,10 @@
 
 #include "niti_gfx950.h"
 
+#ifndef NITI_SLOT_STRIDE
+#define NITI_SLOT_STRIDE 4
+#endif
+
 namespace niti {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
@@ -89,27 +93,49 @@ __device__ inline uint32_t wave_max_u32(uint32_t v) {
   return static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(v), 63));
 }
 
-// Called by a whole wavefront: the largest of the nb slot words (0 when none is filled) and whether all are filled.
-// A lane reads eight slots per round with the loads in flight together, so a round costs one trip to memory.
-__device__ inline uint32_t read_slots(const uint32_t* slots, int nb, bool& all) {
+// Range exchange between the resident workgroups of a launch: workgroup b stores (its maximum + 1) in slot b and
+// reads all slots.  Slots are kSlotStride words apart: the 4-byte stores of all workgroups arrive within a
+// microsecond and are serialised per memory channel, so the slots are spread over more of them.
+constexpr int kSlotStride = NITI_SLOT_STRIDE;
+__device__ inline uint32_t* slot_word(uint32_t* slots, int b) { return slots + static_cast<long long>(b) * kSlotStride; }
+inline size_t slot_words(int blocks) { return static_cast<size_t>((blocks + 15) / 16 * 16) * kSlotStride; }
+
+// Called by a whole wavefront: waits until all nb slots are filled and returns the largest value.  512 slots at a
+// time, eight per lane with the loads in flight together (one trip to memory per look); a lane reads a slot again
+// only while it is still empty, so the reads of the waiting workgroups die down as the slots fill.  Gives up after
+// spin_limit ticks of the 100 MHz clock: *timed_out is set to 1 and the largest value seen so far is returned.
+__device__ inline uint32_t wait_slots(uint32_t* slots, int nb, long long spin_limit, uint32_t* timed_out) {
   constexpr int kLook = 8;
   const int lane = threadIdx.x & 63;
-  bool ok = true;
+  const long long t0 = wall_clock64();
   uint32_t g = 0;
-  for (int base = 0; base < nb; base += 64 * kLook) {
+  bool gave_up = false;
+  for (int base = 0; base < nb && !gave_up; base += 64 * kLook) {
     uint32_t v[kLook];
 #pragma unroll
-    for (int u = 0; u < kLook; ++u) {
-      const int i = base + u * 64 + lane;
-      v[u] = i < nb ? __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 1u;
+    for (int u = 0; u < kLook; ++u) v[u] = base + u * 64 + lane < nb ? 0u : 1u;
+    for (;;) {
+      uint32_t t[kLook];
+#pragma unroll
+      for (int u = 0; u < kLook; ++u)
+        t[u] = v[u] == 0u ? __hip_atomic_load(slot_word(slots, base + u * 64 + lane), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : v[u];
+      bool ok = true;
+#pragma unroll
+      for (int u = 0; u < kLook; ++u) {
+        v[u] = t[u];
+        ok = ok && v[u] != 0u;
+      }
+      if (__all(ok)) break;
+      if (wall_clock64() - t0 > spin_limit) {
+        if (lane == 0) __hip_atomic_store(timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        gave_up = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(8);
     }
 #pragma unroll
-    for (int u = 0; u < kLook; ++u) {
-      ok = ok && v[u] != 0u;
-      g = v[u] > g ? v[u] : g;
-    }
+    for (int u = 0; u < kLook; ++u) g = v[u] > g ? v[u] : g;
   }
-  all = __all(ok);
   return wave_max_u32(g);
 }
 

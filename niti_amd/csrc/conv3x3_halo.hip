@@ -405,7 +405,6 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const int nb = gridDim.x * gridDim.y;
     uint32_t* const slots = a.sync + kSyncSlot0;
     constexpr int kLook = 8;   // slots a lane reads with its loads in flight together
-    auto look = [&](bool& all) { return read_slots(slots, nb, all); };   // wavefront 0
     // NITI_RQ_SHIFT_HINT: *shift_out holds the caller's prediction (the previous training step's shift of this
     // tensor).  Read before this workgroup fills its slot: workgroup (0, 0) overwrites the word only after all slots
     // are filled.
@@ -414,7 +413,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
     for (int u = 0; u < kLook; ++u) {
       const int i = u * 64 + lane;
-      early[u] = (wave == 0 && i < nb) ? __hip_atomic_load(&slots[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+      early[u] = (wave == 0 && i < nb) ? __hip_atomic_load(slot_word(slots, i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
     }
     const uint32_t wmax = wave_max_u32(lmax);
     __syncthreads();  // the tiles are dead from here on
@@ -424,7 +423,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       uint32_t bmax = lane < 8 ? red[lane] : 0u;
       bmax = wave_max_u32(bmax);
       const int b = blockIdx.y * gridDim.x + blockIdx.x;
-      if (lane == 0) __hip_atomic_store(&slots[b], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) __hip_atomic_store(slot_word(slots, b), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       uint32_t g = bmax + 1u;
 #pragma unroll
       for (int u = 0; u < kLook; ++u) g = early[u] > g ? early[u] : g;
@@ -512,18 +511,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (final_range) break;
       // ---- wait for the slots of all workgroups; the maximum over them is the tensor's range
       if (wave == 0) {
-        const long long t0 = wall_clock64();
-        uint32_t g = 0;
-        for (;;) {
-          bool all;
-          g = look(all);
-          if (all) break;
-          if (wall_clock64() - t0 > a.spin_limit) {  // not every workgroup showed up: flag it and leave anyway
-            if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            break;
-          }
-          __builtin_amdgcn_s_sleep(4);
-        }
+        const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
         if (lane == 0) red[8] = g != 0u ? g - 1u : 0u;
       }
       __syncthreads();
@@ -697,7 +685,7 @@ int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S,
   return nb <= 2048 ? static_cast<int>(nb) : 0;  // the device check happens at launch; this bounds the workspace
 }
 
-size_t conv3x3_halo_sync_words(int blocks) { return static_cast<size_t>(kSyncSlot0 + (blocks + 15) / 16 * 16); }
+size_t conv3x3_halo_sync_words(int blocks) { return static_cast<size_t>(kSyncSlot0) + slot_words(blocks); }
 
 int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, int N, int H, int C, int K, unsigned flags,
                                 uint32_t* sync, const RequantSpec& rq, hipStream_t stream) {

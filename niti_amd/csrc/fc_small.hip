@@ -56,19 +56,8 @@ __device__ inline uint32_t exchange_range(const FcArgs& a, uint32_t bmax) {
   const int lane = threadIdx.x & 63;
   const int nb = gridDim.x;
   uint32_t* const slots = a.sync + kSlot0;
-  if (lane == 0) __hip_atomic_store(&slots[blockIdx.x], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const long long t0 = wall_clock64();
-  uint32_t g = 0;
-  for (;;) {
-    bool all;
-    g = read_slots(slots, nb, all);
-    if (all) break;
-    if (wall_clock64() - t0 > a.spin_limit) {   // not every workgroup showed up: flag it and leave anyway
-      if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      break;
-    }
-    __builtin_amdgcn_s_sleep(4);
-  }
+  if (lane == 0) __hip_atomic_store(slot_word(slots, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
   return g != 0u ? g - 1u : 0u;
 }
 
@@ -362,7 +351,7 @@ using namespace niti;
 extern "C" size_t niti_fc_i8_sync_words(int which, int M, int O, int F) {
   const long long nb = blocks_of(which, M, O, F);
   if (nb == 0) return 0;
-  return static_cast<size_t>(kSlot0 + (nb + 15) / 16 * 16);
+  return static_cast<size_t>(kSlot0) + slot_words(static_cast<int>(nb));
 }
 
 static int fc_common(const char* who, int which, FcArgs& a, int M, int O, int F, int target_bits, int method, int div_mode,

@@ -567,19 +567,8 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
     bmax = wave_max_u32(bmax);
     const int nb = gridDim.x;
     uint32_t* const slots = a.sync + kFinishSlot0;
-    if (lane == 0) __hip_atomic_store(&slots[blockIdx.x], bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const long long t0 = wall_clock64();
-    uint32_t g = 0;
-    for (;;) {
-      bool all;
-      g = read_slots(slots, nb, all);
-      if (all) break;
-      if (wall_clock64() - t0 > a.spin_limit) {
-        if (lane == 0) __hip_atomic_store(&a.sync[1], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        break;
-      }
-      __builtin_amdgcn_s_sleep(4);
-    }
+    if (lane == 0) __hip_atomic_store(slot_word(slots, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
     if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
   }
   __syncthreads();
@@ -783,7 +772,7 @@ int wgrad3x3_finish_blocks(int C, int K) {
   return static_cast<int>(nb < 1 ? 1 : nb);
 }
 
-size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0 + (blocks + 15) / 16 * 16); }
+size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0) + slot_words(blocks); }
 
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
                            bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
