@@ -64,6 +64,7 @@ class ConvTriple:
             # requantisation shifts of the layer's forward and data-gradient results, kept from step to step
             L["shift_f"] = torch.zeros(1, dtype=torch.int32, device=dev)
             L["shift_d"] = torch.zeros(1, dtype=torch.int32, device=dev)
+            L["shift_w"] = torch.zeros(1, dtype=torch.int32, device=dev)
             self.layers.append(L)
         self.absmax = torch.zeros(3 * len(LAYERS), dtype=torch.int32, device=dev)
         # zeroed words the single-launch conv + requantisation kernels exchange their tile ranges through
@@ -138,7 +139,8 @@ class ConvTriple:
             so, sn = L["sync_w"]
             if sn:
                 ops.conv2d_wgrad_update(L["x16"], L["err"], L["w"], 1, 1, f32_epilogue=(i > 0), mu=5, method="psto",
-                                        sync=self.sync[so:so + sn], workspace=self.ws, prepared_filter=L["wp"])
+                                        sync=self.sync[so:so + sn], workspace=self.ws, prepared_filter=L["wp"],
+                                        shift_out=L["shift_w"], shift_hint=True)
             else:
                 L["wp"] = None
                 dw = ops.conv2d_wgrad(L["x16"], L["err"], 3, 3, 1, 1, f32_epilogue=(i > 0), absmax=am[2:3], workspace=self.ws)

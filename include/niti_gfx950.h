@@ -36,6 +36,8 @@ enum {
                                      (pytorch/cutlass-extension/cutlassconv_kernel.cu:78-85) */
 #define NITI_CONV_FILTER_PREPARED 2u /* fprop / dgrad: `w` already is the kernel-ready filter copy written
                                         by niti_conv2d_i8_filter_prepare for the same shape; no workspace */
+#define NITI_CONV_SHIFT_HINT 8u /* niti_conv2d_i8_wgrad_update only: *shift_out holds a predicted shift on entry, see
+                                   NITI_RQ_SHIFT_HINT */
 #define NITI_CONV_FILTER_FORWARD_COPY 4u /* data gradient only, with NITI_CONV_FILTER_PREPARED: `w` is the
                                             copy that niti_conv2d_i8_filter_prepare(.., dgrad = 0) made of
                                             the same filter (the one the forward pass reads) */

@@ -14,6 +14,7 @@ OK = 0
 EPI_F32_ROUNDTRIP = 1
 CONV_FILTER_PREPARED = 2
 CONV_FILTER_FORWARD_COPY = 4
+CONV_SHIFT_HINT = 8
 RQ_RELU = 1
 RQ_SHIFT_HINT = 2
 ROUND = {"round": 0, "sto": 1, "psto": 2}

@@ -503,6 +503,7 @@ struct FinishArgs {
   int8_t* wprep;       // optional: the halo convolution kernel's forward copy of the [K][9][C] filter, kept in step with w
   uint32_t* sync;      // word 0: max |sum| (output); word 1: wait gave up; words kFinishSlot0..: slots, zero on entry
   int roundtrip, target_bits, method, trunc, bw_mode;
+  int predict;         // *shift_out holds a predicted shift on entry
   long long spin_limit;
   int32_t* shift_out;
   const int32_t* exp_a;
@@ -518,6 +519,8 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
   __shared__ uint32_t gshare;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  // read before this workgroup fills its slot: workgroup 0 overwrites the word only after all slots are filled
+  const int predicted = (a.predict != 0 && a.shift_out != nullptr) ? max(*a.shift_out, 0) : 0;
   v4i sum[kFinishV];
   // phase 1: every wavefront adds its share of the slices for all of the workgroup's columns
 #pragma unroll
@@ -561,80 +564,99 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
   lmax = wave_max_u32(lmax);
   if (lane == 0) wmax[wave] = lmax;
   __syncthreads();
-  if (wave == 0) {
-    uint32_t bmax = 0;
-    for (int w = lane; w < NW; w += 64) bmax = max(bmax, wmax[w]);
-    bmax = wave_max_u32(bmax);
-    const int nb = gridDim.x;
-    uint32_t* const slots = a.sync + kFinishSlot0;
-    if (lane == 0) __hip_atomic_store(slot_word(slots, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
-    if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
-  }
-  __syncthreads();
-  const uint32_t gmax = gshare;
-  const int shift = bitwidth_of(gmax, a.bw_mode) - a.target_bits;
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    const int sh = shift > 0 ? shift : 0;
-    a.sync[0] = gmax;
-    if (a.shift_out != nullptr) *a.shift_out = sh;
-    if (a.exp_out != nullptr)
-      *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
-  }
-  // phase 3: every wavefront rounds its columns and updates their weights (element counts fit 31 bits: host check)
+  uint32_t bmax = 0;   // the workgroup's largest magnitude, in every wavefront
+#pragma unroll
+  for (int w = 0; w < NW; ++w) bmax = max(bmax, wmax[w]);
+  if (wave == 0 && lane == 0)
+    __hip_atomic_store(slot_word(a.sync + kFinishSlot0, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  // phase 3: every wavefront rounds its columns and updates their weights (element counts fit 31 bits: host check).
+  // With a predicted shift (a.predict) the update is applied before the range is final, so that its stores overlap
+  // the wait for the other workgroups, and applied once more from the same old weights if the final shift differs.
   const bool trunc = a.trunc != 0;
   const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
   const bool same_layout = a.Cw == a.C;
   const uint32_t C = static_cast<uint32_t>(a.C), Cw = static_cast<uint32_t>(a.Cw);
+  uint32_t wold[OWN];
 #pragma unroll
   for (int j = 0; j < OWN; ++j) {
     const int v = j * NW + wave;
-    if (v >= kFinishV) continue;
     const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
-    if (col >= a.nv) continue;
-    const v4i s = fin[j];
-    if (a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
-    int r[4];
+    wold[j] = (same_layout && v < kFinishV && col < a.nv) ? reinterpret_cast<const uint32_t*>(a.w)[col] : 0u;
+  }
+  auto apply = [&](int shift, bool first) {
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
-      else r[e] = wrap_to_i8(s[e]);
-    }
-    const uint32_t e0 = static_cast<uint32_t>(col) * 4u;
-    const uint32_t rt = e0 / C;               // k * 9 + tap
-    const uint32_t c0 = e0 - rt * C;
-    uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
-    if (same_layout) {
-      const uint32_t wold = reinterpret_cast<const uint32_t*>(a.w)[col];
-      uint32_t gp = 0;
+    for (int j = 0; j < OWN; ++j) {
+      const int v = j * NW + wave;
+      if (v >= kFinishV) continue;
+      const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
+      if (col >= a.nv) continue;
+      const v4i s = fin[j];
+      if (first && a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
+      int r[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * e)) & 0xFFu));
-        wnew |= (static_cast<uint32_t>(clip127(wo - r[e])) & 0xFFu) << (8 * e);
-        gp |= (static_cast<uint32_t>(r[e]) & 0xFFu) << (8 * e);
+        if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
+        else r[e] = wrap_to_i8(s[e]);
       }
-      reinterpret_cast<uint32_t*>(a.w)[col] = wnew;
-      if (a.g8 != nullptr) reinterpret_cast<uint32_t*>(a.g8)[col] = gp;
-    } else {
+      const uint32_t e0 = static_cast<uint32_t>(col) * 4u;
+      const uint32_t rt = e0 / C;               // k * 9 + tap
+      const uint32_t c0 = e0 - rt * C;
+      uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
+      if (same_layout) {
+        uint32_t gp = 0;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (c0 + e < Cw) {
-          const uint32_t wi = rt * Cw + c0 + e;
-          const int wn = clip127(static_cast<int>(a.w[wi]) - r[e]);
-          a.w[wi] = static_cast<int8_t>(wn);
-          wnew |= (static_cast<uint32_t>(wn) & 0xFFu) << (8 * e);
-          if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
+        for (int e = 0; e < 4; ++e) {
+          const int wo = static_cast<int>(static_cast<int8_t>((wold[j] >> (8 * e)) & 0xFFu));
+          wnew |= (static_cast<uint32_t>(clip127(wo - r[e])) & 0xFFu) << (8 * e);
+          gp |= (static_cast<uint32_t>(r[e]) & 0xFFu) << (8 * e);
+        }
+        reinterpret_cast<uint32_t*>(a.w)[col] = wnew;
+        if (a.g8 != nullptr) reinterpret_cast<uint32_t*>(a.g8)[col] = gp;
+      } else {   // applied once only (the old weights are read here)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (c0 + e < Cw) {
+            const uint32_t wi = rt * Cw + c0 + e;
+            const int wn = clip127(static_cast<int>(a.w[wi]) - r[e]);
+            a.w[wi] = static_cast<int8_t>(wn);
+            wnew |= (static_cast<uint32_t>(wn) & 0xFFu) << (8 * e);
+            if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
+          }
         }
       }
+      if (a.wprep != nullptr) {
+        // [64-channel group][32-channel slice][tap][64 rows][32 bytes], 16-byte halves swapped where (row >> 3) is odd
+        const uint32_t k = rt / 9u, tap = rt - k * 9u;
+        const uint32_t row = k & 63u, cs = c0 >> 5;
+        const uint32_t half = ((c0 >> 4) & 1u) ^ ((row >> 3) & 1u);
+        const uint32_t dst = (((((k >> 6) * ((C + 31u) >> 5) + cs) * 9u + tap) * 64u + row) << 5) + half * 16u + (c0 & 15u);
+        *reinterpret_cast<uint32_t*>(a.wprep + dst) = wnew;
+      }
     }
-    if (a.wprep != nullptr) {
-      // [64-channel group][32-channel slice][tap][64 rows][32 bytes], 16-byte halves swapped where (row >> 3) is odd
-      const uint32_t k = rt / 9u, tap = rt - k * 9u;
-      const uint32_t row = k & 63u, cs = c0 >> 5;
-      const uint32_t half = ((c0 >> 4) & 1u) ^ ((row >> 3) & 1u);
-      const uint32_t dst = (((((k >> 6) * ((C + 31u) >> 5) + cs) * 9u + tap) * 64u + row) << 5) + half * 16u + (c0 & 15u);
-      *reinterpret_cast<uint32_t*>(a.wprep + dst) = wnew;
-    }
+  };
+  const bool speculate = a.predict != 0 && same_layout && gridDim.x > 1;
+  int applied = -1;
+  if (speculate) {
+    applied = max(max(bitwidth_of(bmax, a.bw_mode) - a.target_bits, 0), predicted);
+    apply(applied, true);
+  }
+  if (wave == 0) {
+    const uint32_t g = wait_slots(a.sync + kFinishSlot0, gridDim.x, a.spin_limit, &a.sync[1]);
+    if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
+  }
+  __syncthreads();
+  const uint32_t gmax = gshare;
+  const int shift = max(bitwidth_of(gmax, a.bw_mode) - a.target_bits, 0);
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    a.sync[0] = gmax;
+    if (a.shift_out != nullptr) *a.shift_out = shift;
+    if (a.exp_out != nullptr)
+      *a.exp_out = shift + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+  }
+  if (shift != applied) {
+    if (applied >= 0) __builtin_amdgcn_s_waitcnt(0);   // the first update's stores leave before those that replace them
+    apply(shift, applied < 0);
   }
 }
 
@@ -811,6 +833,7 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   f.target_bits = rq.target_bits;
   f.method = rq.method;
   f.trunc = rq.trunc;
+  f.predict = (rq.flags & NITI_RQ_SHIFT_HINT) != 0 ? 1 : 0;
   f.bw_mode = rq.bw_mode;
   f.spin_limit = rq.spin_limit;
   f.shift_out = rq.shift_out;

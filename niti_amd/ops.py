@@ -277,11 +277,14 @@ def wgrad_update_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1) -> int
 
 def conv2d_wgrad_update(act, err, w, stride=1, padding=1, f32_epilogue=False, mu=5, method="psto", div_mode="floor",
                         bw_mode="int", sync=None, want_grad=False, want_dw=False, shift_out=None, exp_a=None, exp_b=None,
-                        exp_out=None, workspace=None, prepared_filter=None):
+                        exp_out=None, workspace=None, prepared_filter=None, shift_hint=False):
     """Weight gradient + grad_calc + weight update: act [N,H,W,C] int8 (C may carry zero channel padding), err
     [N,H,W,K] int8, w [K,3,3,Cw] int8 updated in place.  Returns (g8 or None, dw int32 or None, device shift, sync).
     ``prepared_filter``: conv_filter_prepare(w padded to C channels, N, H, W) made earlier; it receives the updated
-    weights too and stays valid for the next forward pass."""
+    weights too and stays valid for the next forward pass.  ``shift_hint``: ``shift_out`` holds a predicted shift
+    on entry (the previous step's): the update's stores then overlap the wait for the tensor's range."""
+    if shift_hint and shift_out is None:
+        raise RuntimeError("conv2d_wgrad_update: shift_hint needs shift_out, holding the predicted shift")
     _chk_dev(act, err, w, sync, shift_out, exp_a, exp_b, exp_out, workspace, prepared_filter)
     if act.dtype != torch.int8 or err.dtype != torch.int8 or w.dtype != torch.int8:
         raise RuntimeError("conv2d_wgrad_update: int8 tensors expected")
@@ -307,7 +310,8 @@ def conv2d_wgrad_update(act, err, w, stride=1, padding=1, f32_epilogue=False, mu
     if shift_out is None:
         shift_out = torch.empty(1, dtype=torch.int32, device=w.device)
     st = L.lib().niti_conv2d_i8_wgrad_update(_ptr(act), _ptr(err), _ptr(w), Cw, N, H, W, C, K, R, S, stride, padding,
-                                             _flags(f32_epilogue), mu, L.ROUND[method], L.DIV[div_mode], L.BW[bw_mode],
+                                             _flags(f32_epilogue) | (L.CONV_SHIFT_HINT if shift_hint else 0), mu, L.ROUND[method],
+                                             L.DIV[div_mode], L.BW[bw_mode],
                                              _ptr(sync), sync.numel(), _ptr(g8), _ptr(dw), _ptr(prepared_filter), _ptr(shift_out), _ptr(exp_a),
                                              _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes, _stream(act))
     L.check(st, "niti_conv2d_i8_wgrad_update")

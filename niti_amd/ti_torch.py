@@ -504,7 +504,8 @@ class TiConv2d(UpdateWeight):
             self.act16, err_in, self.weight, self.stride, self.padding, f32_epilogue=F32_EPILOGUE and not self.first_layer,
             mu=GRAD_BITWIDTH, method=method, div_mode=DIV_MODE, bw_mode=BW_MODE, want_grad=self.keep_grad,
             want_dw=KEEP_INT32_GRAD, exp_a=_exp_tensor(self.err_exp, dev), exp_b=_exp_tensor(self.act_in_exp, dev),
-            exp_out=self.grad_exp, workspace=self._wgrad_workspace(err_in), prepared_filter=self._synced_filter())
+            exp_out=self.grad_exp, workspace=self._wgrad_workspace(err_in), prepared_filter=self._synced_filter(),
+            shift_out=self._shift_state("grad", dev), shift_hint=True)
         self.grad_int32acc = None if dw is None else (dw if dw.shape[3] == C else dw[..., :C].contiguous())
         return True
 

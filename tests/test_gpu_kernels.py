@@ -432,6 +432,14 @@ def test_conv_wgrad_update(dev, case, div_mode):
         assert int(sh.cpu()) == sh_ref and int(eo.cpu()) == sh_ref - 4
         assert torch.equal(g8.cpu(), g8_ref)
         assert torch.equal(wd.cpu(), w_ref)
+        # a predicted shift (right, too small, too large) changes when the update is stored, never its result
+        for guess in (sh_ref, max(sh_ref - 1, 0), sh_ref + 2):
+            wd3 = w.to(dev).clone()
+            so = torch.tensor([guess], dtype=torch.int32, device=dev)
+            g8p, _, shp, syncp = ops.conv2d_wgrad_update(act16.to(dev).contiguous(), err.to(dev), wd3, mu=mu, method=method,
+                                                         div_mode=div_mode, want_grad=True, shift_out=so, shift_hint=True)
+            assert int(syncp.cpu()[1]) == 0 and int(so.cpu()) == sh_ref
+            assert torch.equal(g8p.cpu(), g8_ref) and torch.equal(wd3.cpu(), w_ref)
         # without the optional outputs, and with a kernel-ready forward filter copy that has to follow the update
         wd2 = w.to(dev).clone()
         w16 = (F.pad(w, (0, 16 - C % 16)) if C % 16 else w).to(dev).contiguous()
