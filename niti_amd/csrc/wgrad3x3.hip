@@ -50,6 +50,25 @@ struct WgradArgs {
   long long act_bytes, err_bytes;
 };
 
+// Workgroups are handed to the eight accelerator dies (each with its own L2) round robin in launch order.  The
+// workgroups that read the same pixels - all tiles of one pixel range - should share a die: workgroup p of the
+// launch therefore takes the work item (p % 8) * (total / 8) + p / 8 of the order "tiles fastest, pixel ranges
+// slowest", which gives every die a contiguous run of that order.  (A mapping for locality only: any assignment
+// of work items to workgroups computes the same sums.)
+struct WorkItem { int x, y, z; };
+__device__ inline WorkItem die_local_work_item() {
+  const int gx = gridDim.x, gy = gridDim.y, gz = gridDim.z;
+  const int total = gx * gy * gz;
+  int p = blockIdx.x + gx * (blockIdx.y + gy * blockIdx.z);
+  if (total % 8 == 0) p = (p % 8) * (total / 8) + p / 8;
+  WorkItem w;
+  w.x = p % gx;
+  p /= gx;
+  w.y = p % gy;
+  w.z = p / gy;
+  return w;
+}
+
 // Q: image width = height; BR: output rows of one image per band; NI: images per band; BR*NI*Q == 128
 template <int Q, int BR, int NI>
 struct Geom {
@@ -74,9 +93,10 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int k0 = blockIdx.x * 128;
-  const int c0 = blockIdx.y * 64;
-  const int band_begin = blockIdx.z * a.bands_per_split;
+  const WorkItem item = die_local_work_item();
+  const int k0 = item.x * 128;
+  const int c0 = item.y * 64;
+  const int band_begin = item.z * a.bands_per_split;
   const int band_end = min(band_begin + a.bands_per_split, a.bands);
   const int nb = band_end - band_begin;
 
@@ -230,7 +250,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
   }
 
   // ---- partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+wc*32+(lane&31)]
-  int32_t* out = a.partial + static_cast<long long>(blockIdx.z) * a.slice_stride;
+  int32_t* out = a.partial + static_cast<long long>(item.z) * a.slice_stride;
   const int c = c0 + wc * 32 + (lane & 31);
   if (c < a.C) {
 #pragma unroll
@@ -282,9 +302,10 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int k0 = blockIdx.x * 128;
-  const int c0 = blockIdx.y * 32;
-  const int band_begin = blockIdx.z * a.bands_per_split;   // bands of 256 pixels here
+  const WorkItem item = die_local_work_item();
+  const int k0 = item.x * 128;
+  const int c0 = item.y * 32;
+  const int band_begin = item.z * a.bands_per_split;   // bands of 256 pixels here
   const int band_end = min(band_begin + a.bands_per_split, a.bands);
   const int nb = band_end - band_begin;
 
@@ -428,7 +449,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   __syncthreads();
   if (ph == 0) {
     // partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+(lane&31)]
-    int32_t* out = a.partial + static_cast<long long>(blockIdx.z) * a.slice_stride;
+    int32_t* out = a.partial + static_cast<long long>(item.z) * a.slice_stride;
     const int c = c0 + (lane & 31);
 #pragma unroll
     for (int g = 0; g < 4; ++g)
