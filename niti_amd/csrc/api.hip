@@ -222,9 +222,10 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
 long long niti::sync_spin_limit() {
   static long long spin_limit = -1;
   if (spin_limit < 0) {
-    const char* e = getenv("NITI_SYNC_TIMEOUT_MS");
-    const long long ms = e != nullptr ? atoll(e) : 10000;
-    spin_limit = (ms > 0 ? ms : 1) * 100000LL;
+    const char* e = getenv("NITI_SYNC_TIMEOUT_MS");   // fractions allowed: 0.00001 ms is one tick
+    const double ms = e != nullptr ? atof(e) : 10000.0;
+    const double ticks = ms * 100000.0;
+    spin_limit = ticks >= 1.0 ? static_cast<long long>(ticks) : 1LL;
   }
   return spin_limit;
 }

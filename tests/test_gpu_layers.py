@@ -248,3 +248,33 @@ def test_shims_match_reference_conventions():
     assert dx.dtype == torch.float16
     assert torch.equal(dx.type(torch.int8).cpu(), po.maxpool_bwd(po.maxpool_fwd(x), dy, x))
     assert hasattr(int8conv_cuda, "group_conv") and hasattr(cutlassconv_cuda, "weight_grad")
+
+
+def test_grid_wide_wait_gives_up_and_says_so():
+    """With a wait limit of one clock tick (set from the host, in a process of its own because the library reads
+    the limit once) the single-launch kernels do not wait for late workgroups: every workgroup still runs to its
+    end, the launch completes, and the sync words report that the result is not to be used."""
+    import os
+    import subprocess
+    import sys
+    code = r"""
+import torch
+from niti_amd import ops
+dev = torch.device("cuda:0")
+g = torch.Generator().manual_seed(1)
+x = torch.randint(-127, 128, (64, 32, 32, 64), generator=g, dtype=torch.int8).to(dev)
+w = torch.randint(-127, 128, (128, 3, 3, 64), generator=g, dtype=torch.int8).to(dev)
+ops.sync_arena.reset(dev)
+flagged = 0
+for i in range(4):
+    y, sh, sync = ops.conv2d_fprop_requant(x, w)
+    torch.cuda.synchronize()
+    flagged += int(sync.cpu()[1] != 0)
+print("FLAGGED", flagged, "ARENA", int(ops.sync_arena.timed_out(dev)))
+"""
+    env = dict(os.environ, NITI_SYNC_TIMEOUT_MS="0.00001")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = subprocess.run([sys.executable, "-c", code], cwd=root, env=env, capture_output=True, text=True, timeout=120)
+    assert out.returncode == 0, out.stderr[-2000:]
+    line = [l for l in out.stdout.splitlines() if l.startswith("FLAGGED")][0].split()
+    assert int(line[1]) >= 1 and int(line[3]) == 1
