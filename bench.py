@@ -205,18 +205,19 @@ def cpu_baseline(min_seconds=10.0):
             "sample": "%d pass(es) of the full six-layer conv triple at batch %d (plain-C oracle, OpenMP), %.1f s" % (passes, BATCH, t_total)}
 
 
-def train_step_rate(dev, steps, warmup):
-    """images/s of a complete VGG-small (six conv + FC) integer training step, batch 128 (configs[3])."""
+def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH):
+    """images/s of a complete integer training step: VGG-small (six conv + FC), batch 128 (configs[3]), or the
+    ten-convolution VGG-13 widths, batch 256 (configs[4])."""
     import torch
     from niti_amd import ti_torch, ti_vgg
-    g = torch.Generator().manual_seed(1237)
-    net = ti_vgg.TiVGG_cifar(7)
+    g = torch.Generator().manual_seed(1237 + depth)
+    net = ti_vgg.TiVGG_cifar(depth)
     for l in net.forward_layers:
         if hasattr(l, "weight"):
             l.weight = torch.randint(-127, 128, tuple(l.weight.shape), generator=g, dtype=torch.int8).to(dev)
             l.weight_exp = torch.tensor(-8.0)
-    x = torch.randint(-127, 128, (BATCH, 32, 32, 3), generator=g, dtype=torch.int8).to(dev)
-    target = torch.randint(0, 10, (BATCH,), generator=g).to(dev)
+    x = torch.randint(-127, 128, (batch, 32, 32, 3), generator=g, dtype=torch.int8).to(dev)
+    target = torch.randint(0, 10, (batch,), generator=g).to(dev)
     ti_torch.TRAINING = True
     ti_torch.GRAD_BITWIDTH = 5
 
@@ -231,7 +232,7 @@ def train_step_rate(dev, steps, warmup):
         run()
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
-    return BATCH / dt, dt * 1e3, mode
+    return batch / dt, dt * 1e3, mode
 
 
 def main():
@@ -331,6 +332,9 @@ def main():
         ips, ms, tmode = train_step_rate(dev, max(args.steps, 5), max(args.warmup, 2))
         out["train_step"] = {"workload": "BASELINE configs[3]: VGG-small (6 conv + FC) integer training step, batch 128",
                              "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": tmode}
+        ips, ms, tmode = train_step_rate(dev, max(args.steps, 5), max(args.warmup, 2), depth=13, batch=256)
+        out["train_step_vgg13"] = {"workload": "BASELINE configs[4]: VGG-13 widths (10 conv + FC) integer training step, batch 256",
+                                   "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": tmode}
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
