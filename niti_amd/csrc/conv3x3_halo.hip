@@ -80,14 +80,15 @@ struct HaloArgs {
 constexpr int kSyncSlot0 = 16;
 
 // Q: image width = height; BR: output rows of one image per workgroup; NI: images per workgroup; BR*NI*Q == 256.
-// The halo tile is NI*(BR+2) rows of Q slots of 32 bytes; Q is a multiple of 8 so that the bank of a slot
-// depends on its column only, and the 16-byte halves of a slot are swapped where ((column >> 3) ^ row) is odd:
-// 16 lanes reading consecutive columns of one row, or 8 + 8 columns of two adjacent rows, then hit 16 distinct
-// bank groups.
+// The halo tile is NI*(BR+2) rows of Q slots of 32 bytes; for Q a multiple of 8 the bank of a slot depends on its
+// column only, and the 16-byte halves of a slot are swapped where ((column >> 3) ^ row) is odd: 16 lanes reading
+// consecutive columns of one row, or 8 + 8 columns of two adjacent rows, then hit 16 distinct bank groups.  The
+// 4 x 4 and 2 x 2 maps at the end of a deep network use the same code (16 / 64 whole images per workgroup) with
+// some bank conflicts in their short rows.
 template <int Q, int BR, int NI, int KT>
 struct HGeom {
   static constexpr int RP = Q;                             // no halo columns: horizontal neighbours come from lane shifts
-  static_assert(Q % 8 == 0, "bank mapping");
+  static_assert(Q == 2 || Q == 4 || Q % 8 == 0, "rows of 2, 4 or a multiple of 8 pixels");
   static constexpr int HR = BR + 2;
   static constexpr int SLOTS = NI * HR * RP;
   static constexpr int ACT_INSTR = (SLOTS + 31) / 32;      // one instruction fills 32 slots
@@ -562,7 +563,8 @@ __global__ __launch_bounds__(256) void halo_filter_prepare_kernel(const int8_t* 
 
 // Channel tile of a launch: 128 unless that leaves fewer workgroups than the device runs at once while
 // a tile of 64 would give it more to do.
-int halo_ktile(long long pix, int K) {
+int halo_ktile(long long pix, int K, int H) {
+  if (H == 2) return 128;   // the 2 x 2 maps' halo tile leaves room for the wide tile's filter ring only
   static int cus = 0;
   if (cus == 0) {
     int dev = 0;
@@ -571,7 +573,8 @@ int halo_ktile(long long pix, int K) {
   }
   const char* e = getenv("NITI_HALO_KT");  // tests and tuning runs pin the tile
   const int forced = e != nullptr ? atoi(e) : 0;
-  if (forced == 128 || (forced == 64 && K > 64)) return forced;
+  if (forced == 128 || forced == 64) return forced;
+  if (K <= 64) return 64;   // nothing to gain from computing 128 channels
   const long long b128 = (pix / 256) * ((K + 127) / 128);
   return (b128 < 2LL * cus && K > 64) ? 64 : 128;
 }
@@ -608,15 +611,18 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
 
 template <bool kFused, bool kWT>
 int launch_halo_tiles(const HaloArgs& a, int H, hipStream_t stream) {
-  const int ktile = halo_ktile(static_cast<long long>(a.N) * H * H, a.K);
+  const int ktile = halo_ktile(static_cast<long long>(a.N) * H * H, a.K, H);
   if (ktile == 128) {
     if (H == 32) return launch_halo<32, 8, 1, 128, kFused, kWT>(a, stream);
     if (H == 16) return launch_halo<16, 16, 1, 128, kFused, kWT>(a, stream);
-    return launch_halo<8, 8, 4, 128, kFused, kWT>(a, stream);
+    if (H == 8) return launch_halo<8, 8, 4, 128, kFused, kWT>(a, stream);
+    if (H == 4) return launch_halo<4, 4, 16, 128, kFused, kWT>(a, stream);
+    return launch_halo<2, 2, 64, 128, kFused, kWT>(a, stream);
   }
   if (H == 32) return launch_halo<32, 8, 1, 64, kFused, kWT>(a, stream);
   if (H == 16) return launch_halo<16, 16, 1, 64, kFused, kWT>(a, stream);
-  return launch_halo<8, 8, 4, 64, kFused, kWT>(a, stream);
+  if (H == 8) return launch_halo<8, 8, 4, 64, kFused, kWT>(a, stream);
+  return launch_halo<4, 4, 16, 64, kFused, kWT>(a, stream);
 }
 
 template <bool kFused>
@@ -644,7 +650,7 @@ void fill_common(HaloArgs& a, const int8_t* x, const int8_t* wp, int N, int H, i
 
 bool conv3x3_halo_supported(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
   if (R != 3 || S != 3 || stride != 1 || pad != 1 || H != W) return false;
-  if (H != 8 && H != 16 && H != 32) return false;
+  if (H != 2 && H != 4 && H != 8 && H != 16 && H != 32) return false;
   if (C % 16 != 0 || K % 4 != 0) return false;
   const long long pix = static_cast<long long>(N) * H * W;
   if (pix % 256 != 0) return false;  // workgroups own whole rows / whole images
@@ -680,7 +686,7 @@ int launch_conv3x3_halo(const int8_t* x, const int8_t* wp, int32_t* y, int N, in
 int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
   if (!conv3x3_halo_supported(N, H, W, C, K, R, S, stride, pad) || K % 16 != 0) return 0;
   const long long pix = static_cast<long long>(N) * H * W;
-  const int ktile = halo_ktile(pix, K);
+  const int ktile = halo_ktile(pix, K, H);
   const long long nb = (pix / 256) * ((K + ktile - 1) / ktile);
   return nb <= 2048 ? static_cast<int>(nb) : 0;  // the device check happens at launch; this bounds the workspace
 }

@@ -106,7 +106,7 @@ def test_conv_dgrad(dev, case):
 
 # convolution + requantisation in one launch: N,Q,C,K (3x3, stride 1, pad 1), small sums / large sums / ragged tiles
 FUSED_CASES = [(4, 8, 16, 16), (4, 8, 64, 128), (8, 8, 80, 144), (1, 16, 16, 48), (3, 16, 192, 272), (2, 32, 16, 64),
-               (8, 32, 128, 128), (12, 8, 512, 128)]
+               (8, 32, 128, 128), (12, 8, 512, 128), (16, 4, 64, 128), (48, 4, 256, 80), (64, 2, 512, 512), (128, 2, 32, 48)]
 
 
 @pytest.fixture(params=["auto", "64", "128"])
@@ -123,7 +123,8 @@ def halo_tile(request):
         os.environ["NITI_HALO_KT"] = old
 
 
-@pytest.mark.parametrize("case", [(8, 8, 64, 128), (4, 8, 80, 24), (3, 16, 192, 260), (2, 32, 16, 64), (8, 32, 128, 256), (12, 8, 512, 128)])
+@pytest.mark.parametrize("case", [(8, 8, 64, 128), (4, 8, 80, 24), (3, 16, 192, 260), (2, 32, 16, 64), (8, 32, 128, 256), (12, 8, 512, 128),
+                                  (32, 4, 128, 256), (16, 4, 48, 16), (64, 2, 256, 128), (192, 2, 64, 32)])
 def test_conv_halo_tiles(dev, case, halo_tile):
     """Forward, data gradient and the requantising variant with both channel tiles of the halo kernel."""
     from niti_amd import ops
