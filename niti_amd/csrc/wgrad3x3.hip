@@ -287,7 +287,7 @@ struct NGeom {
   static constexpr int NL = 4 + ACT_LOADS;                  // loads per wavefront per stage
   static constexpr int REDUCE_BYTES = 4 * 9 * 16 * 64 * 4;  // four wavefronts park their accumulators
   static constexpr int LDS_BYTES = (STAGES * STAGE_BYTES > REDUCE_BYTES ? STAGES * STAGE_BYTES : REDUCE_BYTES) + 1024;
-  static constexpr int HALF_ROWS = Q == 8 ? 2 * HR : 128 / Q;  // halo rows between the two pixel halves of a stage
+  static constexpr int HALF_ROWS = NI > 1 ? (NI / 2) * HR : 128 / Q;  // halo rows between the two pixel halves of a stage
   static_assert(BR * NI * Q == 256, "a stage is 256 output pixels");
   static_assert(NI == 1 || BR == Q, "several images per stage only as whole images");
   static_assert(LDS_BYTES <= 160 * 1024, "stages must fit in LDS");
@@ -367,7 +367,10 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   const int wk = wave & 3;    // 32-output-channel quarter of the tile
   const int ph = wave >> 2;   // 128-pixel half of a stage
   int a_base[2];
-  constexpr int NB = Q >= 16 ? 3 : 4;
+  // Rows of at least 8 pixels: the second and third tap of a filter row are byte shifts of the first one's pixels
+  // (3 or 4 reads per filter row).  Shorter rows (4 x 4 maps: eight pixels are two rows) read every tap.
+  constexpr bool kShiftTaps = Q >= 8;
+  constexpr int NB = kShiftTaps ? (Q >= 16 ? 3 : 4) : 6;
   int b_base[NB];
 #pragma unroll
   for (int o = 0; o < 2; ++o) {
@@ -377,9 +380,19 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   }
   {
     const int cb = gg * 16 + 8 * (j & 1);
-    auto slot_addr = [&](int lrow, int w) { return G::ERR_BYTES + ((ph * G::HALF_ROWS + lrow) * G::RP + w) * 32 + cb; };
+    // lrow: output row inside the 32 pixels of a reduction step (which may span several whole images)
+    auto slot_addr = [&](int lrow, int w) {
+      const int hrow = (lrow / BR) * G::HR + lrow % BR;
+      return G::ERR_BYTES + ((ph * G::HALF_ROWS + hrow) * G::RP + w) * 32 + cb;
+    };
     const int p0 = 16 * lk + (j >> 1), p1 = p0 + 8;
-    if (Q >= 16) {
+    if (!kShiftTaps) {
+#pragma unroll
+      for (int t = 0; t < 3; ++t) {
+        b_base[2 * t] = slot_addr(p0 / Q, p0 % Q + t);
+        b_base[2 * t + 1] = slot_addr(p1 / Q, p1 % Q + t);
+      }
+    } else if (Q >= 16) {
       b_base[0] = slot_addr(p0 / Q, p0 % Q);
       b_base[1] = slot_addr(p1 / Q, p1 % Q);
       b_base[2] = slot_addr(p0 / Q, p0 % Q + 16);
@@ -423,15 +436,22 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
 #pragma unroll
         for (int q = 0; q < NB; ++q)
           rd[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(sbase + b_base[q] + roff));
-        const int d0 = rd[0][0], d1 = rd[0][1], d2 = rd[1][0];
-        const int e0 = Q >= 16 ? rd[1][0] : rd[2][0], e1 = Q >= 16 ? rd[1][1] : rd[2][1];
-        const int e2 = rd[NB - 1][0];
-        acc[r * 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{d0, d1, e0, e1}, acc[r * 3], 0, 0, 0);
+        if constexpr (!kShiftTaps) {
 #pragma unroll
-        for (int s = 1; s < 3; ++s) {
-          const v4i bf = {static_cast<int>(__builtin_amdgcn_alignbyte(d1, d0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(d2, d1, s)),
-                          static_cast<int>(__builtin_amdgcn_alignbyte(e1, e0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(e2, e1, s))};
-          acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[r * 3 + s], 0, 0, 0);
+          for (int s = 0; s < 3; ++s)
+            acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{rd[2 * s][0], rd[2 * s][1], rd[2 * s + 1][0], rd[2 * s + 1][1]},
+                                                                   acc[r * 3 + s], 0, 0, 0);
+        } else {
+          const int d0 = rd[0][0], d1 = rd[0][1], d2 = rd[1][0];
+          const int e0 = Q >= 16 ? rd[1][0] : rd[2][0], e1 = Q >= 16 ? rd[1][1] : rd[2][1];
+          const int e2 = rd[NB - 1][0];
+          acc[r * 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{d0, d1, e0, e1}, acc[r * 3], 0, 0, 0);
+#pragma unroll
+          for (int s = 1; s < 3; ++s) {
+            const v4i bf = {static_cast<int>(__builtin_amdgcn_alignbyte(d1, d0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(d2, d1, s)),
+                            static_cast<int>(__builtin_amdgcn_alignbyte(e1, e0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(e2, e1, s))};
+            acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[r * 3 + s], 0, 0, 0);
+          }
         }
       }
     }
@@ -691,6 +711,7 @@ long long slice_stride_for(int C, int K) {
 // The narrow-tile arrangement needs whole stages of 256 pixels.  NITI_WGRAD_NARROW=0/1 pins the choice (tests).
 bool use_narrow_arrangement(int N, int Q) {
   const bool fits = (static_cast<long long>(N) * Q * Q) % 256 == 0;
+  if (Q < 8) return true;   // the only arrangement for the small maps (the shape check requires whole stages)
   const char* e = getenv("NITI_WGRAD_NARROW");
   if (e != nullptr) return e[0] == '1' && fits;
   return fits;
@@ -754,10 +775,11 @@ int launch_geom(const WgradArgs& a, int splits, hipStream_t stream) {
 
 bool wgrad3x3_supported(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
   if (R != 3 || S != 3 || stride != 1 || pad != 1 || H != W) return false;
-  if (H != 8 && H != 16 && H != 32) return false;
+  if (H != 4 && H != 8 && H != 16 && H != 32) return false;
   if (C % 16 != 0 || K % 16 != 0) return false;
   const long long pix = static_cast<long long>(N) * H * W;
   if (pix % 128 != 0) return false;  // bands of 128 pixels: whole rows / whole images
+  if (H == 4 && pix % 256 != 0) return false;  // 4 x 4 maps: only the arrangement with stages of 256 pixels
   if (H == 8 && N % 2 != 0) return false;
   if (pix * C >= 0x7fffffffLL || pix * K >= 0x7fffffffLL) return false;
   return true;
@@ -785,7 +807,8 @@ static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N,
   if (narrow) {
     if (H == 32) return launch_narrow_geom<32, 8, 1>(a, splits, stream);
     if (H == 16) return launch_narrow_geom<16, 16, 1>(a, splits, stream);
-    return launch_narrow_geom<8, 8, 4>(a, splits, stream);
+    if (H == 8) return launch_narrow_geom<8, 8, 4>(a, splits, stream);
+    return launch_narrow_geom<4, 4, 16>(a, splits, stream);
   }
   if (H == 32) return launch_geom<32, 4, 1>(a, splits, stream);
   if (H == 16) return launch_geom<16, 8, 1>(a, splits, stream);
