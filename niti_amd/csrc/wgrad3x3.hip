@@ -283,7 +283,7 @@ struct NGeom {
   static constexpr int ACT_LOADS = (ACT_INSTR + 7) / 8;
   static constexpr int ERR_BYTES = 256 * 128;               // 32 instructions of 8 pixels x 128 bytes
   static constexpr int STAGE_BYTES = ERR_BYTES + ACT_BYTES;
-  static constexpr int STAGES = 3;
+  static constexpr int STAGES = Q == 2 ? 2 : 3;             // the 2 x 2 maps' halo tile is as large as the error tile
   static constexpr int NL = 4 + ACT_LOADS;                  // loads per wavefront per stage
   static constexpr int REDUCE_BYTES = 4 * 9 * 16 * 64 * 4;  // four wavefronts park their accumulators
   static constexpr int LDS_BYTES = (STAGES * STAGE_BYTES > REDUCE_BYTES ? STAGES * STAGE_BYTES : REDUCE_BYTES) + 1024;
@@ -368,7 +368,8 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   const int ph = wave >> 2;   // 128-pixel half of a stage
   int a_base[2];
   // Rows of at least 8 pixels: the second and third tap of a filter row are byte shifts of the first one's pixels
-  // (3 or 4 reads per filter row).  Shorter rows (4 x 4 maps: eight pixels are two rows) read every tap.
+  // (3 or 4 reads per filter row).  Shorter rows (4 x 4 and 2 x 2 maps: eight pixels are two or four rows) read
+  // every tap.
   constexpr bool kShiftTaps = Q >= 8;
   constexpr int NB = kShiftTaps ? (Q >= 16 ? 3 : 4) : 6;
   int b_base[NB];
@@ -775,11 +776,11 @@ int launch_geom(const WgradArgs& a, int splits, hipStream_t stream) {
 
 bool wgrad3x3_supported(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
   if (R != 3 || S != 3 || stride != 1 || pad != 1 || H != W) return false;
-  if (H != 4 && H != 8 && H != 16 && H != 32) return false;
+  if (H != 2 && H != 4 && H != 8 && H != 16 && H != 32) return false;
   if (C % 16 != 0 || K % 16 != 0) return false;
   const long long pix = static_cast<long long>(N) * H * W;
   if (pix % 128 != 0) return false;  // bands of 128 pixels: whole rows / whole images
-  if (H == 4 && pix % 256 != 0) return false;  // 4 x 4 maps: only the arrangement with stages of 256 pixels
+  if (H <= 4 && pix % 256 != 0) return false;  // small maps: only the arrangement with stages of 256 pixels
   if (H == 8 && N % 2 != 0) return false;
   if (pix * C >= 0x7fffffffLL || pix * K >= 0x7fffffffLL) return false;
   return true;
@@ -808,7 +809,8 @@ static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N,
     if (H == 32) return launch_narrow_geom<32, 8, 1>(a, splits, stream);
     if (H == 16) return launch_narrow_geom<16, 16, 1>(a, splits, stream);
     if (H == 8) return launch_narrow_geom<8, 8, 4>(a, splits, stream);
-    return launch_narrow_geom<4, 4, 16>(a, splits, stream);
+    if (H == 4) return launch_narrow_geom<4, 4, 16>(a, splits, stream);
+    return launch_narrow_geom<2, 2, 64>(a, splits, stream);
   }
   if (H == 32) return launch_geom<32, 4, 1>(a, splits, stream);
   if (H == 16) return launch_geom<16, 8, 1>(a, splits, stream);

@@ -403,7 +403,7 @@ def test_conv_wgrad_arrangements(dev, case, wgrad_arrangement):
 
 
 @pytest.mark.parametrize("case", [(4, 32, 16, 32), (8, 16, 128, 64), (6, 8, 80, 144), (64, 8, 64, 256), (16, 16, 256, 128),
-                                  (2, 8, 16, 16), (4, 8, 3, 16), (8, 32, 3, 128), (32, 8, 512, 512), (16, 4, 64, 128), (64, 4, 512, 256)])
+                                  (2, 8, 16, 16), (4, 8, 3, 16), (8, 32, 3, 128), (32, 8, 512, 512), (16, 4, 64, 128), (64, 4, 512, 256), (64, 2, 128, 64), (256, 2, 512, 512)])
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 def test_conv_wgrad_update(dev, case, div_mode):
     """wgrad + grad_calc + weight update in one call against the oracle's three steps."""
@@ -528,7 +528,8 @@ def test_conv_requant_rejects_what_it_does_not_cover(dev):
 WGRAD_CASES = [(4, 32, 32, 16, 32, 3, 1), (8, 16, 16, 128, 64, 3, 1), (6, 8, 8, 80, 144, 3, 1), (2, 32, 32, 64, 128, 3, 1),
                (64, 8, 8, 64, 256, 3, 1), (16, 16, 16, 256, 128, 3, 1), (2, 8, 8, 16, 16, 3, 1), (16, 8, 8, 32, 48, 3, 1), (5, 7, 9, 40, 24, 3, 1), (32, 16, 16, 64, 128, 3, 1),
                (4, 8, 8, 3, 16, 3, 1), (6, 8, 8, 16, 10, 5, 2), (3, 6, 6, 8, 8, 3, 0), (128, 8, 8, 16, 16, 3, 1),
-               (16, 4, 4, 64, 128, 3, 1), (48, 4, 4, 272, 80, 3, 1), (256, 4, 4, 32, 16, 3, 1), (8, 4, 4, 16, 16, 3, 1)]
+               (16, 4, 4, 64, 128, 3, 1), (48, 4, 4, 272, 80, 3, 1), (256, 4, 4, 32, 16, 3, 1), (8, 4, 4, 16, 16, 3, 1),
+               (64, 2, 2, 64, 128, 3, 1), (192, 2, 2, 272, 48, 3, 1), (256, 2, 2, 512, 512, 3, 1), (32, 2, 2, 16, 16, 3, 1)]
 
 
 @pytest.mark.parametrize("case", WGRAD_CASES)
