@@ -26,6 +26,8 @@
 // int32 store + separate requantisation pass this removes 8 of the 9 bytes moved per output element.
 #include <stdlib.h>
 
+#include <utility>
+
 #include "common.h"
 #include "requant_math.h"
 
@@ -51,6 +53,41 @@ __device__ inline void hc_sync() {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
   asm volatile("" ::: "memory");
+}
+
+// ds_read_b64_tr_b8 as inline assembly.  Before the builtin form the compiler places s_waitcnt vmcnt(0) whenever a
+// buffer_load ... lds is in flight (it cannot tell which LDS bytes that load writes), which would make every stage
+// wait for the loads it has just issued.  The compiler does not count these reads either: the caller waits with
+// lds_settle<N>() - at most N LDS operations issued after the wanted ones still in flight; operations the compiler
+// adds in between only make that wait stricter - and passes the results through lds_landed() before using them.
+template <int OFF>
+__device__ inline v2i lds_read_tr8(unsigned addr) {
+  v2i r;
+  asm volatile("ds_read_b64_tr_b8 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
+__device__ inline v4i lds_read_b128(unsigned addr) {
+  v4i r;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
+  return r;
+}
+template <int N>
+__device__ inline void lds_settle() {
+  asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N));
+}
+__device__ inline v4i lds_landed(v2i lo, v2i hi) {
+  asm volatile("" : "+v"(lo), "+v"(hi));
+  return v4i{lo[0], lo[1], hi[0], hi[1]};
+}
+__device__ inline unsigned lds_addr(const void* p) { return static_cast<unsigned>(reinterpret_cast<uintptr_t>(NITI_LDS(p))); }
+
+template <class F, int... I>
+__device__ inline void static_for_impl(F& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, class F>
+__device__ inline void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
 }
 
 struct HaloArgs {
@@ -83,12 +120,12 @@ constexpr int kSyncSlot0 = 16;
 // The halo tile is NI*(BR+2) rows of Q slots of 32 bytes; for Q a multiple of 8 the bank of a slot depends on its
 // column only, and the 16-byte halves of a slot are swapped where ((column >> 3) ^ row) is odd: 16 lanes reading
 // consecutive columns of one row, or 8 + 8 columns of two adjacent rows, then hit 16 distinct bank groups.  The
-// 4 x 4 and 2 x 2 maps at the end of a deep network use the same code (16 / 64 whole images per workgroup) with
-// some bank conflicts in their short rows.
+// 4 x 4 maps of a deep network use the same code (16 whole images per workgroup) with some bank conflicts in
+// their short rows; 2 x 2 maps have a kernel of their own below.
 template <int Q, int BR, int NI, int KT>
 struct HGeom {
   static constexpr int RP = Q;                             // no halo columns: horizontal neighbours come from lane shifts
-  static_assert(Q == 2 || Q == 4 || Q % 8 == 0, "rows of 2, 4 or a multiple of 8 pixels");
+  static_assert(Q == 4 || Q % 8 == 0, "rows of 4 or a multiple of 8 pixels");
   static constexpr int HR = BR + 2;
   static constexpr int SLOTS = NI * HR * RP;
   static constexpr int ACT_INSTR = (SLOTS + 31) / 32;      // one instruction fills 32 slots
@@ -246,23 +283,45 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     // 16 channels lane / 32), so the pixel to the left is one lane down and the one to the right one lane up
     v4i pc[2];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) pc[j] = *reinterpret_cast<const v4i*>(sa + ((p_addr[j] + roff) ^ ((r & 1) << 4)));
+    for (int j = 0; j < 2; ++j) {
+      const int at = (p_addr[j] + roff) ^ ((r & 1) << 4);
+      if constexpr (kWT) pc[j] = lds_read_b128(lds_addr(sa) + at);   // counted by hand like the filter reads behind it
+      else pc[j] = *reinterpret_cast<const v4i*>(sa + at);
+    }
     v4i wf[3][NWF];
-#pragma unroll
-    for (int s = 0; s < 3; ++s)
-#pragma unroll
-      for (int i = 0; i < NWF; ++i) {
-        const int8_t* src = sw + ((s + 1) % 3) * TAPB;
-        if (kWT) {
-          typedef int v2i_t __attribute__((ext_vector_type(2)));
-          const v2i_t lo = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(src + w_addr[i][0]));
-          const v2i_t hi = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(src + w_addr[i][kWT ? 1 : 0]));
-          wf[s][i] = v4i{lo[0], lo[1], hi[0], hi[1]};
-        } else {
-          wf[s][i] = *reinterpret_cast<const v4i*>(src + w_addr[i][0]);
-        }
-      }
+    v2i tlo[3][NWF], thi[3][NWF];   // kWT: halves of the transposed fragments until they have landed
     // order: centre tap (needs no shifting) first, then right, then left; wf[0] = tap s=1, wf[1] = s=2, wf[2] = s=0
+    if constexpr (kWT) {
+      const unsigned swa = lds_addr(sw);
+      static_for<3>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        constexpr int off = ((s + 1) % 3) * TAPB;
+#pragma unroll
+        for (int i = 0; i < NWF; ++i) {
+          tlo[s][i] = lds_read_tr8<off>(swa + w_addr[i][0]);
+          thi[s][i] = lds_read_tr8<off>(swa + w_addr[i][kWT ? 1 : 0]);
+        }
+      });
+    } else {
+#pragma unroll
+      for (int s = 0; s < 3; ++s)
+#pragma unroll
+        for (int i = 0; i < NWF; ++i) wf[s][i] = *reinterpret_cast<const v4i*>(sw + ((s + 1) % 3) * TAPB + w_addr[i][0]);
+    }
+    // kWT: the reads of a tap are 2 * NWF operations; those of the taps behind it may still be in flight
+    auto tap_ready = [&](auto sc) {
+      if constexpr (kWT) {
+        constexpr int s = decltype(sc)::value;
+        lds_settle<(2 - s) * 2 * NWF>();
+        if (s == 0) {
+#pragma unroll
+          for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(pc[j]));
+        }
+#pragma unroll
+        for (int i = 0; i < NWF; ++i) wf[s][i] = lds_landed(tlo[s][i], thi[s][i]);
+      }
+    };
+    tap_ready(std::integral_constant<int, 0>{});
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
 #pragma unroll
@@ -272,6 +331,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
+    tap_ready(std::integral_constant<int, 1>{});
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
 #pragma unroll
@@ -280,6 +340,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     for (int j = 0; j < 2; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
+    tap_ready(std::integral_constant<int, 2>{});
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
 #pragma unroll
@@ -532,6 +593,198 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   }
 }
 
+// ---- 2 x 2 maps -----------------------------------------------------------------------------------------
+// With one pixel of padding every output pixel of a 2 x 2 map sees all four input pixels, each through one filter
+// tap: the convolution is a dense product [N] x [4 C] x [4 K] whose filter operand for output pixel p and input
+// pixel q is tap (qy - py + 1, qx - px + 1).  The halo kernel would give such a layer (the last ones of a deep
+// network: few pixels, many channels) one workgroup per 64 images and spend 5 of its 9 taps on padding; here a
+// workgroup owns 32 images x 32 output channels, wavefront (p, half) computes output pixel p over one half of the
+// channel slices, and the two halves are added through LDS.  Both operands are fetched as MFMA fragments without a
+// shared tile: the activation rows straight into registers, the filter from the same prepared copy the halo kernel
+// reads (a 32 x 32 block of it is 1 KB in a row) - into registers, or, for the data gradient reading the forward
+// copy, into a per-wavefront LDS slot that ds_read_b64_tr_b8 transposes.  Loads run eight reduction steps ahead.
+constexpr int kMap2Depth = 8;                               // reduction steps with their loads in flight, per wavefront
+constexpr int kMap2RedBytes = 4 * 64 * 16 * 4;              // sums of the second reduction half
+constexpr int kMap2StageBytes = 8 * kMap2Depth * 1024;      // kWT: filter blocks in flight, all wavefronts
+constexpr size_t map2_lds_bytes(bool wt) { return static_cast<size_t>(kMap2RedBytes) + 64 + (wt ? kMap2StageBytes : 0); }
+
+template <bool kFused, bool kWT>
+__global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int itiles) {
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];
+  int* const red = reinterpret_cast<int*>(smem);                                      // [p][4][64] x 16 bytes
+  uint32_t* const words = reinterpret_cast<uint32_t*>(smem + kMap2RedBytes);          // 4 maxima, the range
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int p = wave & 3, rh = wave >> 2;
+  const int lr = lane & 31, lk = lane >> 5;
+  // consecutive workgroups go to consecutive dies: give each die a contiguous range of tiles, so that the tiles
+  // sharing a block of the filter (same output channels) read it through one L2
+  const int nb = gridDim.x;
+  const int b = (nb & 7) == 0 ? (blockIdx.x & 7) * (nb >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+  const int kt = b / itiles, it = b - kt * itiles;      // 32-channel tile, 32-image tile
+  const int n = it * 32 + lr;
+
+  const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.x), 0, a.x_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.wp), 0, a.wp_bytes, 0x00020000);
+
+  // this wavefront's channel slices and its reduction steps (slice, input pixel)
+  const int half0 = (a.cslices + 1) >> 1;
+  const int cs0 = rh == 0 ? 0 : half0;
+  const int nsteps = (rh == 0 ? half0 : a.cslices - half0) * 4;
+  const int py = p >> 1, px = p & 1;
+  const int a_base = n < a.N ? n * 4 * a.C + lk * 16 : kOob;
+  // filter fragment of this lane inside a 1 KB block (32 rows of 32 bytes, 16-byte halves swapped in odd groups of 8 rows)
+  int w_frag[2];
+  if (kWT) {
+    const int j16 = lane & 15, gg = (lane >> 4) & 1;
+#pragma unroll
+    for (int o = 0; o < 2; ++o) {
+      const int krow = 16 * lk + 8 * o + (j16 >> 1);
+      w_frag[o] = krow * 32 + ((gg ^ ((krow >> 3) & 1)) << 4) + 8 * (j16 & 1);
+    }
+  } else {
+    w_frag[0] = w_frag[1] = lr * 32 + ((lk ^ ((lr >> 3) & 1)) << 4);
+  }
+  int8_t* const stage = smem + kMap2RedBytes + 64 + wave * (kMap2Depth * 1024);
+
+  v4i fa[kMap2Depth], fw[kMap2Depth];
+  // Loads of step s into slot u.  Steps past the wavefront's last one are issued all the same, with out-of-range
+  // offsets (zeros, no memory traffic): the loop body is free of branches, so the number of loads in flight behind
+  // any load is a constant - for the compiler's wait counts as for those written by hand below.
+  auto issue = [&](int s, int u) {
+    const int cs = cs0 + (s >> 2), q = s & 3;
+    const int tap = ((q >> 1) - py + 1) * 3 + (q & 1) - px + 1;
+    const bool live = s < nsteps;
+    int aoff = kOob;
+    if (live && a_base != kOob && cs * 32 + lk * 16 < a.C) aoff = a_base + q * a.C + cs * 32;
+    fa[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, aoff, 0, 0);
+    if (kWT) {
+      // forward copy [reduction group of 64][this launch's output slice][flipped tap][64 rows][32 bytes]
+      const int blk = (((cs >> 1) * a.src_cslices + kt) * 9 + 8 - tap) * 2048 + (cs & 1) * 1024;
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(stage + u * 1024), 16, live ? blk + lane * 16 : kOob, 0, 0, 0);
+      asm volatile("" ::: "memory");   // both loads leave here, in this order
+    } else {
+      const int blk = (((kt >> 1) * a.cslices + cs) * 9 + tap) * 2048 + (kt & 1) * 1024;
+      fw[u] = __builtin_amdgcn_raw_buffer_load_b128(rw, live ? blk + w_frag[0] : kOob, 0, 0);
+    }
+  };
+
+  v16i acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+#pragma unroll
+  for (int u = 0; u < kMap2Depth; ++u) issue(u, u);
+  for (int base = 0; base < nsteps; base += kMap2Depth) {
+#pragma unroll
+    for (int u = 0; u < kMap2Depth; ++u) {
+      if (kWT) {
+        // two loads per step, completing in order: all but those of the seven younger steps have landed
+        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (kMap2Depth - 1)));
+        asm volatile("" ::: "memory");
+        const unsigned src = lds_addr(stage + u * 1024);
+        const v2i lo = lds_read_tr8<0>(src + w_frag[0]);
+        const v2i hi = lds_read_tr8<0>(src + w_frag[1]);
+        lds_settle<0>();   // also: the slot is read out before the next block is sent to it
+        fw[u] = lds_landed(lo, hi);
+      }
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[u], fa[u], acc, 0, 0, 0);
+      issue(base + u + kMap2Depth, u);
+    }
+  }
+  __builtin_amdgcn_s_waitcnt(0x0F70);   // the (empty) loads issued ahead of the last steps
+  asm volatile("" ::: "memory");
+
+  // ---- add the two reduction halves: acc[4g + e] = channel kt*32 + 8g + 4*lk + e of image n, pixel p
+  if (rh == 1) {
+#pragma unroll
+    for (int g = 0; g < 4; ++g)
+      *reinterpret_cast<v4i*>(red + ((p * 4 + g) * 64 + lane) * 4) = v4i{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
+  }
+  __syncthreads();
+  const bool roundtrip = (a.flags & NITI_EPI_F32_ROUNDTRIP) != 0;
+  if (rh == 0) {
+    uint32_t lmax = 0;
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const v4i o = *reinterpret_cast<const v4i*>(red + ((p * 4 + g) * 64 + lane) * 4);
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        int v = acc[4 * g + e] + o[e];
+        if (roundtrip) v = f32_roundtrip(v);
+        acc[4 * g + e] = v;
+        const uint32_t m = uabs(v);
+        lmax = m > lmax ? m : lmax;
+      }
+    }
+    lmax = wave_max_u32(lmax);
+    if (lane == 0) words[wave] = lmax;
+  }
+  __syncthreads();
+  const long long row = (static_cast<long long>(n) * 4 + p) * a.K;   // first output element of (image, pixel)
+  const int ch = kt * 32 + 4 * lk;                                   // + 8g
+  if constexpr (!kFused) {
+    if (rh == 0) {
+      const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int c = ch + 8 * g;
+        const int off = (n < a.N && c < a.K) ? static_cast<int>((row + c) * 4) : kOob;
+        __builtin_amdgcn_raw_buffer_store_b128(v4i{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]}, ry, off, 0, 0);
+      }
+    }
+    if (a.absmax != nullptr && wave == 0) fold_absmax(a.absmax, lane < 4 ? words[lane] : 0u);
+  } else {
+    // ---- tensor-wide range: workgroup maximum -> own slot -> maximum over the slots of all workgroups
+    if (wave == 0) {
+      uint32_t bmax = lane < 4 ? words[lane] : 0u;
+      bmax = wave_max_u32(bmax);
+      uint32_t* const slots = a.sync + kSyncSlot0;
+      if (lane == 0) __hip_atomic_store(slot_word(slots, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
+      if (lane == 0) words[4] = g != 0u ? g - 1u : 0u;
+    }
+    __syncthreads();
+    const uint32_t gmax = words[4];
+    const int shift = max(bitwidth_of(gmax, a.bw_mode) - a.target_bits, 0);
+    if (rh == 0) {
+      const bool trunc = a.trunc != 0;
+      const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
+      const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
+      const bool fast = shift >= 1 && !trunc && !psto;
+      const int sm1 = shift - 1, lo = relu ? 0 : -127;
+      const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y8, 0, a.y8_bytes, 0x00020000);
+      const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask != nullptr ? a.mask : a.y8), 0, a.y8_bytes, 0x00020000);
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        int r[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int x = acc[4 * g + e];
+          if (fast) {
+            r[e] = round_nearest_floor_fast(x, sm1, lo);
+          } else {
+            if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
+            else r[e] = wrap_to_i8(x);
+            if (relu && r[e] < 0) r[e] = 0;
+          }
+        }
+        uint32_t v = pack4_i8(r[0], r[1], r[2], r[3]);
+        const int c = ch + 8 * g;
+        const int off = (n < a.N && c < a.K) ? static_cast<int>(row + c) : kOob;
+        if (a.mask != nullptr)   // ReLU backward of the layer below, folded in: its output is this layer's input
+          v &= positive_bytes(static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b32(rm, off, 0, 0)));
+        __builtin_amdgcn_raw_buffer_store_b32(v, ry, off, 0, 0);
+      }
+    }
+    if (blockIdx.x == 0 && tid == 0) {
+      a.sync[0] = gmax;
+      if (a.shift_out != nullptr) *a.shift_out = shift;
+      if (a.exp_out != nullptr) *a.exp_out = shift + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+    }
+  }
+}
+
 // Filter arrangement for the kernel above.  mode 0 (forward): F(k, tap, c) = w[k][tap][c], w is [K][9][C].
 // mode 1 (data gradient): the roles of the channel dimensions swap and the taps flip:
 // F(k', tap, c') = w[c'][8 - tap][k'], with k' < C and c' < K of the original filter.
@@ -564,7 +817,6 @@ __global__ __launch_bounds__(256) void halo_filter_prepare_kernel(const int8_t* 
 // Channel tile of a launch: 128 unless that leaves fewer workgroups than the device runs at once while
 // a tile of 64 would give it more to do.
 int halo_ktile(long long pix, int K, int H) {
-  if (H == 2) return 128;   // the 2 x 2 maps' halo tile leaves room for the wide tile's filter ring only
   static int cus = 0;
   if (cus == 0) {
     int dev = 0;
@@ -609,15 +861,43 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
   return check_launch("conv3x3_halo");
 }
 
+inline int map2_blocks(int N, int K) { return ((N + 31) / 32) * ((K + 31) / 32); }
+
+template <bool kFused, bool kWT>
+int launch_map2(const HaloArgs& a, hipStream_t stream) {
+  constexpr size_t lds = map2_lds_bytes(kWT);
+  auto k = conv3x3_map2_kernel<kFused, kWT>;
+  static bool attr_set = false;
+  static int resident = 0;  // workgroups the device holds at once
+  if (!attr_set) {
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
+      return fail(NITI_ERR_LAUNCH, "conv3x3_map2: cannot reserve %zu bytes of LDS", lds);
+    if (kFused) {
+      int dev = 0, cus = 0, per_cu = 0;
+      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+          hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(k), 512, lds) != hipSuccess)
+        return fail(NITI_ERR_LAUNCH, "conv3x3_map2: cannot query occupancy");
+      resident = cus * per_cu;
+    }
+    attr_set = true;
+  }
+  const int itiles = (a.N + 31) / 32;
+  const int nb = map2_blocks(a.N, a.K);
+  if (kFused && nb > resident)
+    return fail(NITI_ERR_UNSUPPORTED, "conv3x3_map2: %d workgroups do not fit on the device at once (%d)", nb, resident);
+  hipLaunchKernelGGL(k, dim3(nb), dim3(512), lds, stream, a, itiles);
+  return check_launch("conv3x3_map2");
+}
+
 template <bool kFused, bool kWT>
 int launch_halo_tiles(const HaloArgs& a, int H, hipStream_t stream) {
+  if (H == 2) return launch_map2<kFused, kWT>(a, stream);
   const int ktile = halo_ktile(static_cast<long long>(a.N) * H * H, a.K, H);
   if (ktile == 128) {
     if (H == 32) return launch_halo<32, 8, 1, 128, kFused, kWT>(a, stream);
     if (H == 16) return launch_halo<16, 16, 1, 128, kFused, kWT>(a, stream);
     if (H == 8) return launch_halo<8, 8, 4, 128, kFused, kWT>(a, stream);
-    if (H == 4) return launch_halo<4, 4, 16, 128, kFused, kWT>(a, stream);
-    return launch_halo<2, 2, 64, 128, kFused, kWT>(a, stream);
+    return launch_halo<4, 4, 16, 128, kFused, kWT>(a, stream);
   }
   if (H == 32) return launch_halo<32, 8, 1, 64, kFused, kWT>(a, stream);
   if (H == 16) return launch_halo<16, 16, 1, 64, kFused, kWT>(a, stream);
@@ -653,7 +933,7 @@ bool conv3x3_halo_supported(int N, int H, int W, int C, int K, int R, int S, int
   if (H != 2 && H != 4 && H != 8 && H != 16 && H != 32) return false;
   if (C % 16 != 0 || K % 4 != 0) return false;
   const long long pix = static_cast<long long>(N) * H * W;
-  if (pix % 256 != 0) return false;  // workgroups own whole rows / whole images
+  if (H != 2 && pix % 256 != 0) return false;  // workgroups own whole rows / whole images (2 x 2 maps: any batch)
   if (pix * C >= 0x7fffffffLL || pix * K * 4 >= 0x7fffffffLL) return false;
   if (conv3x3_halo_filter_bytes(C, K) >= 0x7fffffffULL) return false;
   return true;
@@ -687,7 +967,7 @@ int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S,
   if (!conv3x3_halo_supported(N, H, W, C, K, R, S, stride, pad) || K % 16 != 0) return 0;
   const long long pix = static_cast<long long>(N) * H * W;
   const int ktile = halo_ktile(pix, K, H);
-  const long long nb = (pix / 256) * ((K + ktile - 1) / ktile);
+  const long long nb = H == 2 ? map2_blocks(N, K) : (pix / 256) * ((K + ktile - 1) / ktile);
   return nb <= 2048 ? static_cast<int>(nb) : 0;  // the device check happens at launch; this bounds the workspace
 }
 

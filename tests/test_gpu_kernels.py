@@ -106,7 +106,8 @@ def test_conv_dgrad(dev, case):
 
 # convolution + requantisation in one launch: N,Q,C,K (3x3, stride 1, pad 1), small sums / large sums / ragged tiles
 FUSED_CASES = [(4, 8, 16, 16), (4, 8, 64, 128), (8, 8, 80, 144), (1, 16, 16, 48), (3, 16, 192, 272), (2, 32, 16, 64),
-               (8, 32, 128, 128), (12, 8, 512, 128), (16, 4, 64, 128), (48, 4, 256, 80), (64, 2, 512, 512), (128, 2, 32, 48)]
+               (8, 32, 128, 128), (12, 8, 512, 128), (16, 4, 64, 128), (48, 4, 256, 80), (64, 2, 512, 512), (128, 2, 32, 48),
+               (5, 2, 48, 16), (33, 2, 16, 80), (256, 2, 160, 96), (1, 2, 96, 32)]
 
 
 @pytest.fixture(params=["auto", "64", "128"])
@@ -124,7 +125,8 @@ def halo_tile(request):
 
 
 @pytest.mark.parametrize("case", [(8, 8, 64, 128), (4, 8, 80, 24), (3, 16, 192, 260), (2, 32, 16, 64), (8, 32, 128, 256), (12, 8, 512, 128),
-                                  (32, 4, 128, 256), (16, 4, 48, 16), (64, 2, 256, 128), (192, 2, 64, 32)])
+                                  (32, 4, 128, 256), (16, 4, 48, 16), (64, 2, 256, 128), (192, 2, 64, 32),
+                                  (7, 2, 48, 20), (40, 2, 16, 132), (1, 2, 32, 4)])
 def test_conv_halo_tiles(dev, case, halo_tile):
     """Forward, data gradient and the requantising variant with both channel tiles of the halo kernel."""
     from niti_amd import ops
@@ -156,6 +158,11 @@ def test_conv_halo_tiles(dev, case, halo_tile):
         assert torch.equal(dx.cpu(), dref)
         dx8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), forward_filter=wf)
         assert int(sync.cpu()[1]) == 0 and torch.equal(dx8.cpu(), d8) and int(sh.cpu()) == dsh
+        # ... and zeroing the gradient where the layer's input was not positive
+        mask = ri8(g, N, Q, Q, C)
+        dx8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), forward_filter=wf, relu_mask=mask.to(dev))
+        assert int(sync.cpu()[1]) == 0 and int(sh.cpu()) == dsh
+        assert torch.equal(dx8.cpu(), torch.where(mask > 0, d8, torch.zeros_like(d8)))
 
 
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
