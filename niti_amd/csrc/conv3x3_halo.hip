@@ -312,6 +312,8 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     auto tap_ready = [&](auto sc) {
       if constexpr (kWT) {
         constexpr int s = decltype(sc)::value;
+        // the products of the tap before stay ahead of this wait (nothing else orders them against it)
+        if (s > 0) __builtin_amdgcn_sched_barrier(0);
         lds_settle<(2 - s) * 2 * NWF>();
         if (s == 0) {
 #pragma unroll

@@ -250,6 +250,33 @@ def test_shims_match_reference_conventions():
     assert hasattr(int8conv_cuda, "group_conv") and hasattr(cutlassconv_cuda, "weight_grad")
 
 
+def test_epoch_driver_learns_and_checkpoints(tt, tmp_path):
+    """The epoch driver (regime, train pass, evaluation pass, checkpoint files) on a synthetic ten-class task: the
+    integer step must actually learn (chance is 10 %), and a checkpoint loaded into a fresh model must reproduce
+    the trained model's outputs bit for bit."""
+    import os
+    from niti_amd import train
+    from niti_amd.ti_vgg import TiVGG_cifar
+    _say("epoch_driver")
+    torch.manual_seed(3)
+    model = TiVGG_cifar(depth=7)
+    model.regime = [{'epoch': 0, 'gb': 5}, {'epoch': 3, 'gb': 4}]
+    tr, te = train.synthetic_loaders(128, train_batches=16, test_batches=4, noise=0.5, seed=1)
+    hist = train.fit(model, tr, te, epochs=4, save_path=str(tmp_path), save_all=True)
+    assert [h['grad_bitwidth'] for h in hist] == [5, 5, 5, 4]
+    assert hist[0]['val_prec1'] < 60.0 and max(h['val_prec1'] for h in hist) > 80.0, hist
+    assert sorted(os.listdir(tmp_path)) == ['checkpoint_epoch_0.pth.tar', 'checkpoint_epoch_1.pth.tar', 'checkpoint_epoch_2.pth.tar',
+                                            'checkpoint_epoch_3.pth.tar', 'ckpt.pth', 'model_best.pth.tar']
+    fresh = TiVGG_cifar(depth=7)
+    ckpt = train.load_checkpoint(fresh, os.path.join(tmp_path, 'ckpt.pth'))
+    assert ckpt['epoch'] == 3 and ckpt['best_prec1'] == hist[-1]['best_prec1']
+    tt.TRAINING = False
+    x, _ = next(iter(te))
+    out_a, exp_a = model(x.to("cuda:0"))
+    out_b, exp_b = fresh(x.to("cuda:0"))
+    assert torch.equal(out_a, out_b) and _ei(exp_a) == _ei(exp_b)
+
+
 def test_grid_wide_wait_gives_up_and_says_so():
     """With a wait limit of one clock tick (set from the host, in a process of its own because the library reads
     the limit once) the single-launch kernels do not wait for late workgroups: every workgroup still runs to its
