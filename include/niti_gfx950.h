@@ -118,9 +118,10 @@ int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N,
  * but the int32 sums stay in registers: every workgroup publishes the largest magnitude of its tile,
  * waits for all others, derives the tensor-wide shift and stores int8.
  *
- * Covered: 3x3, stride 1, pad 1, square inputs of side 8, 16 or 32, N*H*W % 256 == 0, input channels % 16 == 0,
- * output channels % 16 == 0, rounding NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC, and a launch whose
- * workgroups (N*H*W/256 x ceil(out channels/128)) all fit on the device at once.  niti_conv2d_i8_requant_sync_words
+ * Covered: 3x3, stride 1, pad 1, square inputs of side 2, 4, 8, 16 or 32, N*H*W % 256 == 0 (side 2: any N), input
+ * channels % 16 == 0, output channels % 16 == 0, rounding NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC, and a
+ * launch whose workgroups (N*H*W/256 x ceil(out channels/128 or 64); side 2: ceil(N/32) x ceil(out channels/32)) all
+ * fit on the device at once.  niti_conv2d_i8_requant_sync_words
  * returns 0 for shapes outside that (then use the two-pass entry points); the entry points return
  * NITI_ERR_UNSUPPORTED for them and for a device too small for the launch.
  *
@@ -173,8 +174,9 @@ int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int 
  * tensor-wide range is exchanged between the workgroups of the finishing kernel, and
  *   g = round(dw >> max(bitwidth(max|dw|) - mu, 0)),  w = clip(w - g, +-127).
  *
- * Covered: the shapes of the native 3x3 weight-gradient kernel (3x3, stride 1, pad 1, square maps of side 8, 16
- * or 32, C % 16 == 0, K % 16 == 0, N*H*W % 128 == 0, even N for side 8) with K*9*C <= 4M, rounding
+ * Covered: the shapes of the native 3x3 weight-gradient kernel (3x3, stride 1, pad 1, square maps of side 2, 4, 8,
+ * 16 or 32, C % 16 == 0, K % 16 == 0, N*H*W % 128 == 0, even N for side 8, N*H*W % 256 == 0 for sides 2 and 4) with
+ * K*9*C <= 4M, rounding
  * NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC.  niti_conv2d_i8_wgrad_update_sync_words returns 0 otherwise.
  *
  * act: [N,H,W,C] int8 (C may include zero channel padding); err: [N,H,W,K] int8; w: [K,3,3,w_channels] int8,
