@@ -21,13 +21,12 @@
 #include <stdlib.h>
 
 #include "common.h"
+#include "lds_asm.h"
 #include "requant_math.h"
 
 namespace niti {
 namespace {
 
-#define NITI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
-typedef int v2i_t __attribute__((ext_vector_type(2)));
 constexpr int kOob = -1;
 
 template <int N>
@@ -67,6 +66,63 @@ __device__ inline WorkItem die_local_work_item() {
   w.y = p % gy;
   w.z = p / gy;
   return w;
+}
+
+// One stage of the main loop: four reduction steps of 32 pixels x three filter rows x three taps, all fragments by
+// transposing LDS reads.  The reads are inline assembly (see lds_asm.h: the builtin form would wait for the loads
+// of the following stages, just issued, before every read) and run one filter row ahead of the MFMAs: row i + 1 is
+// requested, then the wait leaves exactly those requests in flight, then row i multiplies.
+// a_base: error-tile offsets of the lane's two 8-byte rows (reduction step 0); b_base: halo-tile offsets of its rows
+// (reduction step 0, filter row 0); ROWB: bytes of a halo row.  kShiftTaps: the second and third tap of a filter row
+// are byte shifts of the first one's pixel sequence (rows of at least 8 pixels), otherwise every tap is read.
+template <int Q, int BR, int HR, int ROWB, bool kShiftTaps, int NB>
+__device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const int (&b_base)[NB], v16i (&acc)[9]) {
+  v2i alo[2], ahi[2];   // [reduction step & 1]
+  v2i rd[2][NB];        // [row step & 1]
+  v4i af[2];
+  auto request = [&](auto stepc) {
+    constexpr int step = decltype(stepc)::value;
+    constexpr int ks = step / 3, r = step % 3;
+    constexpr int prow = ks * 32 / Q;                         // first output row of this reduction step inside the tile
+    constexpr int hrow0 = (prow / BR) * HR + (prow % BR);     // its halo row for filter row 0
+    if constexpr (r == 0) {
+      alo[ks & 1] = lds_read_tr8<ks * 4096>(sbase + a_base[0]);
+      ahi[ks & 1] = lds_read_tr8<ks * 4096>(sbase + a_base[1]);
+    }
+#pragma unroll
+    for (int q = 0; q < NB; ++q) rd[step & 1][q] = lds_read_tr8<(hrow0 + r) * ROWB>(sbase + b_base[q]);
+  };
+  request(std::integral_constant<int, 0>{});
+  static_for<12>([&](auto stepc) {
+    constexpr int step = decltype(stepc)::value;
+    constexpr int ks = step / 3, r = step % 3;
+    if constexpr (step + 1 < 12) request(std::integral_constant<int, step + 1>{});
+    lds_settle<(step + 1 < 12) ? NB + ((step + 1) % 3 == 0 ? 2 : 0) : 0>();
+    if constexpr (r == 0) af[ks & 1] = lds_landed(alo[ks & 1], ahi[ks & 1]);
+    v2i (&d)[NB] = rd[step & 1];
+#pragma unroll
+    for (int q = 0; q < NB; ++q) asm volatile("" : "+v"(d[q]));
+    const v4i a4 = af[ks & 1];
+    if constexpr (!kShiftTaps) {
+#pragma unroll
+      for (int s = 0; s < 3; ++s)
+        acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, v4i{d[2 * s][0], d[2 * s][1], d[2 * s + 1][0], d[2 * s + 1][1]},
+                                                               acc[r * 3 + s], 0, 0, 0);
+    } else {
+      // the byte sequences the two 8-pixel halves are cut from: [d0 d1 d2] and [e0 e1 e2] (dwords)
+      const int d0 = d[0][0], d1 = d[0][1], d2 = d[1][0];
+      const int e0 = Q >= 16 ? d[1][0] : d[2][0], e1 = Q >= 16 ? d[1][1] : d[2][1];
+      const int e2 = d[NB - 1][0];
+      acc[r * 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, v4i{d0, d1, e0, e1}, acc[r * 3], 0, 0, 0);
+#pragma unroll
+      for (int s = 1; s < 3; ++s) {
+        const v4i bf = {static_cast<int>(__builtin_amdgcn_alignbyte(d1, d0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(d2, d1, s)),
+                        static_cast<int>(__builtin_amdgcn_alignbyte(e1, e0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(e2, e1, s))};
+        acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, bf, acc[r * 3 + s], 0, 0, 0);
+      }
+    }
+    __builtin_amdgcn_sched_barrier(0);   // the next row's requests and wait stay behind these products
+  });
 }
 
 // Q: image width = height; BR: output rows of one image per band; NI: images per band; BR*NI*Q == 128
@@ -216,37 +272,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
     else wg_wait_vmcnt<0>();
     wg_sync();
     if (it + STAGES - 1 < nb) issue(band_begin + it + STAGES - 1, (it + STAGES - 1) % STAGES);
-    const int8_t* sbase = smem + (it % STAGES) * G::STAGE_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const int prow = ks * 32 / Q;                         // first output row of this reduction step inside the band
-      const int hrow0 = (prow / BR) * G::HR + (prow % BR);  // its halo row for filter row 0
-      const v2i_t alo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[0] + ks * 4096));
-      const v2i_t ahi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[1] + ks * 4096));
-      const v4i af = v4i{alo[0], alo[1], ahi[0], ahi[1]};
-#pragma unroll
-      for (int r = 0; r < 3; ++r) {
-        const int roff = (hrow0 + r) * G::RP * 64;
-        v2i_t rd[NB];
-#pragma unroll
-        for (int q = 0; q < NB; ++q)
-          rd[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(sbase + b_base[q] + roff));
-        // the byte sequences the two 8-pixel halves are cut from: [d0 d1 d2] and [e0 e1 e2] (dwords)
-        const int d0 = rd[0][0], d1 = rd[0][1];
-        const int d2 = Q >= 16 ? rd[1][0] : rd[1][0];
-        const int e0 = Q >= 16 ? rd[1][0] : rd[2][0], e1 = Q >= 16 ? rd[1][1] : rd[2][1];
-        const int e2 = rd[NB - 1][0];
-        acc[r * 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{d0, d1, e0, e1}, acc[r * 3], 0, 0, 0);
-#pragma unroll
-        for (int s = 1; s < 3; ++s) {
-          const v4i bf = {static_cast<int>(__builtin_amdgcn_alignbyte(d1, d0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(d2, d1, s)),
-                          static_cast<int>(__builtin_amdgcn_alignbyte(e1, e0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(e2, e1, s))};
-          acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[r * 3 + s], 0, 0, 0);
-        }
-      }
-    }
+    wgrad_stage<Q, BR, G::HR, G::RP * 64, true, NB>(lds_addr(smem + (it % STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
   }
 
   // ---- partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+wc*32+(lane&31)]
@@ -420,42 +446,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
     else wg_wait_vmcnt<0>();
     wg_sync();
     if (it + G::STAGES - 1 < nb) issue(band_begin + it + G::STAGES - 1, (it + G::STAGES - 1) % G::STAGES);
-    const int8_t* sbase = smem + (it % G::STAGES) * G::STAGE_BYTES;
-#pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
-      const int prow = ks * 32 / Q;                         // first output row of this step inside the pixel half
-      const int hrow0 = (prow / BR) * G::HR + (prow % BR);  // its halo row for filter row 0
-      const v2i_t alo = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[0] + ks * 4096));
-      const v2i_t ahi = __builtin_amdgcn_ds_read_tr8_b64_v2i32(
-          (__attribute__((address_space(3))) v2i_t*)(sbase + a_base[1] + ks * 4096));
-      const v4i af = v4i{alo[0], alo[1], ahi[0], ahi[1]};
-#pragma unroll
-      for (int r = 0; r < 3; ++r) {
-        const int roff = (hrow0 + r) * G::RP * 32;
-        v2i_t rd[NB];
-#pragma unroll
-        for (int q = 0; q < NB; ++q)
-          rd[q] = __builtin_amdgcn_ds_read_tr8_b64_v2i32((__attribute__((address_space(3))) v2i_t*)(sbase + b_base[q] + roff));
-        if constexpr (!kShiftTaps) {
-#pragma unroll
-          for (int s = 0; s < 3; ++s)
-            acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{rd[2 * s][0], rd[2 * s][1], rd[2 * s + 1][0], rd[2 * s + 1][1]},
-                                                                   acc[r * 3 + s], 0, 0, 0);
-        } else {
-          const int d0 = rd[0][0], d1 = rd[0][1], d2 = rd[1][0];
-          const int e0 = Q >= 16 ? rd[1][0] : rd[2][0], e1 = Q >= 16 ? rd[1][1] : rd[2][1];
-          const int e2 = rd[NB - 1][0];
-          acc[r * 3] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, v4i{d0, d1, e0, e1}, acc[r * 3], 0, 0, 0);
-#pragma unroll
-          for (int s = 1; s < 3; ++s) {
-            const v4i bf = {static_cast<int>(__builtin_amdgcn_alignbyte(d1, d0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(d2, d1, s)),
-                            static_cast<int>(__builtin_amdgcn_alignbyte(e1, e0, s)), static_cast<int>(__builtin_amdgcn_alignbyte(e2, e1, s))};
-            acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, bf, acc[r * 3 + s], 0, 0, 0);
-          }
-        }
-      }
-    }
+    wgrad_stage<Q, BR, G::HR, G::RP * 32, kShiftTaps, NB>(lds_addr(smem + (it % G::STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
   }
 
   // ---- add the two pixel halves: half 1 -> LDS -> half 0 -> memory.  Slot layout [value][lane].
