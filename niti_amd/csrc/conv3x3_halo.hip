@@ -312,6 +312,84 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
   };
 
+  // A whole slice (three filter rows) from one stage, for the pipeline with one slice per stage.  All fragment reads
+  // are inline assembly and run one filter row ahead of the products: row r + 1 is requested, then the wait leaves
+  // exactly those requests in flight, then row r multiplies - so only the first row of a stage waits for LDS.  (Left
+  // to itself the compiler keeps the fragments in few registers and alternates read, wait, product.)
+  auto stage_rows = [&](unsigned saa, unsigned swa) {
+    constexpr int PER_TAP = NWF * (kWT ? 2 : 1);
+    constexpr int ROW_READS = 2 + 3 * PER_TAP;
+    static_assert(ROW_READS <= 15, "the wait counter holds 15");
+    v4i pcb[2][2];
+    v4i wfb[2][3][NWF];
+    v2i tlo[2][3][NWF], thi[2][3][NWF];
+    auto request = [&](auto rc) {
+      constexpr int r = decltype(rc)::value;
+      constexpr int b = r & 1;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) pcb[b][j] = lds_read_b128_at<r * G::RP * 32>(saa + (p_addr[j] ^ ((r & 1) << 4)));
+      static_for<3>([&](auto sc) {
+        constexpr int s = decltype(sc)::value;
+        constexpr int off = ((s + 1) % 3 + 3 * r) * TAPB;
+#pragma unroll
+        for (int i = 0; i < NWF; ++i) {
+          if constexpr (kWT) {
+            tlo[b][s][i] = lds_read_tr8<off>(swa + w_addr[i][0]);
+            thi[b][s][i] = lds_read_tr8<off>(swa + w_addr[i][kWT ? 1 : 0]);
+          } else {
+            wfb[b][s][i] = lds_read_b128_at<off>(swa + w_addr[i][0]);
+          }
+        }
+      });
+    };
+    request(std::integral_constant<int, 0>{});
+    static_for<3>([&](auto rc) {
+      constexpr int r = decltype(rc)::value;
+      constexpr int b = r & 1;
+      if constexpr (r < 2) request(std::integral_constant<int, r + 1>{});
+      lds_settle<(r < 2) ? ROW_READS : 0>();
+      v4i pc[2], wf[3][NWF];
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        pc[j] = pcb[b][j];
+        asm volatile("" : "+v"(pc[j]));
+      }
+#pragma unroll
+      for (int s = 0; s < 3; ++s)
+#pragma unroll
+        for (int i = 0; i < NWF; ++i) {
+          if constexpr (kWT) {
+            wf[s][i] = lds_landed(tlo[b][s][i], thi[b][s][i]);
+          } else {
+            wf[s][i] = wfb[b][s][i];
+            asm volatile("" : "+v"(wf[s][i]));
+          }
+        }
+#pragma unroll
+      for (int i = 0; i < NWF; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
+      v4i ps[2];
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
+#pragma unroll
+      for (int i = 0; i < NWF; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
+#pragma unroll
+      for (int i = 0; i < NWF; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);   // the next row's requests and wait stay behind these products
+    });
+  };
+
   if constexpr (G::RPS == 1) {
     // ---- pipeline, one filter row per stage.  Stage t = 3 * slice + filter row.  Per-wavefront load order: act(0),
     // W(0), W(1); inside stage t after its barrier: W(t+2), then - in the first stage of a slice - act(next slice).
@@ -354,8 +432,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (ci + 1 < a.cslices) issue_act(ci + 1, (ci + 1) & 1);
       if (ci + 2 < a.cslices) issue_w(ci + 2, 0, (ci + 2) % G::WSTAGES);
       const int8_t* sw = w_buf + (ci % G::WSTAGES) * G::W_BYTES;
-#pragma unroll
-      for (int r = 0; r < 3; ++r) filter_row(sa, sw + r * 3 * TAPB, r);
+      stage_rows(lds_addr(sa), lds_addr(sw));
     }
   }
 

@@ -24,6 +24,12 @@ __device__ inline v4i lds_read_b128(unsigned addr) {
   asm volatile("ds_read_b128 %0, %1" : "=v"(r) : "v"(addr));
   return r;
 }
+template <int OFF>
+__device__ inline v4i lds_read_b128_at(unsigned addr) {
+  v4i r;
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=v"(r) : "v"(addr), "n"(OFF));
+  return r;
+}
 template <int N>
 __device__ inline void lds_settle() {
   asm volatile("s_waitcnt lgkmcnt(%0)" ::"n"(N));
