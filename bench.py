@@ -205,7 +205,7 @@ def cpu_baseline(min_seconds=10.0):
             "sample": "%d pass(es) of the full six-layer conv triple at batch %d (plain-C oracle, OpenMP), %.1f s" % (passes, BATCH, t_total)}
 
 
-def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH):
+def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH, graph=True):
     """images/s of a complete integer training step: VGG-small (six conv + FC), batch 128 (configs[3]), or the
     ten-convolution VGG-13 widths, batch 256 (configs[4])."""
     import torch
@@ -225,7 +225,7 @@ def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH):
         net.forward_int8(x, 0)
         net.backward(target)
 
-    run, mode = make_runner(one, warmup)
+    run, mode = make_runner(one, warmup, graph)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for _ in range(steps):
@@ -235,6 +235,21 @@ def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH):
     return batch / dt, dt * 1e3, mode
 
 
+TRAIN_STEPS = (("train_step", 7, BATCH, "BASELINE configs[3]: VGG-small (6 conv + FC) integer training step, batch 128"),
+               ("train_step_vgg13", 13, 256, "BASELINE configs[4]: VGG-13 widths (10 conv + FC) integer training step, batch 256"))
+
+
+def train_step_objects(dev, steps, warmup, graph=True):
+    out = {}
+    for name, depth, batch, workload in TRAIN_STEPS:
+        try:
+            ips, ms, mode = train_step_rate(dev, steps, warmup, depth, batch, graph)
+            out[name] = {"workload": workload, "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": mode}
+        except Exception as e:  # the headline line must still be printed
+            out[name] = {"error": str(e)[:200]}
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -242,6 +257,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train-step", action="store_true")
+    ap.add_argument("--train-steps-only", action="store_true",
+                    help="run only the two training-step workloads and print their objects (for kernel traces of a step)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a kernel of known traffic, to scale "
@@ -267,6 +284,10 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.train_steps_only:
+        print(json.dumps(train_step_objects(dev, args.steps, args.warmup, not args.eager)))
+        return 0
 
     wl = ConvTriple(dev)
     run, mode = make_runner(wl.step, args.warmup, not args.eager)
@@ -329,12 +350,7 @@ def main():
            "pct_int8_mfma_peak": round(100.0 * tops / INT8_MFMA_PEAK_TOPS, 2),
            "roofline": roofline}
     if not args.no_train_step:
-        ips, ms, tmode = train_step_rate(dev, max(args.steps, 5), max(args.warmup, 2))
-        out["train_step"] = {"workload": "BASELINE configs[3]: VGG-small (6 conv + FC) integer training step, batch 128",
-                             "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": tmode}
-        ips, ms, tmode = train_step_rate(dev, max(args.steps, 5), max(args.warmup, 2), depth=13, batch=256)
-        out["train_step_vgg13"] = {"workload": "BASELINE configs[4]: VGG-13 widths (10 conv + FC) integer training step, batch 256",
-                                   "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": tmode}
+        out.update(train_step_objects(dev, max(args.steps, 5), max(args.warmup, 2)))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
