@@ -554,6 +554,38 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   // read before this workgroup fills its slot: workgroup 0 overwrites the word only after all slots are filled
   const int predicted = (a.predict != 0 && a.shift_out != nullptr) ? max(*a.shift_out, 0) : 0;
+  v4i fin[OWN];
+  uint32_t lmax = 0;
+  // Every wavefront has columns of its own at least in the first round (uniform over the grid): then each adds all
+  // slices of its own columns and nothing goes through LDS.  With fewer columns than wavefronts the slices are
+  // shared instead (phases 1 and 2 below), so that no wavefront idles while another walks over all slices.
+  const bool direct = a.nv >= static_cast<long long>(NW) * gridDim.x * 64;
+  if (direct) {
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int v = j * NW + wave;
+      const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
+      v4i s = {0, 0, 0, 0};
+      if (v < kFinishV && col < a.nv) {
+        int z = 0;
+        for (; z + 3 < a.splits; z += 4) {
+          const v4i v0 = reinterpret_cast<const v4i*>(a.partial + (z + 0) * a.slice_stride)[col];
+          const v4i v1 = reinterpret_cast<const v4i*>(a.partial + (z + 1) * a.slice_stride)[col];
+          const v4i v2 = reinterpret_cast<const v4i*>(a.partial + (z + 2) * a.slice_stride)[col];
+          const v4i v3 = reinterpret_cast<const v4i*>(a.partial + (z + 3) * a.slice_stride)[col];
+          s += (v0 + v1) + (v2 + v3);
+        }
+        for (; z < a.splits; ++z) s += reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
+        const uint32_t u = uabs(s[e]);
+        lmax = u > lmax ? u : lmax;
+      }
+      fin[j] = s;
+    }
+  } else {
   v4i sum[kFinishV];
   // phase 1: every wavefront adds its share of the slices for all of the workgroup's columns
 #pragma unroll
@@ -574,8 +606,6 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
     sum[v] = s;
   }
   // phase 2: column v is completed by wavefront v % NW (two LDS buffers in turn: one barrier per column)
-  v4i fin[OWN];
-  uint32_t lmax = 0;
 #pragma unroll
   for (int v = 0; v < kFinishV; ++v) {
     if (static_cast<long long>(v) * gridDim.x * 64 >= a.nv) continue;  // uniform over the grid: nothing at this stride
@@ -593,6 +623,7 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
       }
       fin[v / NW] = s;
     }
+  }
   }
   lmax = wave_max_u32(lmax);
   if (lane == 0) wmax[wave] = lmax;
