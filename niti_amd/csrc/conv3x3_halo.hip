@@ -94,14 +94,18 @@ struct HGeom {
   static constexpr int ACT_INSTR = (SLOTS + 31) / 32;      // one instruction fills 32 slots
   static constexpr int ACT_BYTES = ACT_INSTR * 1024;
   static constexpr int ACT_LOADS = (ACT_INSTR + 7) / 8;    // per wavefront per slice
-  static constexpr int NWF = KT / 64;                      // 32-channel tiles per wavefront
-  static constexpr int RPS = KT == 64 ? 3 : 1;             // filter rows per stage: the narrow tile takes a whole slice
+  static constexpr int PX = BR * NI * Q;                   // output pixels per workgroup
+  // 512 pixels x 64 channels: both halves of the workgroup's wavefronts work on the same 64 channels, each on 256 of
+  // the pixels (for launches of the 64-channel tile with more workgroups than the device holds at once)
+  static constexpr bool TWO = PX == 512;
+  static constexpr int NWF = TWO ? 2 : KT / 64;            // 32-channel tiles per wavefront
+  static constexpr int RPS = (KT == 64 && !TWO) ? 3 : 1;   // filter rows per stage: the narrow tile takes a whole slice
   static constexpr int W_BYTES = RPS * 3 * KT * 32;        // one filter stage: RPS filter rows of three taps
   static constexpr int W_INSTR = W_BYTES / 1024;
   static constexpr int WSTAGES = 3;
   static constexpr int TILE_BYTES = 2 * ACT_BYTES + WSTAGES * W_BYTES;
   static constexpr int LDS_BYTES = TILE_BYTES + 1024;      // + dump slot / reduction words
-  static_assert(BR * NI * Q == 256, "a workgroup owns 256 output pixels");
+  static_assert(PX == 256 || (PX == 512 && KT == 64), "a workgroup owns 256 output pixels, or 512 with the 64-channel tile");
   static_assert(KT == 64 || KT == 128, "channel tile");
   static_assert(NI == 1 || BR == Q, "several images per workgroup only as whole images");
 };
@@ -121,7 +125,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  const int pixbase = blockIdx.x * 256;  // first output pixel of this workgroup in [N*Q*Q]
+  const int pixbase = blockIdx.x * G::PX;  // first output pixel of this workgroup in [N*Q*Q]
   const int kt = blockIdx.y;
   const int n0 = pixbase / (Q * Q);
   const int p0 = (pixbase - n0 * (Q * Q)) / Q;
@@ -179,7 +183,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   auto issue_w = [&](int cs, int r, int st) {
     // kWT: reduction slice cs = rows (cs & 1) * 32.. of group cs >> 1; a later filter row is an earlier forward tap
     const int rel = kWT ? (cs >> 1) * a.src_cslices * (9 * 2048) + (cs & 1) * 1024 - r * 3 * 2048 : (cs * 9 + r * 3) * 2048;
-    {
+    if (wave < G::W_INSTR) {
       int8_t* dst = w_buf + st * G::W_BYTES + wave * 1024;
       const int off = wsrc_a + rel;
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
@@ -198,7 +202,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 
   // ---- fragment addressing
   const int wp_ = wave & 3;   // 64-pixel group
-  const int wc = wave >> 2;   // channel group of KT/2
+  const int wc = wave >> 2;   // channel group of KT/2 (TWO: pixel half, all wavefronts share the 64 channels)
   const int lr = lane & 31, lk = lane >> 5;
   constexpr int TAPB = kWT ? (KT / 32) * 1024 : 2048;   // bytes between consecutive taps inside a stage
   int w_addr[NWF][kWT ? 2 : 1];   // this lane's filter row(s) inside a stage, tap 0
@@ -207,7 +211,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     if (kWT) {
       // block (tap, slice j) = [32 reduction rows][32 output bytes]; two transposing reads of 8 rows x 16 outputs
       const int j16 = lane & 15, gg = (lane >> 4) & 1;
-      const int jslice = KT == 128 ? wc * 2 + i : wc;
+      const int jslice = G::TWO ? i : (KT == 128 ? wc * 2 + i : wc);
 #pragma unroll
       for (int o = 0; o < (kWT ? 2 : 1); ++o) {
         const int krow = 16 * lk + 8 * o + (j16 >> 1);
@@ -215,14 +219,14 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       }
     } else {
       // row inside the 64-channel group the stage holds at (KT == 128 ? wc * 6144 : 0)
-      const int grow = KT == 128 ? i * 32 + lr : wc * 32 + lr;
+      const int grow = (KT == 128 || G::TWO) ? i * 32 + lr : wc * 32 + lr;
       w_addr[i][0] = (KT == 128 ? wc * 6144 : 0) + grow * 32 + ((lk ^ ((grow >> 3) & 1)) << 4);
     }
   }
   int p_addr[2];              // [pixel tile]: halo slot of this lane's pixel, filter row 0
 #pragma unroll
   for (int j = 0; j < 2; ++j) {
-    const int pix = wp_ * 64 + j * 32 + lr;       // output pixel inside the workgroup's 256
+    const int pix = (G::TWO ? wc * 256 : 0) + wp_ * 64 + j * 32 + lr;   // output pixel inside the workgroup's share
     const int prow = pix / Q, pw = pix % Q;        // row inside the workgroup's rows, column
     const int hrow = (prow / BR) * G::HR + (prow % BR);
     p_addr[j] = (hrow * G::RP + pw) * 32 + ((lk ^ (((pw >> 3) ^ hrow) & 1)) << 4);
@@ -459,7 +463,8 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   }
   const uint32_t lmax = max(static_cast<uint32_t>(vmax), 0u - static_cast<uint32_t>(vmin));
   const long long total_pix = static_cast<long long>(a.N) * Q * Q;
-  const int chbase = kt * KT + wc * (KT / 2);
+  const int chbase = G::TWO ? kt * KT : kt * KT + wc * (KT / 2);
+  const int pixwave = pixbase + (G::TWO ? wc * 256 : 0) + wp_ * 64;   // first pixel of this wavefront
   uint32_t* const red = reinterpret_cast<uint32_t*>(dump);  // behind the tiles, clear of the patches below
   if constexpr (!kFused) {
     hc_sync();  // all wavefronts are done with the tiles: reuse LDS as per-wavefront transposition patches
@@ -469,7 +474,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-      const int mrow = pixbase + wp_ * 64 + j * 32 + rrow;
+      const int mrow = pixwave + j * 32 + rrow;
 #pragma unroll
       for (int i = 0; i < NWF; ++i) {
 #pragma unroll
@@ -599,7 +604,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       for (int t = 0; t < 64 / PPI; ++t) {
         const int pl = t * PPI + prow;
         v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
-        const int m = pixbase + wp_ * 64 + pl;
+        const int m = pixwave + pl;
         const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
         if (a.mask != nullptr) {  // ReLU backward of the layer below, folded in: its output is this layer's input
           const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
@@ -610,7 +615,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         // the 128-channel tile writes 64 bytes per pixel and wavefront: streaming stores start the write-back of the
         // 16 MiB result while the kernel still runs (measured 2 us per launch); the 32-byte pieces of the 64-channel
         // tile are slower that way
-        __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, KT == 128 ? 2 : 0);
+        __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, NWF == 2 ? 2 : 0);
       }
       if (final_range) break;
       // ---- wait for the slots of all workgroups; the maximum over them is the tensor's range
@@ -873,6 +878,16 @@ int halo_ktile(long long pix, int K, int H) {
   return (b128 < 2LL * cus && K > 64) ? 64 : 128;
 }
 
+// The 64-channel tile with 512 pixels per workgroup: where 256-pixel workgroups would be more than the device holds
+// at once (a condition of the requantising variant), on the large maps where such launches occur.
+bool halo_two_pixel_tiles(long long pix, int K, int H, int ktile) {
+  if (ktile != 64 || (H != 32 && H != 16) || pix % 512 != 0) return false;
+  int dev = 0, cus = 0;
+  if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
+    cus = 256;
+  return (pix / 256) * ((K + 63) / 64) > 2LL * cus;
+}
+
 template <int Q, int BR, int NI, int KT, bool kFused, bool kWT>
 int launch_halo(const HaloArgs& a, hipStream_t stream) {
   using G = HGeom<Q, BR, NI, KT>;
@@ -896,7 +911,7 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
     attr_set = true;
   }
   const long long pix = static_cast<long long>(a.N) * Q * Q;
-  dim3 grid(static_cast<unsigned>((pix + 255) / 256), (a.K + KT - 1) / KT);
+  dim3 grid(static_cast<unsigned>((pix + G::PX - 1) / G::PX), (a.K + KT - 1) / KT);
   if (kFused && static_cast<long long>(grid.x) * grid.y > resident)
     return fail(NITI_ERR_UNSUPPORTED, "conv3x3_halo: %u workgroups do not fit on the device at once (%d)", grid.x * grid.y, resident);
   hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, a);
@@ -940,6 +955,12 @@ int launch_halo_tiles(const HaloArgs& a, int H, hipStream_t stream) {
     if (H == 16) return launch_halo<16, 16, 1, 128, kFused, kWT>(a, stream);
     if (H == 8) return launch_halo<8, 8, 4, 128, kFused, kWT>(a, stream);
     return launch_halo<4, 4, 16, 128, kFused, kWT>(a, stream);
+  }
+  if constexpr (kFused) {
+    if (halo_two_pixel_tiles(static_cast<long long>(a.N) * H * H, a.K, H, ktile)) {
+      if (H == 32) return launch_halo<32, 16, 1, 64, kFused, kWT>(a, stream);
+      return launch_halo<16, 16, 2, 64, kFused, kWT>(a, stream);
+    }
   }
   if (H == 32) return launch_halo<32, 8, 1, 64, kFused, kWT>(a, stream);
   if (H == 16) return launch_halo<16, 16, 1, 64, kFused, kWT>(a, stream);
@@ -1009,7 +1030,8 @@ int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S,
   if (!conv3x3_halo_supported(N, H, W, C, K, R, S, stride, pad) || K % 16 != 0) return 0;
   const long long pix = static_cast<long long>(N) * H * W;
   const int ktile = halo_ktile(pix, K, H);
-  const long long nb = H == 2 ? map2_blocks(N, K) : (pix / 256) * ((K + ktile - 1) / ktile);
+  const long long px = halo_two_pixel_tiles(pix, K, H, ktile) ? 512 : 256;
+  const long long nb = H == 2 ? map2_blocks(N, K) : (pix / px) * ((K + ktile - 1) / ktile);
   return nb <= 2048 ? static_cast<int>(nb) : 0;  // the device check happens at launch; this bounds the workspace
 }
 

@@ -107,7 +107,9 @@ def test_conv_dgrad(dev, case):
 # convolution + requantisation in one launch: N,Q,C,K (3x3, stride 1, pad 1), small sums / large sums / ragged tiles
 FUSED_CASES = [(4, 8, 16, 16), (4, 8, 64, 128), (8, 8, 80, 144), (1, 16, 16, 48), (3, 16, 192, 272), (2, 32, 16, 64),
                (8, 32, 128, 128), (12, 8, 512, 128), (16, 4, 64, 128), (48, 4, 256, 80), (64, 2, 512, 512), (128, 2, 32, 48),
-               (5, 2, 48, 16), (33, 2, 16, 80), (256, 2, 160, 96), (1, 2, 96, 32)]
+               (5, 2, 48, 16), (33, 2, 16, 80), (256, 2, 160, 96), (1, 2, 96, 32),
+               # more than 512 tiles of 256 pixels x 64 channels: workgroups of 512 pixels
+               (256, 32, 16, 64), (1024, 16, 32, 48), (144, 32, 48, 64)]
 
 
 @pytest.fixture(params=["auto", "64", "128"])
@@ -350,7 +352,8 @@ def test_conv_requant_range_set_by_one_tile(dev, hot):
         assert torch.equal(d8.cpu(), torch.where(mask > 0, dref, torch.zeros_like(dref)))
 
 
-@pytest.mark.parametrize("case", [(4, 8, 96, 48), (1, 16, 32, 16), (2, 16, 256, 128), (8, 32, 128, 128), (4, 8, 16, 32)])
+@pytest.mark.parametrize("case", [(4, 8, 96, 48), (1, 16, 32, 16), (2, 16, 256, 128), (8, 32, 128, 128), (4, 8, 16, 32),
+                                  (256, 32, 64, 64), (1024, 16, 48, 32)])   # the last two: workgroups of 512 pixels
 def test_conv_dgrad_requant(dev, case):
     from niti_amd import ops
     from oracle import c_oracle as co
