@@ -145,6 +145,18 @@ int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, int8_t* y8, i
                                  int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
                                  const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
                                  size_t workspace_bytes, void* stream);
+/*
+ * niti_conv2d_i8_fprop_requant that also writes the 2x2 / stride-2 maximum of its output: the TiMaxpool2d.forward ->
+ * int8pool_cuda.int8_pool call that follows the layer (and its ReLU) in the reference's networks (ti_torch.py:302-307,
+ * int8pool_kernel.cu:28-80; ti_vgg.py:28-35), taken from the rounded values before they leave the kernel.
+ * pool_out: [N,H/2,W/2,K] int8, 16-byte aligned.  Same coverage as niti_conv2d_i8_fprop_requant except maps of side 2
+ * (NITI_ERR_UNSUPPORTED: use niti_maxpool_i8_fwd on y8).
+ */
+int niti_conv2d_i8_fprop_requant_pool(const int8_t* x, const int8_t* w, int8_t* y8, int8_t* pool_out, int N, int H, int W, int C,
+                                      int K, int R, int S, int stride, int pad, unsigned flags, int target_bits, int method,
+                                      int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words,
+                                      int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                      void* workspace, size_t workspace_bytes, void* stream);
 int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int N, int H, int W, int C, int K, int R,
                                  int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
                                  int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync, size_t sync_words,

@@ -249,7 +249,7 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
                         int K, int R, int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
                         int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync, size_t sync_words,
                         int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
-                        size_t workspace_bytes, void* stream) {
+                        size_t workspace_bytes, void* stream, int8_t* pool_out = nullptr) {
   clear_error();
   int st = check_conv_dims(who, N, H, W, C, K, R, S, stride, pad);
   if (st != NITI_OK) return st;
@@ -280,7 +280,10 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
     wp = static_cast<const int8_t*>(workspace);
   }
   if (relu_mask != nullptr && !aligned16(relu_mask)) return fail(NITI_ERR_INVALID_ARG, "%s: relu_mask must be 16-byte aligned", who);
-  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out, relu_mask};
+  if (pool_out != nullptr && (!aligned16(pool_out) || H % 2 != 0 || W % 2 != 0))
+    return fail(NITI_ERR_INVALID_ARG, "%s: pool_out must be 16-byte aligned and the map side even", who);
+  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out, relu_mask,
+                 pool_out};
   return launch_conv3x3_halo_requant(x, wp, y8, N, Hk, Ck, Kk, flags, sync, rq, s);
 }
 
@@ -291,6 +294,20 @@ extern "C" int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, in
                                             void* workspace, size_t workspace_bytes, void* stream) {
   return conv_requant("conv_fprop_requant", 0, x, w, y8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method, div_mode,
                       bw_mode, rq_flags, nullptr, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
+}
+
+extern "C" int niti_conv2d_i8_fprop_requant_pool(const int8_t* x, const int8_t* w, int8_t* y8, int8_t* pool_out, int N, int H, int W,
+                                                 int C, int K, int R, int S, int stride, int pad, unsigned flags, int target_bits,
+                                                 int method, int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync,
+                                                 size_t sync_words, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b,
+                                                 int32_t* exp_out, void* workspace, size_t workspace_bytes, void* stream) {
+  if (pool_out == nullptr) {
+    clear_error();
+    return fail(NITI_ERR_INVALID_ARG, "conv_fprop_requant_pool: null pointer");
+  }
+  return conv_requant("conv_fprop_requant_pool", 0, x, w, y8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method, div_mode,
+                      bw_mode, rq_flags, nullptr, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream,
+                      pool_out);
 }
 
 extern "C" int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int N, int H, int W, int C, int K,

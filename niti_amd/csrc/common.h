@@ -194,6 +194,7 @@ struct RequantSpec {
   const int32_t* exp_b;
   int32_t* exp_out;
   const int8_t* mask;      // conv + requantisation only: optional ReLU-backward mask, laid out like the output
+  int8_t* pool;            // forward conv + requantisation only: optional 2x2 / stride-2 maximum of the output
 };
 // wall-clock ticks (100 MHz) a grid-wide wait may last (api.hip)
 long long sync_spin_limit();

@@ -69,6 +69,8 @@ struct HaloArgs {
   uint32_t* sync;     // word 0: max |sum| of the launch (output), word 1: set when the wait gave up,
                       // words kSyncSlot0..: one slot per workgroup, max + 1; all zero on entry
   long long y8_bytes;
+  int8_t* pool;       // optional [N,Q/2,Q/2,K] int8: 2x2 / stride-2 maximum of y8 (the max-pool that follows the layer)
+  long long pool_bytes;
   int target_bits, method, trunc, bw_mode;
   unsigned rq_flags;
   long long spin_limit;  // wall-clock ticks (100 MHz) the wait may last
@@ -617,6 +619,30 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         // tile are slower that way
         __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, NWF == 2 ? 2 : 0);
       }
+      if (a.pool != nullptr) {
+        // The max-pool behind this layer, from the rounded values still in the patch: the wavefront's 64 pixels are a
+        // strip of whole image rows (or whole images), i.e. 16 whole 2 x 2 windows; a lane takes 16 channels of one.
+        constexpr int PC = Q / 2;   // pooled pixels per row
+        const int pq = lane / LPP;
+        if (pq < 16) {
+          const int l0 = 2 * (pq / PC) * Q + 2 * (pq % PC);   // upper left pixel of the window inside the strip
+          const int8_t* src = patch + l0 * PROW + piece * 16;
+          const v4i p00 = *reinterpret_cast<const v4i*>(src), p01 = *reinterpret_cast<const v4i*>(src + PROW);
+          const v4i p10 = *reinterpret_cast<const v4i*>(src + Q * PROW), p11 = *reinterpret_cast<const v4i*>(src + (Q + 1) * PROW);
+          v4i mx;
+#pragma unroll
+          for (int q = 0; q < 4; ++q)
+            mx[q] = static_cast<int>(max_i8x4(max_i8x4(static_cast<uint32_t>(p00[q]), static_cast<uint32_t>(p01[q])),
+                                              max_i8x4(static_cast<uint32_t>(p10[q]), static_cast<uint32_t>(p11[q]))));
+          const int m0 = pixwave + l0;
+          const int n = m0 / (Q * Q), rem = m0 - n * (Q * Q);
+          const int pr = rem / Q, pcol = rem - pr * Q;
+          const int pix2 = (n * PC + (pr >> 1)) * PC + (pcol >> 1);
+          const int off = (m0 < total_pix && ch < a.K) ? pix2 * a.K + ch : kOob;
+          const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(a.pool, 0, a.pool_bytes, 0x00020000);
+          __builtin_amdgcn_raw_buffer_store_b128(mx, rp, off, 0, 0);
+        }
+      }
       if (final_range) break;
       // ---- wait for the slots of all workgroups; the maximum over them is the tensor's range
       if (wave == 0) {
@@ -1045,6 +1071,10 @@ int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, i
   a.mask = rq.mask;
   a.sync = sync;
   a.y8_bytes = static_cast<long long>(N) * H * H * K;
+  a.pool = rq.pool;
+  a.pool_bytes = static_cast<long long>(N) * (H / 2) * (H / 2) * K;
+  if (a.pool != nullptr && H == 2)
+    return fail(NITI_ERR_UNSUPPORTED, "conv_requant: the pooled output is not available on 2 x 2 maps");
   a.target_bits = rq.target_bits;
   a.method = rq.method;
   a.trunc = rq.trunc;

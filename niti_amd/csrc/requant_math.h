@@ -95,6 +95,20 @@ __host__ __device__ inline uint32_t positive_bytes(uint32_t m) {
   return (pos >> 7) * 0xFFu;
 }
 
+// the larger of four signed bytes, byte by byte: each byte in the high half of a 16-bit lane keeps its order there
+__device__ inline uint32_t max_i8x4(uint32_t a, uint32_t b) {
+  typedef short s2_t __attribute__((ext_vector_type(2)));
+  union U { uint32_t u; s2_t s; };
+  U ah, bh, al, bl, mh, ml;
+  ah.u = a & 0xFF00FF00u;
+  bh.u = b & 0xFF00FF00u;
+  al.u = (a << 8) & 0xFF00FF00u;
+  bl.u = (b << 8) & 0xFF00FF00u;
+  mh.s = __builtin_elementwise_max(ah.s, bh.s);
+  ml.s = __builtin_elementwise_max(al.s, bl.s);
+  return mh.u | (ml.u >> 8);
+}
+
 // shift < 1: the reference converts int32 to int8 by keeping the low byte
 __device__ inline int wrap_to_i8(int x) { return static_cast<int>(static_cast<int8_t>(static_cast<uint32_t>(x) & 0xFFu)); }
 

@@ -114,7 +114,7 @@ def conv_requant_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1, dgrad=
 
 def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epilogue, target_bits, method, div_mode,
                   bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None, forward_filter=None,
-                  shift_hint=False):
+                  shift_hint=False, pool_out=None):
     _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask, forward_filter)
     if relu_mask is not None and (relu_mask.dtype != torch.int8 or tuple(relu_mask.shape) != tuple(out_shape)):
         raise RuntimeError("%s: relu_mask must be int8 and shaped like the output" % entry)
@@ -147,6 +147,8 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
     head = (_ptr(x), wptr, _ptr(y), N, H, W, C, K, R, S, stride, padding, flags, target_bits, L.ROUND[method],
             L.DIV[div_mode], L.BW[bw_mode], (L.RQ_RELU if relu else 0) | (L.RQ_SHIFT_HINT if shift_hint else 0))
     tail = (_ptr(sync), sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes, _stream(x))
+    if pool_out is not None:    # the entry with the pooled output takes it right after the output
+        head = head[:3] + (_ptr(pool_out),) + head[3:]
     st = getattr(L.lib(), entry)(*(head + ((_ptr(relu_mask),) if dgrad else ()) + tail))
     L.check(st, entry)
     return y, shift_out, sync
@@ -154,9 +156,9 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
 
 def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", relu=False, sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None, shift_hint=False):
+                         prepared_filter=None, shift_hint=False, pool_out=None):
     """conv2d_fprop + requant as one launch: x [N,H,W,C] int8, w [K,R,S,C] int8 -> ([N,P,Q,K] int8, device shift,
-    sync).  sync[0] holds max|sum| afterwards, sync[1] != 0 flags a timed-out wait (invalid output).  ``sync``, if
+    sync).  ``pool_out`` ([N,P/2,Q/2,K] int8): also receives the 2x2 / stride-2 maximum of the output.  sync[0] holds max|sum| afterwards, sync[1] != 0 flags a timed-out wait (invalid output).  ``sync``, if
     given, must hold conv_requant_sync_words(...) zeroed int32 words.  ``shift_hint``: ``shift_out`` holds a
     predicted shift on entry (e.g. this tensor's shift of the previous training step); a good prediction saves the
     kernel a second store pass, the results do not depend on it."""
@@ -166,9 +168,14 @@ def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_b
         raise RuntimeError("conv2d_fprop_requant: channel mismatch %d vs %d" % (C, C2))
     P = (H + 2 * padding - R) // stride + 1
     Q = (W + 2 * padding - S) // stride + 1
-    return _conv_requant("niti_conv2d_i8_fprop_requant", False, x, w, (N, P, Q, K), (N, H, W, C, K, R, S), stride, padding,
+    if pool_out is not None:
+        _chk_dev(x, pool_out)
+        if pool_out.dtype != torch.int8 or tuple(pool_out.shape) != (N, P // 2, Q // 2, K) or not pool_out.is_contiguous():
+            raise RuntimeError("conv2d_fprop_requant: pool_out must be a contiguous int8 [N,P/2,Q/2,K] tensor")
+    entry = "niti_conv2d_i8_fprop_requant_pool" if pool_out is not None else "niti_conv2d_i8_fprop_requant"
+    return _conv_requant(entry, False, x, w, (N, P, Q, K), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter, shift_hint=shift_hint)
+                         prepared_filter, shift_hint=shift_hint, pool_out=pool_out)
 
 
 def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",

@@ -20,6 +20,11 @@ class TiNet(Module):
             if isinstance(a, ti_torch.TiConv2d) and isinstance(b, ti_torch.TiReLU):
                 a.fuse_relu = True
                 b.fused = True
+        # TiConv2d -> fused ReLU -> 2x2 / stride-2 max-pool: the convolution's launch writes the pooled tensor as well
+        for a, b, c in zip(layers, layers[1:], layers[2:]):
+            if (isinstance(a, ti_torch.TiConv2d) and isinstance(b, ti_torch.TiReLU) and b.fused and isinstance(c, ti_torch.TiMaxpool2d)
+                    and (c.kernel_size, c.stride, c.padding) == (2, 2, 0)):
+                a.pool_after = c
         # ReLU [-> max-pool] -> TiConv2d: the convolution zeroes its data gradient where its own input (the ReLU's
         # possibly pooled output) is not positive, which is that ReLU's backward pass (a max-pool routes gradients
         # only to elements equal to the pooled maximum, so masking before or after its backward is the same)

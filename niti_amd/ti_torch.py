@@ -190,7 +190,7 @@ _fused_refused = set()       # (dgrad, input shape, filter shape, stride, paddin
 
 
 def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None, prepared_filter=None,
-                        forward_filter=None, shift_state=None):
+                        forward_filter=None, shift_state=None, pool_out=None):
     """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
     exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
     single-launch kernel, or more workgroups than the device holds at once."""
@@ -210,6 +210,8 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
     exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
     call = ops.conv2d_dgrad_requant if dgrad else ops.conv2d_fprop_requant
     kw = dict(relu=relu, prepared_filter=prepared_filter) if not dgrad else dict(relu_mask=relu_mask, forward_filter=forward_filter)
+    if pool_out is not None:
+        kw.update(pool_out=pool_out)
     if shift_state is not None:     # the tensor's shift of the previous step: the kernel's prediction for this one
         kw.update(shift_out=shift_state, shift_hint=True)
     try:
@@ -365,6 +367,7 @@ class TiConv2d(UpdateWeight):
         self.padding = padding
         self.fuse_relu = False
         self.relu_below = False
+        self.pool_after = None      # the 2x2 / stride-2 TiMaxpool2d behind this layer's (fused) ReLU, if its forward is folded in
 
     def forward(self, input, rand=None):
         self.act, self.act_in_exp = input
@@ -372,10 +375,16 @@ class TiConv2d(UpdateWeight):
         self.act16 = _pad_channels16(self.act).contiguous()      # channel-padded copy, reused by the weight gradient
         w16 = _pad_channels16(self.weight).contiguous()
         exp_a, exp_b = _exp_tensor(self.act_in_exp, dev), self._wexp()
+        pooled = None
+        N, H, W, _ = self.act16.shape
+        if self.pool_after is not None and self.fuse_relu and self.stride == 1 and self.padding == 1 and H == W and H >= 4 and H % 2 == 0:
+            pooled = torch.empty((N, H // 2, W // 2, self.weight.shape[0]), dtype=torch.int8, device=dev)
         fused = _conv_requant_fused(False, self.act16, w16, self.stride, self.padding, ACT_ROUND_METHOD, rand,
                                     self.fuse_relu, exp_a, exp_b, prepared_filter=self._forward_filter(w16),
-                                    shift_state=self._shift_state("act", dev))
+                                    shift_state=self._shift_state("act", dev), pool_out=pooled)
         if fused is not None:
+            if pooled is not None:      # the pooling layer finds its result ready when it sees this tensor
+                self.pool_after.preset = (fused[0], pooled)
             return fused[0], fused[2]
         am = ops.new_scalar_u32(dev)
         acc = ops.conv2d_fprop(self.act16, w16, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
@@ -622,9 +631,14 @@ class TiMaxpool2d(Module):
         self.stride = stride
         self.padding = padding
         self.relu_below = False     # the ReLU in front of this layer leaves its backward pass to this layer
+        self.preset = None          # (input tensor, pooled tensor) left by the convolution that computed both
 
     def forward(self, input):
         self.act_in, exp_in = input
+        preset, self.preset = self.preset, None
+        if preset is not None and preset[0] is self.act_in:
+            self.act_out = preset[1]
+            return self.act_out, exp_in
         self.act_in = self.act_in.contiguous()
         self.act_out = ops.maxpool_fwd(self.act_in, self.kernel_size, self.stride, self.padding)
         return self.act_out, exp_in

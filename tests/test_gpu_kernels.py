@@ -193,6 +193,13 @@ def test_conv_fprop_requant(dev, case, method, div_mode):
         assert int(sync[0]) == po.absmax(acc)
         assert int(sh.cpu()) == sh_ref and int(eo.cpu()) == sh_ref + 3 - 11
         assert torch.equal(y.cpu(), ref.clamp(min=0) if relu else ref)
+        if Q >= 4:
+            # the same launch also writing the 2x2 / stride-2 maximum of its output
+            pooled = torch.full((N, Q // 2, Q // 2, K), 77, dtype=torch.int8, device=dev)
+            y2, sh2, sync2 = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), 1, 1, target_bits=tgt, method=method, div_mode=div_mode,
+                                                      relu=relu, pool_out=pooled)
+            assert int(sync2.cpu()[1]) == 0 and torch.equal(y2, y) and int(sh2.cpu()) == sh_ref
+            assert torch.equal(pooled.cpu(), po.maxpool_fwd(y.cpu()))
 
 
 def test_conv_fprop_requant_wraps_when_no_shift(dev):
