@@ -263,6 +263,12 @@ int niti_weight_update_i8(int8_t* w, const int8_t* g, int64_t n, void* stream);
 int niti_relu_i8_fwd(const int8_t* x, int8_t* y, int64_t n, void* stream);
 int niti_relu_i8_bwd(const int8_t* act, const int8_t* dy, int8_t* dx, int64_t n, void* stream);
 
+/* TiDropout (ti_torch.py:439-455): y[m][f] = x[m][f] * mask[f] with one keep (1) / drop (0) byte per feature, and - when
+   exp_out is given - exp_out = exp_in + exp_add (the layer raises the exponent by one; exp_in NULL counts as 0), as one
+   launch.  The backward pass is the same product on the error (exp_out NULL).  features % 16 == 0, 16-byte aligned. */
+int niti_mask_features_i8(const int8_t* x, const int8_t* mask, int8_t* y, int64_t rows, int features, const int32_t* exp_in,
+                          int32_t* exp_out, int exp_add, void* stream);
+
 /*
  * NHWC int8 max pooling, replaces int8pool_cuda.int8_pool / int8_pool_backward
  * (pytorch/int8pool-extension/int8pool.cpp:37-57, int8pool_kernel.cu:28-138).

@@ -122,6 +122,26 @@ __global__ __launch_bounds__(256) void weight_update_kernel(int8_t* w, const int
     w[i] = static_cast<int8_t>(clip127(static_cast<int>(w[i]) - static_cast<int>(g[i])));
 }
 
+// y[m][f] = x[m][f] * mask[f] with mask bytes 0 / 1 (a keep / drop decision per feature); optionally exp_out = exp_in + add
+__global__ __launch_bounds__(256) void mask_features_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ mask,
+                                                            int8_t* __restrict__ y, int64_t rows, int features,
+                                                            const int32_t* exp_in, int32_t* exp_out, int exp_add) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  const int64_t t0 = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (t0 == 0 && exp_out != nullptr) *exp_out = (exp_in != nullptr ? *exp_in : 0) + exp_add;
+  const int fv = features >> 4;   // features % 16 == 0 (host check)
+  const int64_t nv = rows * fv;
+  for (int64_t i = t0; i < nv; i += stride) {
+    const int f = static_cast<int>(i % fv);
+    const v4i xv = reinterpret_cast<const v4i*>(x)[i];
+    const v4i mv = reinterpret_cast<const v4i*>(mask)[f];
+    v4i o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d) o[d] = xv[d] & static_cast<int>((static_cast<uint32_t>(mv[d]) & 0x01010101u) * 0xFFu);
+    reinterpret_cast<v4i*>(y)[i] = o;
+  }
+}
+
 // kBwd == false: y = max(x, 0).  kBwd == true: y = x(act) > 0 ? dy : 0
 template <bool kBwd>
 __global__ __launch_bounds__(256) void relu_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ dy,
@@ -247,6 +267,19 @@ extern "C" int niti_relu_i8_fwd(const int8_t* x, int8_t* y, int64_t n, void* str
   hipLaunchKernelGGL(relu_kernel<false>, dim3(grid_for((n + 15) / 16, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      x, static_cast<const int8_t*>(nullptr), y, n);
   return check_launch("relu_fwd");
+}
+
+extern "C" int niti_mask_features_i8(const int8_t* x, const int8_t* mask, int8_t* y, int64_t rows, int features,
+                                     const int32_t* exp_in, int32_t* exp_out, int exp_add, void* stream) {
+  clear_error();
+  if (rows < 0 || features <= 0 || features % 16 != 0)
+    return fail(NITI_ERR_INVALID_ARG, "mask_features: rows=%lld features=%d (a multiple of 16)", static_cast<long long>(rows), features);
+  if (x == nullptr || mask == nullptr || y == nullptr) return fail(NITI_ERR_INVALID_ARG, "mask_features: null pointer");
+  if (!aligned16(x) || !aligned16(mask) || !aligned16(y)) return fail(NITI_ERR_INVALID_ARG, "mask_features: pointers must be 16-byte aligned");
+  const int64_t nv = rows * (features >> 4);
+  hipLaunchKernelGGL(mask_features_kernel, dim3(grid_for(nv > 0 ? nv : 1, 256)), dim3(256), 0, static_cast<hipStream_t>(stream), x, mask, y,
+                     rows, features, exp_in, exp_out, exp_add);
+  return check_launch("mask_features");
 }
 
 extern "C" int niti_relu_i8_bwd(const int8_t* act, const int8_t* dy, int8_t* dx, int64_t n, void* stream) {

@@ -401,6 +401,19 @@ def relu_fwd(x):
     return y
 
 
+def mask_features(x, mask, exp_in=None, exp_add=None):
+    """x [rows, F] int8 times a keep / drop byte per feature (mask [F] int8 0/1) in one launch.  With ``exp_add`` also
+    returns a 1-element int32 tensor holding exp_in + exp_add."""
+    _chk_dev(x, mask, exp_in)
+    if x.dtype != torch.int8 or mask.dtype != torch.int8 or x.dim() != 2 or mask.numel() != x.shape[1]:
+        raise RuntimeError("mask_features: int8 [rows, F] tensor and int8 [F] mask expected")
+    y = torch.empty_like(x)
+    exp_out = torch.empty(1, dtype=torch.int32, device=x.device) if exp_add is not None else None
+    L.check(L.lib().niti_mask_features_i8(_ptr(x), _ptr(mask), _ptr(y), x.shape[0], x.shape[1], _ptr(exp_in), _ptr(exp_out),
+                                         int(exp_add or 0), _stream(x)), "niti_mask_features_i8")
+    return (y, exp_out) if exp_add is not None else y
+
+
 def relu_bwd(act, dy):
     _chk_dev(act, dy)
     dx = torch.empty_like(dy)

@@ -700,6 +700,22 @@ def test_maxpool(dev, case):
             assert torch.equal(dxr.cpu(), torch.where(x > 0, ref, torch.zeros_like(ref))), ties
 
 
+def test_mask_features(dev):
+    """Dropout as one launch: a keep / drop byte per feature times every row, exponent + 1."""
+    from niti_amd import ops
+    _say("mask_features")
+    g = torch.Generator().manual_seed(4242)
+    for rows, feats in ((128, 8192), (7, 48), (1, 16), (256, 512)):
+        x = ri8(g, rows, feats, lo=-128)
+        mask = torch.randint(0, 2, (feats,), generator=g, dtype=torch.int8)
+        e = torch.tensor([-9], dtype=torch.int32, device=dev)
+        y, eo = ops.mask_features(x.to(dev), mask.to(dev), e, 1)
+        assert torch.equal(y.cpu(), x * mask) and int(eo.cpu()) == -8
+        assert torch.equal(ops.mask_features(x.to(dev), mask.to(dev)).cpu(), x * mask)
+    with pytest.raises(Exception):
+        ops.mask_features(torch.zeros((4, 24), dtype=torch.int8, device=dev), torch.ones(24, dtype=torch.int8, device=dev))
+
+
 def test_pad_last_dim(dev):
     import torch.nn.functional as F
     from niti_amd import ops
