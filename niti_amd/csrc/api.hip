@@ -260,6 +260,7 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
     return fail(NITI_ERR_UNSUPPORTED, "%s: rounding method %d needs random input; use the two-pass path", who, method);
   if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "%s: div_mode=%d", who, div_mode);
   if (bw_mode != NITI_BW_INT && bw_mode != NITI_BW_F32) return fail(NITI_ERR_INVALID_ARG, "%s: bw_mode=%d", who, bw_mode);
+  if ((rq_flags & ~(NITI_RQ_RELU | NITI_RQ_SHIFT_HINT)) != 0u) return fail(NITI_ERR_INVALID_ARG, "%s: rq_flags=%#x", who, rq_flags);
   const int nb = fused_blocks(N, H, W, C, K, R, S, stride, pad, dgrad);
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "%s: shape not covered by the single-launch path; use the two-pass path", who);
   st = check_forward_copy_flag(who, dgrad, flags, N, H, W, C, K, R, S, stride, pad);

@@ -80,6 +80,15 @@ struct HaloArgs {
   int32_t* exp_out;
 };
 constexpr int kSyncSlot0 = 16;
+// A grid with more workgroups than the device holds at once cannot wait for itself.  It runs as two launches of the
+// same kernel instead (set by the launcher in rq_flags, not part of the interface):
+//   kRqNoWait  every workgroup fills its slot (largest magnitude + 1, and next to it the shift it used), stores its
+//              tile rounded with the predicted shift or what its own sums need, and ends;
+//   kRqSettle  every workgroup first reads all slots - final after the first launch -, and ends at once if its tile
+//              was stored with the final shift; otherwise it computes its tile again and stores it with that shift.
+// With a good prediction (the previous training step's shift) the second launch does nothing but look.
+constexpr unsigned kRqNoWait = 1u << 30, kRqSettle = 1u << 31;
+constexpr int kMaxSlots = 4096;
 
 // Q: image width = height; BR: output rows of one image per workgroup; NI: images per workgroup; BR*NI*Q == 256.
 // The halo tile is NI*(BR+2) rows of Q slots of 32 bytes; for Q a multiple of 8 the bank of a slot depends on its
@@ -131,6 +140,35 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const int kt = blockIdx.y;
   const int n0 = pixbase / (Q * Q);
   const int p0 = (pixbase - n0 * (Q * Q)) / Q;
+
+  int settle_shift = -1;   // kRqSettle: the final shift, when this workgroup has to store its tile again
+  if constexpr (kFused) {
+    if ((a.rq_flags & kRqSettle) != 0) {
+      uint32_t* const slots = a.sync + kSyncSlot0;
+      uint32_t* const words = reinterpret_cast<uint32_t*>(dump);
+      const int nb = gridDim.x * gridDim.y;
+      const int b = blockIdx.y * gridDim.x + blockIdx.x;
+      uint32_t m = 0;
+      for (int i = tid; i < nb; i += 512) m = max(m, __hip_atomic_load(slot_word(slots, i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+      m = wave_max_u32(m);
+      if (lane == 0) words[wave] = m;
+      __syncthreads();
+      uint32_t g = words[0];
+#pragma unroll
+      for (int w = 1; w < 8; ++w) g = max(g, words[w]);
+      const uint32_t gmax = g != 0u ? g - 1u : 0u;
+      const int fshift = max(bitwidth_of(gmax, a.bw_mode) - a.target_bits, 0);
+      const int used = static_cast<int>(slot_word(slots, b)[1]);
+      if (b == 0 && tid == 0) {
+        a.sync[0] = gmax;
+        if (a.shift_out != nullptr) *a.shift_out = fshift;
+        if (a.exp_out != nullptr) *a.exp_out = fshift + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+      }
+      if (used == fshift) return;
+      settle_shift = fshift;
+      __syncthreads();   // the words are written again below
+    }
+  }
 
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.x), 0, a.x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.wp), 0, a.wp_bytes, 0x00020000);
@@ -519,18 +557,20 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     // NITI_RQ_SHIFT_HINT: *shift_out holds the caller's prediction (the previous training step's shift of this
     // tensor).  Read before this workgroup fills its slot: workgroup (0, 0) overwrites the word only after all slots
     // are filled.
-    const int predicted = ((a.rq_flags & NITI_RQ_SHIFT_HINT) != 0 && a.shift_out != nullptr && wave == 0) ? *a.shift_out : 0;
+    const bool nowait = (a.rq_flags & kRqNoWait) != 0;
+    const bool settled = settle_shift >= 0;
+    const int predicted = ((a.rq_flags & NITI_RQ_SHIFT_HINT) != 0 && a.shift_out != nullptr && wave == 0 && !settled) ? *a.shift_out : 0;
     uint32_t early[kLook];   // a hint: the first 64 * kLook slots as they are now
 #pragma unroll
     for (int u = 0; u < kLook; ++u) {
       const int i = u * 64 + lane;
-      early[u] = (wave == 0 && i < nb) ? __hip_atomic_load(slot_word(slots, i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+      early[u] = (wave == 0 && i < nb && !nowait && !settled) ? __hip_atomic_load(slot_word(slots, i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
     }
     const uint32_t wmax = wave_max_u32(lmax);
     __syncthreads();  // the tiles are dead from here on
     if (lane == 0) red[wave] = wmax;
     __syncthreads();
-    if (wave == 0) {
+    if (wave == 0 && !settled) {
       uint32_t bmax = lane < 8 ? red[lane] : 0u;
       bmax = wave_max_u32(bmax);
       const int b = blockIdx.y * gridDim.x + blockIdx.x;
@@ -551,6 +591,11 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     int shift = max(bitwidth_of(red[8], a.bw_mode) - a.target_bits, 0);
     bool final_range = red[9] != 0u;
     if (!final_range) shift = max(shift, static_cast<int>(red[10]));
+    if (settled) shift = settle_shift;
+    if (nowait) {   // the shift this tile is stored with, for the settling launch
+      if (tid == 0) slot_word(slots, blockIdx.y * gridDim.x + blockIdx.x)[1] = static_cast<uint32_t>(shift);
+    }
+    final_range = final_range || nowait || settled;
     const bool trunc = a.trunc != 0;
     const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
     const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
@@ -656,7 +701,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       shift = fshift;
       __builtin_amdgcn_s_waitcnt(0);   // the stores of the first pass leave before those that replace them
     }
-    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0) {
+    if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0 && !nowait && !settled) {
       const int sh = shift > 0 ? shift : 0;
       a.sync[0] = red[8];
       if (a.shift_out != nullptr) *a.shift_out = sh;
@@ -938,8 +983,18 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
   }
   const long long pix = static_cast<long long>(a.N) * Q * Q;
   dim3 grid(static_cast<unsigned>((pix + G::PX - 1) / G::PX), (a.K + KT - 1) / KT);
-  if (kFused && static_cast<long long>(grid.x) * grid.y > resident)
-    return fail(NITI_ERR_UNSUPPORTED, "conv3x3_halo: %u workgroups do not fit on the device at once (%d)", grid.x * grid.y, resident);
+  if (kFused && static_cast<long long>(grid.x) * grid.y > resident) {
+    // more workgroups than the device holds at once: nobody waits; a second launch settles the tiles stored with
+    // another shift than the final one
+    if (static_cast<long long>(grid.x) * grid.y > kMaxSlots)
+      return fail(NITI_ERR_UNSUPPORTED, "conv3x3_halo: %u workgroups exceed the %d range slots", grid.x * grid.y, kMaxSlots);
+    HaloArgs b = a;
+    b.rq_flags = a.rq_flags | kRqNoWait;
+    hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, b);
+    b.rq_flags = a.rq_flags | kRqSettle;
+    hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, b);
+    return check_launch("conv3x3_halo");
+  }
   hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, a);
   return check_launch("conv3x3_halo");
 }
@@ -1058,7 +1113,7 @@ int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S,
   const int ktile = halo_ktile(pix, K, H);
   const long long px = halo_two_pixel_tiles(pix, K, H, ktile) ? 512 : 256;
   const long long nb = H == 2 ? map2_blocks(N, K) : (pix / px) * ((K + ktile - 1) / ktile);
-  return nb <= 2048 ? static_cast<int>(nb) : 0;  // the device check happens at launch; this bounds the workspace
+  return nb <= kMaxSlots ? static_cast<int>(nb) : 0;  // more than the device holds at once run as two launches
 }
 
 size_t conv3x3_halo_sync_words(int blocks) { return static_cast<size_t>(kSyncSlot0) + slot_words(blocks); }

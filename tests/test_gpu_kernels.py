@@ -109,7 +109,9 @@ FUSED_CASES = [(4, 8, 16, 16), (4, 8, 64, 128), (8, 8, 80, 144), (1, 16, 16, 48)
                (8, 32, 128, 128), (12, 8, 512, 128), (16, 4, 64, 128), (48, 4, 256, 80), (64, 2, 512, 512), (128, 2, 32, 48),
                (5, 2, 48, 16), (33, 2, 16, 80), (256, 2, 160, 96), (1, 2, 96, 32),
                # more than 512 tiles of 256 pixels x 64 channels: workgroups of 512 pixels
-               (256, 32, 16, 64), (1024, 16, 32, 48), (144, 32, 48, 64)]
+               (256, 32, 16, 64), (1024, 16, 32, 48), (144, 32, 48, 64),
+               # more workgroups than the device holds at once: two launches, the second one settling the shift
+               (264, 16, 16, 272), (600, 32, 16, 48)]
 
 
 @pytest.fixture(params=["auto", "64", "128"])
@@ -300,7 +302,8 @@ def test_conv_triple_at_benchmark_size(dev, layer):
         assert int(sync.cpu()[1]) == 0 and torch.equal(d8, r8) and int(sh.cpu()) == int(rsh.cpu())
 
 
-@pytest.mark.parametrize("case", [(8, 32, 64, 128), (16, 8, 256, 64), (4, 16, 32, 48)])
+@pytest.mark.parametrize("case", [(8, 32, 64, 128), (16, 8, 256, 64), (4, 16, 32, 48),
+                                  (264, 16, 16, 272), (136, 32, 16, 144)])   # the last two: more workgroups than fit at once
 def test_conv_requant_predicted_shift(dev, case):
     """A predicted shift (right, too small, too large, absurd) changes how often the kernel stores, never what."""
     from niti_amd import ops
@@ -326,6 +329,37 @@ def test_conv_requant_predicted_shift(dev, case):
     so = torch.tensor([5], dtype=torch.int32, device=dev)
     y, sh, sync = ops.conv2d_fprop_requant(torch.zeros_like(x).to(dev), w.to(dev), shift_out=so, shift_hint=True)
     assert int(y.abs().max()) == 0 and int(so.cpu()) == 0
+
+
+def test_conv_requant_oversubscribed_range_set_by_one_tile(dev):
+    """Two-launch form (more workgroups than fit at once): one image with large values among images of tiny ones makes
+    nearly every workgroup of the second launch compute and store its tile again; with the mask of a ReLU below and
+    with the pooled output."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = 136, 32, 144, 144
+    _say("conv_requant_oversubscribed_range_set_by_one_tile")
+    g = torch.Generator().manual_seed(6160)
+    x = ri8(g, N, Q, Q, C, lo=-1, hi=1)
+    x[77] = ri8(g, Q, Q, C)
+    w = ri8(g, K, 3, 3, C)
+    acc = po.conv2d_fprop_i32(x, w, 1, 1)
+    ref, sh_ref = po.act_calc(acc, 0)
+    pooled = torch.empty((N, Q // 2, Q // 2, K), dtype=torch.int8, device=dev)
+    y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), relu=True, pool_out=pooled)
+    assert int(sync.cpu()[1]) == 0 and int(sync.cpu()[0]) == po.absmax(acc) and int(sh.cpu()) == sh_ref
+    assert torch.equal(y.cpu(), ref.clamp(min=0)) and torch.equal(pooled.cpu(), po.maxpool_fwd(ref.clamp(min=0)))
+    e = ri8(g, N, Q, Q, K, lo=-1, hi=1)
+    e[5] = ri8(g, Q, Q, K)
+    dacc = co.conv_dgrad(e, w, Q, Q, 1, 1)
+    dref, dsh = po.err_calc(dacc)
+    mask = ri8(g, N, Q, Q, C)
+    wf = ops.conv_filter_prepare(w.to(dev), N, Q, Q)
+    for kw in (dict(), dict(forward_filter=wf)):
+        d8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), relu_mask=mask.to(dev), **kw)
+        assert int(sync.cpu()[1]) == 0 and int(sh.cpu()) == dsh
+        assert torch.equal(d8.cpu(), torch.where(mask > 0, dref, torch.zeros_like(dref)))
 
 
 @pytest.mark.parametrize("hot", [0, 3, 7])
@@ -534,12 +568,25 @@ def test_conv_requant_rejects_what_it_does_not_cover(dev):
     e = torch.zeros((3, 7, 9, 32), dtype=torch.int8, device=dev)
     with pytest.raises(NitiError):
         ops.conv2d_dgrad(e, torch.zeros((32, 3, 3, 16), dtype=torch.int8, device=dev), forward_filter=torch.zeros(64, dtype=torch.int8, device=dev))
-    # a launch that would not be resident at once is refused by the library, not started
-    N = 2048                                                          # 2048 workgroups of 256 pixels
+    # a launch that would not be resident at once runs as two launches that do not wait for each other
+    from oracle import niti_oracle as po
+    N = 2048                                                          # 2048 tiles of 256 pixels
     assert ops.conv_requant_sync_words(N, 16, 16, 16, 16) > 0
-    x = torch.zeros((N, 16, 16, 16), dtype=torch.int8, device=dev)
-    with pytest.raises(NitiError):
-        ops.conv2d_fprop_requant(x, w)
+    g = torch.Generator().manual_seed(31)
+    x, w = ri8(g, N, 16, 16, 16), ri8(g, 16, 3, 3, 16)
+    ref, sh_ref = po.act_calc(po.conv2d_fprop_i32(x, w, 1, 1), 0)
+    y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev))
+    assert int(sync.cpu()[1]) == 0 and int(sh.cpu()) == sh_ref and torch.equal(y.cpu(), ref)
+    # internal flag bits are not part of the interface
+    from niti_amd import _lib as L
+    xs = torch.zeros((4, 8, 8, 16), dtype=torch.int8, device=dev)
+    y8 = torch.empty((4, 8, 8, 16), dtype=torch.int8, device=dev)
+    words = ops.conv_requant_sync_words(4, 8, 8, 16, 16)
+    sync = torch.zeros(words, dtype=torch.int32, device=dev)
+    ws = torch.empty(1 << 20, dtype=torch.int8, device=dev)
+    st = L.lib().niti_conv2d_i8_fprop_requant(xs.data_ptr(), w.to(dev).data_ptr(), y8.data_ptr(), 4, 8, 8, 16, 16, 3, 3, 1, 1, 0, 7, 0, 0, 0,
+                                              1 << 30, sync.data_ptr(), words, None, None, None, None, ws.data_ptr(), ws.numel(), None)
+    assert st != 0
 
 
 WGRAD_CASES = [(4, 32, 32, 16, 32, 3, 1), (8, 16, 16, 128, 64, 3, 1), (6, 8, 8, 80, 144, 3, 1), (2, 32, 32, 64, 128, 3, 1),
