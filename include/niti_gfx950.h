@@ -122,9 +122,9 @@ int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N,
  * channels % 16 == 0, output channels % 16 == 0, rounding NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC, and a
  * launch of at most 4096 workgroups (N*H*W/256 x ceil(out channels/128 or 64); side 2: ceil(N/32) x ceil(out
  * channels/32), which must fit on the device at once).  Launches of the other sides that do not fit on the device at
- * once run as two launches that do not wait (the second one settles tiles stored with another shift than the final one).  niti_conv2d_i8_requant_sync_words
- * returns 0 for shapes outside that (then use the two-pass entry points); the entry points return
- * NITI_ERR_UNSUPPORTED for them and for a device too small for the launch.
+ * once run as two launches that do not wait (the second one settles tiles stored with another shift than the final
+ * one).  niti_conv2d_i8_requant_sync_words returns 0 for shapes outside that (then use the two-pass entry points); the
+ * entry points return NITI_ERR_UNSUPPORTED for them.
  *
  * sync: niti_conv2d_i8_requant_sync_words(...) uint32 words that are ZERO on entry (niti_fill_u32).  On return
  * word 0 holds max |sum| over the tensor; word 1 is non-zero if the wait for the other workgroups ran into its
