@@ -45,6 +45,7 @@ struct WgradArgs {
   int32_t* partial;   // [splits][slice_stride], slice z holds K*9*C partial sums
   long long slice_stride;
   int N, C, K;
+  int Cp;             // gradient columns (input channels) kept per tap in the partial sums: C, or fewer when the rest is padding
   int bands, bands_per_split;
   long long act_bytes, err_bytes;
 };
@@ -278,7 +279,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
   // ---- partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+wc*32+(lane&31)]
   int32_t* out = a.partial + static_cast<long long>(item.z) * a.slice_stride;
   const int c = c0 + wc * 32 + (lane & 31);
-  if (c < a.C) {
+  if (c < a.Cp) {
 #pragma unroll
     for (int g = 0; g < 4; ++g)
 #pragma unroll
@@ -286,7 +287,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
         const int k = k0 + wk * 32 + g * 8 + lk * 4 + e;
         if (k >= a.K) continue;
 #pragma unroll
-        for (int t = 0; t < 9; ++t) out[(static_cast<long long>(k) * 9 + t) * a.C + c] = acc[t][4 * g + e];
+        for (int t = 0; t < 9; ++t) out[(static_cast<long long>(k) * 9 + t) * a.Cp + c] = acc[t][4 * g + e];
       }
   }
 }
@@ -471,7 +472,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
 #pragma unroll
         for (int t = 0; t < 9; ++t) {
           const int v = acc[t][4 * g + e] + park[(t * 16 + 4 * g + e) * 64];
-          if (c < a.C && k < a.K) out[(static_cast<long long>(k) * 9 + t) * a.C + c] = v;
+          if (c < a.Cp && k < a.K) out[(static_cast<long long>(k) * 9 + t) * a.Cp + c] = v;
         }
       }
   }
@@ -812,15 +813,16 @@ size_t wgrad3x3_workspace(int N, int H, int C, int K) {
   return static_cast<size_t>(pick_splits(N, H, C, K)) * slice_stride_for(C, K) * sizeof(int32_t);
 }
 
-static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N, int H, int C, int K, void* workspace,
+static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N, int H, int C, int K, int Cp, void* workspace,
                                     WgradArgs& a, int& splits, hipStream_t stream) {
   a.act = act;
   a.err = err;
   a.partial = static_cast<int32_t*>(workspace);
-  a.slice_stride = slice_stride_for(C, K);
+  a.slice_stride = slice_stride_for(Cp, K);
   a.N = N;
   a.C = C;
   a.K = K;
+  a.Cp = Cp;
   const bool narrow = use_narrow_arrangement(N, H);
   a.bands = N * H * H / (narrow ? 256 : 128);
   splits = pick_splits(N, H, C, K);
@@ -843,7 +845,7 @@ int launch_wgrad3x3(const int8_t* act, const int8_t* err, int32_t* dw, int N, in
                     uint32_t* absmax, void* workspace, hipStream_t stream) {
   WgradArgs a;
   int splits = 1;
-  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, workspace, a, splits, stream);
+  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, C, workspace, a, splits, stream);
   if (st != NITI_OK) return st;
   const int64_t n = static_cast<int64_t>(K) * 9 * C;
   int64_t g = (n / 4 + 63) / 64;
@@ -867,7 +869,10 @@ size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
                            bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
                            void* workspace, hipStream_t stream) {
-  const int nb = wgrad3x3_finish_blocks(C, K);
+  // The first layer's three input channels come padded to 16: unless the caller wants the int32 gradient in that
+  // layout, the partial sums keep four columns per tap (a quarter of the bytes written and read back).
+  const int Cp = (dw == nullptr && C == 16 && w_channels <= 4) ? 4 : C;
+  const int nb = wgrad3x3_finish_blocks(Cp, K);
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large for the single-pass finish", K, C);
   if (static_cast<long long>(K) * 9 * C >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large", K, C);
   static int resident[2] = {0, 0};   // workgroups of 4 / 16 wavefronts the device holds at once
@@ -883,14 +888,14 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   if (nb > resident[0]) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: %d workgroups do not fit on the device at once (%d)", nb, resident[0]);
   WgradArgs a;
   int splits = 1;
-  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, workspace, a, splits, stream);
+  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, Cp, workspace, a, splits, stream);
   if (st != NITI_OK) return st;
   FinishArgs f{};
   f.partial = a.partial;
   f.slice_stride = a.slice_stride;
   f.splits = splits;
-  f.nv = static_cast<long long>(K) * 9 * C / 4;
-  f.C = C;
+  f.nv = static_cast<long long>(K) * 9 * Cp / 4;
+  f.C = Cp;
   f.Cw = w_channels;
   f.w = w;
   f.g8 = g8;
