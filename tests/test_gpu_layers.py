@@ -277,6 +277,19 @@ def test_epoch_driver_learns_and_checkpoints(tt, tmp_path):
     assert torch.equal(out_a, out_b) and _ei(exp_a) == _ei(exp_b)
 
 
+def test_epoch_driver_command_line(tt, tmp_path, monkeypatch):
+    """The command line keeps the reference's option names; without a data file it trains on the synthetic set and
+    leaves its checkpoints under ./results/<--save>; --init continues from one."""
+    import os
+    from niti_amd import train
+    _say("epoch_driver_command_line")
+    monkeypatch.chdir(tmp_path)
+    hist = train.main(["--depth", "7", "--epochs", "1", "--batch-size", "128", "--seed", "5", "--save", "run1", "--log-interval", "8"])
+    assert len(hist) == 1 and os.path.exists(os.path.join("results", "run1", "ckpt.pth"))
+    again = train.main(["--depth", "7", "--epochs", "1", "--batch-size", "128", "--seed", "5", "--init", os.path.join("results", "run1", "ckpt.pth")])
+    assert again[0]["val_prec1"] >= 0.0 and not os.path.exists(os.path.join("results", "test"))
+
+
 def test_grid_wide_wait_gives_up_and_says_so():
     """With a wait limit of one clock tick (set from the host, in a process of its own because the library reads
     the limit once) the single-launch kernels do not wait for late workgroups: every workgroup still runs to its
