@@ -20,10 +20,15 @@
 //
 // Requantising variant (kFused): the int32 sums never leave the registers.  Every workgroup publishes
 // the largest magnitude of its tile in a slot of its own, waits until the slots of all workgroups of the
-// launch are filled (they are all resident: the host refuses grids larger than the chip holds at once,
-// and the wait is bounded by a wall-clock limit so that every wavefront exits whatever happens), derives
-// the tensor-wide shift from the maximum over the slots and stores rounded int8.  Compared with the
-// int32 store + separate requantisation pass this removes 8 of the 9 bytes moved per output element.
+// launch are filled (they are all resident - the host checks that - and the wait is bounded by a wall-clock
+// limit so that every wavefront exits whatever happens), derives the tensor-wide shift from the maximum
+// over the slots and stores rounded int8.  Compared with the int32 store + separate requantisation pass
+// this removes 8 of the 9 bytes moved per output element.  The same epilogue can leave the 2x2 / stride-2
+// maximum of its output next to it (the max-pool that follows the layer).
+//
+// Launches the device cannot hold at once: the 64-channel tile takes 512 pixels per workgroup where that
+// is enough (HGeom::TWO); otherwise the launch runs twice without waiting (kRqNoWait, kRqSettle below).
+// Maps of 2 x 2 pixels have a kernel of their own at the end of this file (conv3x3_map2_kernel).
 #include <stdlib.h>
 
 #include "common.h"
