@@ -68,6 +68,35 @@ def test_conv_layer_fwd_bwd(tt, div_mode, first):
         assert torch.equal(r[0].cpu(), ro[0]) and _ei(r[1]) == ro[1]
 
 
+def test_conv_layer_on_a_grid_larger_than_the_device(tt):
+    """A layer whose convolutions have more workgroups than the device holds at once (136 images of 32 x 32, 80 -> 144
+    channels: 1088 and 544 tiles): forward and data gradient run as two launches that do not wait.  Two training
+    steps in a row, the second one predicting its shifts from the first."""
+    from oracle import niti_model_oracle as mo
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(1100)
+    N, H, C, K = 136, 32, 80, 144
+    _say("conv layer, oversubscribed grid")
+    w, x = ri8(g, K, 3, 3, C), ri8(g, N, H, H, C, lo=-60, hi=60)   # 139264 pixels: keeps the weight gradient's bound below 2^31
+    cfg = mo.Cfg()
+    o = mo.OConv2d(w, -9)
+    layer = tt.TiConv2d(C, K)
+    layer.weight = w.to(dev)
+    layer.weight_exp = torch.tensor(-9.0)
+    layer.relu_below = True
+    for step in range(2):
+        err = laplace_i8(g, (N, H, H, K), b=4.0 * (step + 1))
+        yo, eo = o.forward((x, -3), cfg)
+        ro = o.backward((err, -5), cfg)
+        y, e = layer.forward((x.to(dev), -3))
+        assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+        r = layer.backward((err.to(dev), -5))
+        assert torch.equal(layer.weight.cpu(), o.weight) and _ei(layer.grad_exp) == o.grad_exp
+        assert torch.equal(r[0].cpu(), torch.where(x > 0, ro[0], torch.zeros_like(ro[0]))) and _ei(r[1]) == ro[1]
+    from niti_amd import ops
+    assert not ops.sync_arena.timed_out(dev)
+
+
 # sizes: a ragged small one, the fully connected configuration of the benchmark list (activations 128 x 8192,
 # weights 1024 x 8192, stochastic rounding from seeded random integers), and the classifier (few output features)
 @pytest.mark.parametrize("shape", [(32, 512, 48), (128, 8192, 1024), (128, 8192, 10)])
