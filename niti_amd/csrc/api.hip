@@ -408,7 +408,7 @@ extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err,
   if (w_prepared != nullptr && (filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 0) != 2 || reinterpret_cast<uintptr_t>(w_prepared) % 4 != 0))
     return fail(NITI_ERR_UNSUPPORTED, "conv_wgrad_update: w_prepared needs a shape whose forward pass uses a kernel-ready filter copy, 4-byte aligned");
   RequantSpec rq{mu, method, div_mode == NITI_DIV_TRUNC, bw_mode, (flags & NITI_CONV_SHIFT_HINT) ? NITI_RQ_SHIFT_HINT : 0u, sync_spin_limit(),
-                 shift_out, exp_a, exp_b, exp_out, nullptr};
+                 shift_out, exp_a, exp_b, exp_out, nullptr, nullptr};
   return launch_wgrad3x3_update(act, err, w, w_channels, N, H, C, K, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, sync, rq, g8_out,
                                 dw_out, w_prepared, workspace, static_cast<hipStream_t>(stream));
 }

@@ -65,7 +65,6 @@ __device__ inline uint32_t exchange_range(const FcArgs& a, uint32_t bmax) {
 // One workgroup of 16 wavefronts per tile of 16 samples; wavefront w reduces over features [w * kchunk, (w+1) * kchunk).
 __global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
   __shared__ int part[16][256];
-  __shared__ uint32_t gshare;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int mt = blockIdx.x;
