@@ -87,6 +87,7 @@ class TiNet(Module):
 
     def load_state_dict(self, state_dict):
         """ti_net.py:43-48."""
+        self.__dict__.pop("_step_graphs", None)     # captured steps (train.StepGraph) point at the tensors replaced here
         for idx, l in enumerate(self.forward_layers):
             if hasattr(l, "weight"):
                 prefix = "layers." + str(idx) + "."

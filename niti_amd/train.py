@@ -41,10 +41,83 @@ def apply_regime(regime, epoch):
             break
 
 
-def run_epoch(data_loader, model, training, log_interval=0, epoch=0):
+def _add_metrics(output, output_exp, target, sums):
+    """Adds batch size x (display loss, top-1, top-5) to ``sums`` (main.py:156-163)."""
+    scale = torch.exp2(torch.as_tensor(output_exp, device=output.device).float().reshape(()))
+    loss = F.cross_entropy(output.float() * scale, target)
+    prec1, prec5 = accuracy(output.detach(), target, topk=(1, 5))
+    sums += torch.stack([loss.double(), prec1.double(), prec5.double()]) * target.size(0)
+
+
+def _one_step(model, training, inputs, target, sums):
+    """Forward (+ backward when training) on one batch of float images."""
+    output, output_exp = model(inputs)
+    _add_metrics(output, output_exp, target, sums)
+    if training:
+        model.backward(target)
+
+
+class StepGraph:
+    """The integer part of a training (or evaluation) step replayed from a captured HIP graph: a step is some forty
+    short launches, and issuing them one by one from Python takes about twice as long as the device needs for them.
+    Only the library's own kernels, fills and random-number kernels are captured.  The input quantisation and the
+    display metrics - tensor-library reductions, whose multi-block forms clear their scratch words with memset
+    nodes that do not replay reliably here - run eagerly before and after each replay, on static buffers.  The
+    first ``eager_steps`` batches run eagerly (ordinary steps: nothing is run twice), the next one is captured, from
+    then on batches are replays.  Falls back to eager steps if the capture is refused."""
+
+    def __init__(self, model, training, inputs, target, eager_steps=3):
+        self.model, self.training = model, training
+        n, c, h, w = inputs.shape
+        self.x8 = torch.empty((n, h, w, c), dtype=torch.int8, device=inputs.device)     # quantised batch, NHWC
+        self.x_exp = torch.empty(1, dtype=torch.int32, device=inputs.device)
+        self.target = torch.empty_like(target)
+        self.graph, self.failed, self.eager_left = None, False, eager_steps
+        self.out = None
+        self.side = torch.cuda.Stream()
+
+    def _step(self):
+        self.model.forward_int8(self.x8, self.x_exp)
+        if self.training:
+            self.model.backward(self.target)
+
+    def __call__(self, inputs, target, sums):
+        x_data, x_exp = ti_torch.TiFloatToInt8(inputs)          # ti_net.py:17-19
+        self.x8.copy_(x_data.permute(0, 2, 3, 1))
+        self.x_exp.copy_(x_exp.reshape(1))
+        self.target.copy_(target, non_blocking=True)
+        if self.graph is not None:
+            self.graph.replay()
+        elif self.eager_left > 0 or self.failed:
+            self.eager_left -= 1
+            cur = torch.cuda.current_stream()
+            self.side.wait_stream(cur)
+            with torch.cuda.stream(self.side):
+                self._step()
+            cur.wait_stream(self.side)
+        else:
+            torch.cuda.synchronize()
+            try:
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    self._step()
+                self.graph = g
+                self.out = (self.model.out, self.model.out_exp)     # where every replay leaves its logits
+                g.replay()
+            except Exception as e:      # keep training
+                logging.warning("step graph capture failed (%s); running eager steps", e)
+                torch.cuda.synchronize()
+                self.failed = True
+                self._step()
+        output, output_exp = self.out if self.graph is not None else (self.model.out, self.model.out_exp)
+        _add_metrics(output, output_exp, self.target, sums)
+
+
+def run_epoch(data_loader, model, training, log_interval=0, epoch=0, use_graph=False):
     """One pass over ``data_loader`` (main.py:133-193).  Returns (loss, top-1 %, top-5 %) averaged over the
     samples.  The float cross-entropy is for display only, as in the reference (main.py:156-157); the sums stay on
-    the device until the end of the pass so that the integer step is not held up by host reads."""
+    the device until the end of the pass so that the integer step is not held up by host reads.  ``use_graph``:
+    replay the step from a HIP graph (StepGraph; batches must all have one shape)."""
     ti_torch.TRAINING = bool(training)
     dev = torch.device(ti_torch.GPU)
     sums = torch.zeros(3, dtype=torch.float64, device=dev)
@@ -52,18 +125,20 @@ def run_epoch(data_loader, model, training, log_interval=0, epoch=0):
     for i, (inputs, target) in enumerate(data_loader):
         inputs = inputs.to(dev, non_blocking=True)
         target = target.to(dev, non_blocking=True)
-        output, output_exp = model(inputs)
-        scale = torch.exp2(torch.as_tensor(output_exp, device=dev).float().reshape(()))
-        loss = F.cross_entropy(output.float() * scale, target)
-        prec1, prec5 = accuracy(output.detach(), target, topk=(1, 5))
-        n = inputs.size(0)
-        sums += torch.stack([loss.double(), prec1.double(), prec5.double()]) * n
-        count += n
-        if training:
-            model.backward(target)
-            if log_interval and i % log_interval == 0:
-                s = (sums / count).tolist()
-                logging.info('[%d][%3d] loss %.3f @1 %.3f', epoch, i, s[0], s[1])
+        if use_graph:
+            # graphs are per mode, batch shape and gradient bit width (a kernel argument fixed at capture)
+            key = (bool(training), tuple(inputs.shape), inputs.dtype, ti_torch.GRAD_BITWIDTH)
+            cache = model.__dict__.setdefault('_step_graphs', {})
+            runner = cache.get(key)
+            if runner is None:
+                runner = cache[key] = StepGraph(model, bool(training), inputs, target)
+            runner(inputs, target, sums)
+        else:
+            _one_step(model, bool(training), inputs, target, sums)
+        count += inputs.size(0)
+        if training and log_interval and i % log_interval == 0:
+            s = (sums / count).tolist()
+            logging.info('[%d][%3d] loss %.3f @1 %.3f', epoch, i, s[0], s[1])
     if count == 0:
         return 0.0, 0.0, 0.0
     loss_avg, top1, top5 = (sums / count).tolist()
@@ -88,15 +163,15 @@ def load_checkpoint(model, path):
     return ckpt
 
 
-def fit(model, train_loader, test_loader, epochs, save_path=None, save_all=False, log_interval=0):
+def fit(model, train_loader, test_loader, epochs, save_path=None, save_all=False, log_interval=0, use_graph=False):
     """main.py:66-131 without the TensorBoard writer: per epoch apply the regime, train, evaluate, write
     ``ckpt.pth`` (and ``model_best.pth.tar``) under ``save_path``.  Returns one dict per epoch."""
     history = []
     best_prec1 = 0.0
     for epoch in range(epochs):
         apply_regime(model.regime, epoch)
-        train_loss, train_prec1, _ = run_epoch(train_loader, model, True, log_interval, epoch)
-        val_loss, val_prec1, _ = run_epoch(test_loader, model, False, 0, epoch)
+        train_loss, train_prec1, _ = run_epoch(train_loader, model, True, log_interval, epoch, use_graph)
+        val_loss, val_prec1, _ = run_epoch(test_loader, model, False, 0, epoch, use_graph)
         is_best = val_prec1 > best_prec1
         best_prec1 = max(val_prec1, best_prec1)
         if save_path is not None:
@@ -172,6 +247,7 @@ def main(argv=None):
     p.add_argument('--epochs', default=200, type=int)
     p.add_argument('--init', help='init ckpt')
     p.add_argument('--depth', default=7, type=int)
+    p.add_argument('--no-graph', action='store_true', help='issue every launch of a step from Python instead of replaying a HIP graph')
     args = p.parse_args(argv)
     logging.basicConfig(level=logging.INFO, format='%(asctime)s %(message)s')
     if args.seed > 0:
@@ -186,7 +262,7 @@ def main(argv=None):
         logging.info("no dataset given: synthetic class patterns")
         train_loader, test_loader = synthetic_loaders(args.batch_size, seed=max(args.seed, 0))
     save_path = os.path.join('./results/', args.save) if args.save else None
-    return fit(model, train_loader, test_loader, args.epochs, save_path, args.save_all, args.log_interval)
+    return fit(model, train_loader, test_loader, args.epochs, save_path, args.save_all, args.log_interval, not args.no_graph)
 
 
 if __name__ == '__main__':

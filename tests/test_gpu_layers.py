@@ -279,7 +279,8 @@ def test_shims_match_reference_conventions():
     assert hasattr(int8conv_cuda, "group_conv") and hasattr(cutlassconv_cuda, "weight_grad")
 
 
-def test_epoch_driver_learns_and_checkpoints(tt, tmp_path):
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_epoch_driver_learns_and_checkpoints(tt, tmp_path, use_graph):
     """The epoch driver (regime, train pass, evaluation pass, checkpoint files) on a synthetic ten-class task: the
     integer step must actually learn (chance is 10 %), and a checkpoint loaded into a fresh model must reproduce
     the trained model's outputs bit for bit."""
@@ -291,7 +292,20 @@ def test_epoch_driver_learns_and_checkpoints(tt, tmp_path):
     model = TiVGG_cifar(depth=7)
     model.regime = [{'epoch': 0, 'gb': 5}, {'epoch': 3, 'gb': 4}]
     tr, te = train.synthetic_loaders(128, train_batches=16, test_batches=4, noise=0.5, seed=1)
-    hist = train.fit(model, tr, te, epochs=4, save_path=str(tmp_path), save_all=True)
+    hist = train.fit(model, tr, te, epochs=4, save_path=str(tmp_path), save_all=True, use_graph=use_graph)
+    if use_graph:   # training and evaluation steps at both gradient bit widths of the regime were captured, none refused
+        graphs = model.__dict__["_step_graphs"]
+        assert len(graphs) == 4 and all(g.graph is not None and not g.failed for g in graphs.values())
+        # every replay (52 training and 4 evaluation steps, with eager work and host reads in between) did what the
+        # eager step does: the same run issued launch by launch ends with the same numbers and the same weights
+        torch.manual_seed(3)
+        twin = TiVGG_cifar(depth=7)
+        twin.regime = model.regime
+        tr2, te2 = train.synthetic_loaders(128, train_batches=16, test_batches=4, noise=0.5, seed=1)
+        hist2 = train.fit(twin, tr2, te2, epochs=4, use_graph=False)
+        assert hist2 == hist
+        for a, b in zip(model.state_dict().values(), twin.state_dict().values()):
+            assert torch.equal(a, b)
     assert [h['grad_bitwidth'] for h in hist] == [5, 5, 5, 4]
     assert hist[0]['val_prec1'] < 60.0 and max(h['val_prec1'] for h in hist) > 80.0, hist
     assert sorted(os.listdir(tmp_path)) == ['checkpoint_epoch_0.pth.tar', 'checkpoint_epoch_1.pth.tar', 'checkpoint_epoch_2.pth.tar',
