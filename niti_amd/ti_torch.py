@@ -295,7 +295,9 @@ WEIGHT_INIT_METHOD = UniformWeights
 
 def TiFloatToInt8(input):
     """ti_torch.py:341-356: float tensor -> (int8 tensor on the GPU, exponent).  The exponent is
-    returned as a 0-d float tensor like the reference; no host synchronisation."""
+    returned as a 0-d float tensor like the reference; no host synchronisation.  The range is a tensor-library
+    reduction, whose multi-block form clears its scratch words with a memset node: keep this call outside a captured
+    HIP graph (train.StepGraph quantises eagerly and captures forward_int8 + backward)."""
     input = input.to(GPU)
     input_range = torch.max(torch.abs(input))
     input_bitwidth = torch.ceil(torch.log2(input_range))
