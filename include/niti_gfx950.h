@@ -264,6 +264,14 @@ int niti_weight_update_i8(int8_t* w, const int8_t* g, int64_t n, void* stream);
 int niti_relu_i8_fwd(const int8_t* x, int8_t* y, int64_t n, void* stream);
 int niti_relu_i8_bwd(const int8_t* act, const int8_t* dy, int8_t* dx, int64_t n, void* stream);
 
+/* TiFloatToInt8 (ti_torch.py:341-356) and the NCHW -> NHWC change that follows it (ti_net.py:19), two launches:
+   r = max|x|, bw = ceil(log2 r), y = int8(clamp(round_half_even(x * 2^(bits - bw)), -128, 127)), *exp_out = bw - bits.
+   x: float [N,C,H,W]; y: int8 [N,H,W,cpad] with channels C..cpad-1 zero (cpad % 4 == 0; 16 feeds the convolution kernels
+   directly); absmax_bits: one ZEROED word that receives the bits of r.  An all-zero batch gives zeros and exponent 0
+   (the reference's float sequence produces NaN there). */
+int niti_quantize_f32_i8(const float* x, int8_t* y, int N, int C, int H, int W, int cpad, int bits, uint32_t* absmax_bits,
+                         int32_t* exp_out, void* stream);
+
 /* TiDropout (ti_torch.py:439-455): y[m][f] = x[m][f] * mask[f] with one keep (1) / drop (0) byte per feature, and - when
    exp_out is given - exp_out = exp_in + exp_add (the layer raises the exponent by one; exp_in NULL counts as 0), as one
    launch.  The backward pass is the same product on the error (exp_out NULL).  features % 16 == 0, 16-byte aligned. */

@@ -55,6 +55,7 @@ SIGNATURES = {
     "niti_relu_i8_fwd": (_i, [_vp, _vp, _i64, _vp]),
     "niti_relu_i8_bwd": (_i, [_vp, _vp, _vp, _i64, _vp]),
     "niti_mask_features_i8": (_i, [_vp, _vp, _vp, _i64, _i, _vp, _vp, _i, _vp]),
+    "niti_quantize_f32_i8": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "niti_maxpool_i8_fwd": (_i, [_vp, _vp] + [_i] * 7 + [_vp]),
     "niti_maxpool_i8_bwd": (_i, [_vp, _vp, _vp, _vp] + [_i] * 8 + [_vp]),
     "niti_fc_i8_sync_words": (_sz, [_i] * 4),

@@ -122,6 +122,53 @@ __global__ __launch_bounds__(256) void weight_update_kernel(int8_t* w, const int
     w[i] = static_cast<int8_t>(clip127(static_cast<int>(w[i]) - static_cast<int>(g[i])));
 }
 
+// ---- input quantiser (TiFloatToInt8, ti_torch.py:341-356) with the layout change that follows it (ti_net.py:19) ----
+// r = max |x| over the batch (float bits of non-negative values order like unsigned integers)
+__global__ __launch_bounds__(256) void absmax_f32_kernel(const float* __restrict__ x, int64_t n, uint32_t* __restrict__ out) {
+  __shared__ uint32_t wmax[4];
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  uint32_t m = 0;
+  for (int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; i < n; i += stride) {
+    const uint32_t b = __float_as_uint(x[i]) & 0x7FFFFFFFu;
+    m = b > m ? b : m;
+  }
+  m = wave_max_u32(m);
+  if ((threadIdx.x & 63) == 0) wmax[threadIdx.x >> 6] = m;
+  __syncthreads();
+  if (threadIdx.x < 64) fold_absmax(out, threadIdx.x < 4 ? wmax[threadIdx.x] : 0u);
+}
+
+// bw = ceil(log2 r); y = int8(clamp(round_half_even(x * 2^(bits - bw)), -128, 127)), float NCHW -> int8 NHWC with the
+// channels zero-padded to cpad; exp_out = bw - bits.  The float operations are the reference's, one by one.
+__global__ __launch_bounds__(256) void quantize_f32_i8_kernel(const float* __restrict__ x, int8_t* __restrict__ y, int64_t pixels,
+                                                              int C, int HW, int cpad, const uint32_t* __restrict__ absmax_bits,
+                                                              int32_t* exp_out, int bits) {
+  const float r = __uint_as_float(*absmax_bits);
+  const float bw = ceilf(log2f(r));
+  const float scale = powf(2.0f, static_cast<float>(bits) - bw);
+  if (blockIdx.x == 0 && threadIdx.x == 0 && exp_out != nullptr) *exp_out = r > 0.0f ? static_cast<int>(bw) - bits : 0;
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
+  for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < pixels; p += stride) {
+    const int64_t n = p / HW, hw = p - n * HW;
+    const float* src = x + n * C * HW + hw;
+    int8_t* dst = y + p * cpad;
+    for (int c0 = 0; c0 < cpad; c0 += 4) {
+      uint32_t word = 0;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const int c = c0 + e;
+        int q = 0;
+        if (c < C && r > 0.0f) {
+          const float v = fminf(fmaxf(rintf(src[static_cast<int64_t>(c) * HW] * scale), -128.0f), 127.0f);
+          q = static_cast<int>(v);
+        }
+        word |= (static_cast<uint32_t>(q) & 0xFFu) << (8 * e);
+      }
+      *reinterpret_cast<uint32_t*>(dst + c0) = word;
+    }
+  }
+}
+
 // y[m][f] = x[m][f] * mask[f] with mask bytes 0 / 1 (a keep / drop decision per feature); optionally exp_out = exp_in + add
 __global__ __launch_bounds__(256) void mask_features_kernel(const int8_t* __restrict__ x, const int8_t* __restrict__ mask,
                                                             int8_t* __restrict__ y, int64_t rows, int features,
@@ -267,6 +314,21 @@ extern "C" int niti_relu_i8_fwd(const int8_t* x, int8_t* y, int64_t n, void* str
   hipLaunchKernelGGL(relu_kernel<false>, dim3(grid_for((n + 15) / 16, 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
                      x, static_cast<const int8_t*>(nullptr), y, n);
   return check_launch("relu_fwd");
+}
+
+extern "C" int niti_quantize_f32_i8(const float* x, int8_t* y, int N, int C, int H, int W, int cpad, int bits, uint32_t* absmax_bits,
+                                    int32_t* exp_out, void* stream) {
+  clear_error();
+  if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || cpad < C || cpad % 4 != 0 || bits < 1 || bits > 7)
+    return fail(NITI_ERR_INVALID_ARG, "quantize: N=%d C=%d H=%d W=%d cpad=%d bits=%d", N, C, H, W, cpad, bits);
+  if (x == nullptr || y == nullptr || absmax_bits == nullptr) return fail(NITI_ERR_INVALID_ARG, "quantize: null pointer");
+  if (reinterpret_cast<uintptr_t>(y) % 4 != 0) return fail(NITI_ERR_INVALID_ARG, "quantize: output must be 4-byte aligned");
+  const int64_t pixels = static_cast<int64_t>(N) * H * W, n = pixels * C;
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  hipLaunchKernelGGL(absmax_f32_kernel, dim3(grid_for(n, 256, 1024)), dim3(256), 0, s, x, n, absmax_bits);
+  hipLaunchKernelGGL(quantize_f32_i8_kernel, dim3(grid_for(pixels, 256)), dim3(256), 0, s, x, y, pixels, C, H * W, cpad, absmax_bits,
+                     exp_out, bits);
+  return check_launch("quantize");
 }
 
 extern "C" int niti_mask_features_i8(const int8_t* x, const int8_t* mask, int8_t* y, int64_t rows, int features,

@@ -401,6 +401,22 @@ def relu_fwd(x):
     return y
 
 
+def quantize_input(x, bits=7, cpad=16):
+    """Float NCHW batch -> (int8 NHWC batch with the channels zero-padded to ``cpad``, exponent as a 1-element int32
+    tensor): the reference's input quantiser and the layout change behind it in two launches."""
+    _chk_dev(x)
+    if x.dtype != torch.float32 or x.dim() != 4 or not x.is_contiguous():
+        raise RuntimeError("quantize_input: contiguous float32 [N,C,H,W] tensor expected")
+    N, C, H, W = x.shape
+    cpad = max(cpad, (C + 3) // 4 * 4)
+    y = torch.empty((N, H, W, cpad), dtype=torch.int8, device=x.device)
+    am = torch.zeros(1, dtype=torch.int32, device=x.device)
+    exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
+    L.check(L.lib().niti_quantize_f32_i8(_ptr(x), _ptr(y), N, C, H, W, cpad, bits, _ptr(am), _ptr(exp_out), _stream(x)),
+            "niti_quantize_f32_i8")
+    return y, exp_out
+
+
 def mask_features(x, mask, exp_in=None, exp_add=None):
     """x [rows, F] int8 times a keep / drop byte per feature (mask [F] int8 0/1) in one launch.  With ``exp_add`` also
     returns a 1-element int32 tensor holding exp_in + exp_add."""

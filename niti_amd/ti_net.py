@@ -45,9 +45,19 @@ class TiNet(Module):
 
     def forward(self, x):
         """ti_net.py:17-23: float NCHW batch -> (int8 logits, exponent)."""
-        x_data, x_exp = ti_torch.TiFloatToInt8(x)
-        x_data = x_data.permute(0, 2, 3, 1).contiguous()
+        x_data, x_exp = self.quantize_input(x)
         return self.forward_int8(x_data, x_exp)
+
+    @staticmethod
+    def quantize_input(x):
+        """TiFloatToInt8 + NCHW -> NHWC (ti_net.py:18-19): (int8 NHWC batch, exponent).  A contiguous float32 batch on
+        the GPU takes the library's two launches (channels come zero-padded to 16, which the first convolution
+        would do next anyway); anything else the reference's tensor operations."""
+        x = x.to(ti_torch.GPU)
+        if x.dtype == torch.float32 and x.dim() == 4 and x.is_contiguous() and x.is_cuda:
+            return ops.quantize_input(x, ti_torch.BITWIDTH)
+        x_data, x_exp = ti_torch.TiFloatToInt8(x)
+        return x_data.permute(0, 2, 3, 1).contiguous(), x_exp
 
     def forward_int8(self, x_data, x_exp=0):
         """Same as forward() for a batch that already is int8 NHWC with exponent ``x_exp``."""

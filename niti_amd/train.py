@@ -68,8 +68,8 @@ class StepGraph:
 
     def __init__(self, model, training, inputs, target, eager_steps=3):
         self.model, self.training = model, training
-        n, c, h, w = inputs.shape
-        self.x8 = torch.empty((n, h, w, c), dtype=torch.int8, device=inputs.device)     # quantised batch, NHWC
+        x_data, _ = model.quantize_input(inputs)
+        self.x8 = torch.empty_like(x_data)                                               # quantised batch, NHWC
         self.x_exp = torch.empty(1, dtype=torch.int32, device=inputs.device)
         self.target = torch.empty_like(target)
         self.graph, self.failed, self.eager_left = None, False, eager_steps
@@ -82,8 +82,8 @@ class StepGraph:
             self.model.backward(self.target)
 
     def __call__(self, inputs, target, sums):
-        x_data, x_exp = ti_torch.TiFloatToInt8(inputs)          # ti_net.py:17-19
-        self.x8.copy_(x_data.permute(0, 2, 3, 1))
+        x_data, x_exp = self.model.quantize_input(inputs)       # ti_net.py:17-19
+        self.x8.copy_(x_data)
         self.x_exp.copy_(x_exp.reshape(1))
         self.target.copy_(target, non_blocking=True)
         if self.graph is not None:

@@ -747,6 +747,28 @@ def test_maxpool(dev, case):
             assert torch.equal(dxr.cpu(), torch.where(x > 0, ref, torch.zeros_like(ref))), ties
 
 
+def test_quantize_input(dev):
+    """The input quantiser as two launches against the reference's tensor operations (same device functions, so the
+    results are equal), including ranges at and next to a power of two, where ceil(log2 r) jumps."""
+    from niti_amd import ops, ti_torch
+    _say("quantize_input")
+    g = torch.Generator().manual_seed(77)
+    for shape, top in (((128, 3, 32, 32), None), ((5, 3, 7, 9), 4.0), ((2, 3, 8, 8), 4.000001), ((2, 3, 8, 8), 3.9999998),
+                       ((3, 17, 4, 4), 0.3), ((1, 1, 1, 1), 100.0)):
+        x = torch.randn(shape, generator=g)
+        if top is not None:
+            x = x / x.abs().max() * 0.9 * top
+            x.view(-1)[min(3, x.numel() - 1)] = -top
+        xd = x.to(dev)
+        ref, ref_exp = ti_torch.TiFloatToInt8(xd)
+        y, e = ops.quantize_input(xd)
+        C = shape[1]
+        assert y.shape[3] == max(16, (C + 3) // 4 * 4) and int(e.cpu()) == int(ref_exp.cpu())
+        assert torch.equal(y[..., :C], ref.permute(0, 2, 3, 1)) and int(y[..., C:].abs().max()) == 0
+    y, e = ops.quantize_input(torch.zeros((2, 3, 4, 4), device=dev))
+    assert int(y.abs().max()) == 0 and int(e.cpu()) == 0
+
+
 def test_mask_features(dev):
     """Dropout as one launch: a keep / drop byte per feature times every row, exponent + 1."""
     from niti_amd import ops
