@@ -46,6 +46,13 @@ def build(verbose: bool = False) -> str:
     r = subprocess.run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs], capture_output=True, text=True)
     if r.returncode != 0:
         raise RuntimeError("link failed:\n%s\n%s" % (r.stdout, r.stderr))
+    # a shared library links with undefined symbols left in it: resolve them all now, in a child process, so that
+    # a library that cannot be loaded is never installed
+    chk = subprocess.run([sys.executable, "-c", "import ctypes, os, sys; ctypes.CDLL(sys.argv[1], mode=os.RTLD_NOW)", tmp],
+                         capture_output=True, text=True)
+    if chk.returncode != 0:
+        os.unlink(tmp)
+        raise RuntimeError("the linked library does not load:\n" + chk.stderr[-2000:])
     os.replace(tmp, SO)
     if verbose:
         print("built", SO, os.path.getsize(SO), "bytes")

@@ -39,18 +39,22 @@ namespace niti {
 namespace {
 
 constexpr int kOob = -1;
+constexpr int kOobFar = static_cast<int>(0x80000000u);   // out of range whatever scalar offset below 2^31 is added
 
-// s_waitcnt vmcnt(n) with the other counters left alone; n is wavefront-uniform and small
-__device__ inline void hc_wait_vmcnt_dyn(int n) {
-  switch (n) {
-    case 0: __builtin_amdgcn_s_waitcnt(0x0F70); break;
-    case 1: __builtin_amdgcn_s_waitcnt(0x0F71); break;
-    case 2: __builtin_amdgcn_s_waitcnt(0x0F72); break;
-    case 3: __builtin_amdgcn_s_waitcnt(0x0F73); break;
-    case 4: __builtin_amdgcn_s_waitcnt(0x0F74); break;
-    case 5: __builtin_amdgcn_s_waitcnt(0x0F75); break;
-    default: __builtin_amdgcn_s_waitcnt(0x0F76); break;
-  }
+// s_waitcnt vmcnt(N) with the other counters left alone
+template <int N>
+__device__ inline void hc_wait_vmcnt() {
+  static_assert(N >= 0 && N <= 15);
+  __builtin_amdgcn_s_waitcnt(0x0F70 | N);
+}
+// the same for a wavefront that has N loads in flight if it issues the full number of filter loads per stage and
+// N - 1 if it issues one fewer (the count is an immediate, so the choice is a branch on a wavefront-uniform flag)
+template <int N>
+__device__ inline void hc_wait_vmcnt_pair(bool full) {
+  if (full)
+    hc_wait_vmcnt<N>();
+  else
+    hc_wait_vmcnt<N - 1>();
 }
 __device__ inline void hc_sync() {
   asm volatile("" ::: "memory");
@@ -178,9 +182,14 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.x), 0, a.x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.wp), 0, a.wp_bytes, 0x00020000);
 
-  // ---- activation staging: an instruction fills 32 consecutive slots; lane -> (slot lane/2, half lane%2)
-  int act_off[G::ACT_LOADS];   // byte offset of this lane's 16 bytes for channel slice 0, or kOob
-  int act_c16[G::ACT_LOADS];   // which 16 channels of a slice this lane fetches (0 / 16)
+  // ---- activation staging: an instruction fills 32 consecutive slots; lane -> (slot lane/2, half lane%2).
+  // A lane's offset is split into a part fixed for the whole launch (vector register) and the slice's 32 * cs
+  // (scalar offset of the load), so a stage spends no vector arithmetic on it.  A lane with nothing to fetch
+  // holds kOobFar, which no scalar offset below 2^31 brings back into range: the load then writes zeros.
+  int act_off[G::ACT_LOADS];        // byte offset of this lane's 16 bytes for channel slice 0, or kOobFar
+  int act_off_last[G::ACT_LOADS];   // the same for the last slice, whose upper 16 channels may not exist
+  unsigned act_dst[G::ACT_LOADS];   // LDS byte address inside activation buffer 0, or the dump slot
+  const unsigned act_lds = lds_addr(act_buf), w_lds = lds_addr(w_buf), dump_lds = lds_addr(dump);
 #pragma unroll
   for (int i = 0; i < G::ACT_LOADS; ++i) {
     const int slot = (wave + 8 * i) * 32 + (lane >> 1);
@@ -188,20 +197,23 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const int ni = row / G::HR, h = row - ni * G::HR;
     const int half = (lane & 1) ^ (((col >> 3) ^ row) & 1);
     const int ih = p0 + h - 1, iw = col;
-    int off = kOob;
+    int off = kOobFar;
     if (slot < G::SLOTS && n0 + ni < a.N && ih >= 0 && ih < Q && iw >= 0 && iw < Q)
       off = (((n0 + ni) * Q + ih) * Q + iw) * a.C + half * 16;
     act_off[i] = off;
-    act_c16[i] = half * 16;
+    act_off_last[i] = (a.cslices - 1) * 32 + half * 16 < a.C ? off : kOobFar;
+    act_dst[i] = wave + 8 * i < G::ACT_INSTR ? act_lds + (wave + 8 * i) * 1024 : dump_lds;
   }
   auto issue_act = [&](int cs, int buf) {
+    const bool last = cs == a.cslices - 1;
+    const unsigned shift = buf * G::ACT_BYTES;
 #pragma unroll
     for (int i = 0; i < G::ACT_LOADS; ++i) {
-      const int idx = wave + 8 * i;
-      int off = act_off[i];
-      if (off != kOob) off = (cs * 32 + act_c16[i] < a.C) ? off + cs * 32 : kOob;
-      int8_t* dst = idx < G::ACT_INSTR ? act_buf + buf * G::ACT_BYTES + idx * 1024 : dump;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, NITI_LDS(dst), 16, off, 0, 0, 0);
+      const unsigned dst = wave + 8 * i < G::ACT_INSTR ? act_dst[i] + shift : act_dst[i];
+      // through a local: with the array element written in the call itself the host pass of the compiler emitted no
+      // launch stub for any instantiation of this kernel (the library then fails to load with an undefined symbol)
+      const int off = last ? act_off_last[i] : act_off[i];
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rx, NITI_LDS_AT(dst), 16, off, cs * 32, 0, 0);
     }
   };
   // ---- filter staging.  The copy is [64-channel group][slice][tap][64 rows][32 bytes]: the three taps of a
@@ -213,36 +225,35 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   // A group beyond the last one (K not a multiple of 128) re-reads the last group instead of reading out of
   // range: its sums are never stored.
   const int ngroups = (a.K + 63) / 64;
-  const int wl = (G::W_INSTR - wave + 7) / 8;   // filter loads of this wavefront per stage
+  constexpr int WL = (G::W_INSTR + 7) / 8;               // filter loads per stage of the wavefronts that issue most
+  const bool wfull = wave + 8 * (WL - 1) < G::W_INSTR;   // this wavefront is one of them; the others issue WL - 1
+  static_assert(WL + G::ACT_LOADS <= 15);
+  // kWT with one filter row per stage: a later row is an earlier tap, i.e. a step back of up to 6 taps; the lane's
+  // part gives up those 6 taps (its smallest tap is 6) so that the scalar part never goes below zero
+  constexpr int wback = (kWT && G::RPS == 1) ? 6 * 2048 : 0;
   auto w_src = [&](int q) {  // instruction q of a stage -> byte offset in the copy for slice 0, filter row 0
     if (kWT) {
       // KB q of a stage holds tap q / (KT/32) of the stage and 32-channel slice q % (KT/32) of this tile's output
       // channels: rows = 32 reduction channels (half a 64-row group of the forward copy), 32 bytes = 32 outputs
       const int cs = min(kt * (KT / 32) + q % (KT / 32), a.src_cslices - 1);
-      return (cs * 9 + 8 - q / (KT / 32)) * 2048 + lane * 16;
+      return (cs * 9 + 8 - q / (KT / 32)) * 2048 + lane * 16 - wback;
     }
     const int g = min(KT == 128 ? kt * 2 + q / 6 : kt, ngroups - 1);
     return g * a.cslices * (9 * 2048) + (KT == 128 ? q % 6 : q) * 1024 + lane * 16;
   };
+  // The per-lane part of the three offsets is fixed for the launch; slice and filter row go into the scalar offset.
   const int wsrc_a = w_src(wave), wsrc_b = w_src(wave + 8), wsrc_c = w_src(wave + 16);
+  const unsigned wdst = w_lds + wave * 1024;
   auto issue_w = [&](int cs, int r, int st) {
     // kWT: reduction slice cs = rows (cs & 1) * 32.. of group cs >> 1; a later filter row is an earlier forward tap
-    const int rel = kWT ? (cs >> 1) * a.src_cslices * (9 * 2048) + (cs & 1) * 1024 - r * 3 * 2048 : (cs * 9 + r * 3) * 2048;
-    if (wave < G::W_INSTR) {
-      int8_t* dst = w_buf + st * G::W_BYTES + wave * 1024;
-      const int off = wsrc_a + rel;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
-    }
-    if (wave + 8 < G::W_INSTR) {
-      int8_t* dst = w_buf + st * G::W_BYTES + (wave + 8) * 1024;
-      const int off = wsrc_b + rel;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
-    }
-    if (wave + 16 < G::W_INSTR) {
-      int8_t* dst = w_buf + st * G::W_BYTES + (wave + 16) * 1024;
-      const int off = wsrc_c + rel;
-      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS(dst), 16, off, 0, 0, 0);
-    }
+    const int rel =
+        kWT ? (cs >> 1) * a.src_cslices * (9 * 2048) + (cs & 1) * 1024 - r * 3 * 2048 + wback : (cs * 9 + r * 3) * 2048;
+    const unsigned dst = wdst + st * G::W_BYTES;
+    if (wave < G::W_INSTR) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst), 16, wsrc_a, rel, 0, 0);
+    if (wave + 8 < G::W_INSTR)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst + 8 * 1024), 16, wsrc_b, rel, 0, 0);
+    if (wave + 16 < G::W_INSTR)
+      __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst + 16 * 1024), 16, wsrc_c, rel, 0, 0);
   };
 
   // ---- fragment addressing
@@ -455,9 +466,16 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
       for (int r = 0; r < 3; ++r) {
         const int t = ci * 3 + r;
-        int young = t + 1 < nst ? wl : 0;
-        if (r >= 1 && more) young += G::ACT_LOADS;   // issued in the first stage of this slice, after W(t) went out
-        hc_wait_vmcnt_dyn(young);
+        // younger than W(t): W(t+1) if there is one, and from the second stage of a slice on the next slice's
+        // activations (issued in the first stage of this slice, after W(t) went out)
+        if (r == 0 || !more) {
+          if (r < 2 || more)
+            hc_wait_vmcnt_pair<WL>(wfull);
+          else
+            hc_wait_vmcnt<0>();
+        } else {
+          hc_wait_vmcnt_pair<WL + G::ACT_LOADS>(wfull);
+        }
         hc_sync();
         if (t + 2 < nst) {
           const int c2 = r == 0 ? ci : ci + 1, r2 = r == 0 ? 2 : r - 1;
@@ -476,7 +494,10 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     if (a.cslices > 1) issue_w(1, 0, 1);
     for (int ci = 0; ci < a.cslices; ++ci) {
       const int8_t* sa = act_buf + (ci & 1) * G::ACT_BYTES;
-      hc_wait_vmcnt_dyn(ci + 1 < a.cslices ? wl : 0);
+      if (ci + 1 < a.cslices)
+        hc_wait_vmcnt_pair<WL>(wfull);
+      else
+        hc_wait_vmcnt<0>();
       hc_sync();
       if (ci + 1 < a.cslices) issue_act(ci + 1, (ci + 1) & 1);
       if (ci + 2 < a.cslices) issue_w(ci + 2, 0, (ci + 2) % G::WSTAGES);

@@ -7,6 +7,8 @@
 namespace niti {
 
 #define NITI_LDS(p) ((__attribute__((address_space(3))) void*)(p))
+// the same from a 32-bit LDS byte address (no generic pointer, hence no null test in scalar code)
+#define NITI_LDS_AT(addr) (reinterpret_cast<__attribute__((address_space(3))) void*>(static_cast<unsigned>(addr)))
 
 // ds_read_b64_tr_b8 as inline assembly.  Before the builtin form the compiler places s_waitcnt vmcnt(0) whenever a
 // buffer_load ... lds is in flight (it cannot tell which LDS bytes that load writes), which would make every stage
