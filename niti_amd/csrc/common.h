@@ -12,6 +12,16 @@
 
 namespace niti {
 
+// Launch set-up that holds per device (a kernel's function attributes, how many workgroups the device holds at
+// once) is cached in arrays of this many entries, indexed by device_slot().
+constexpr int kDeviceSlots = 64;
+inline int device_slot() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0) dev = 0;
+  return dev % kDeviceSlots;
+}
+
+
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v2i __attribute__((ext_vector_type(2)));
 typedef int v16i __attribute__((ext_vector_type(16)));

@@ -961,7 +961,8 @@ __global__ __launch_bounds__(256) void halo_filter_prepare_kernel(const int8_t* 
 // Channel tile of a launch: 128 unless that leaves fewer workgroups than the device runs at once while
 // a tile of 64 would give it more to do.
 int halo_ktile(long long pix, int K, int H) {
-  static int cus = 0;
+  static int cus_of[kDeviceSlots] = {};
+  int& cus = cus_of[device_slot()];
   if (cus == 0) {
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0)
@@ -993,8 +994,11 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
   static_assert(8 * 64 * (G::NWF * 32 + 16) <= G::TILE_BYTES, "int8 patches must stay clear of the reduction words");
   static_assert(2 * lds <= 160 * 1024, "two workgroups per compute unit");
   auto k = conv3x3_halo_kernel<Q, BR, NI, KT, kFused, kWT>;
-  static bool attr_set = false;
-  static int resident = 0;  // workgroups the device holds at once
+  static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
+  static int resident_of[kDeviceSlots] = {};     // workgroups the device holds at once
+  const int slot = device_slot();
+  bool& attr_set = attr_set_of[slot];
+  int& resident = resident_of[slot];
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return fail(NITI_ERR_LAUNCH, "conv3x3_halo: cannot reserve %zu bytes of LDS", lds);
@@ -1031,8 +1035,11 @@ template <bool kFused, bool kWT>
 int launch_map2(const HaloArgs& a, hipStream_t stream) {
   constexpr size_t lds = map2_lds_bytes(kWT);
   auto k = conv3x3_map2_kernel<kFused, kWT>;
-  static bool attr_set = false;
-  static int resident = 0;  // workgroups the device holds at once
+  static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
+  static int resident_of[kDeviceSlots] = {};     // workgroups the device holds at once
+  const int slot = device_slot();
+  bool& attr_set = attr_set_of[slot];
+  int& resident = resident_of[slot];
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return fail(NITI_ERR_LAUNCH, "conv3x3_map2: cannot reserve %zu bytes of LDS", lds);

@@ -293,7 +293,8 @@ int launch_cfg(const ConvArgs& a_in, int split, hipStream_t stream) {
   dim3 grid((a.M + BM - 1) / BM, (a.K + BN - 1) / BN, split);
   dim3 block(WVM * WVN * 64);
   if (grid.y > 65535u || grid.z > 65535u) return fail(NITI_ERR_UNSUPPORTED, "conv: K=%d too large", a.K);
-  static bool attr_set[2] = {false, false};
+  static bool attr_set_of[kDeviceSlots][2] = {};   // function attributes are per device
+  bool* const attr_set = attr_set_of[device_slot()];
   if (split > 1) {
     auto k = conv_mfma_kernel<WVM, WVN, WP, WC, STAGES, BK, true>;
     if (!attr_set[1]) {

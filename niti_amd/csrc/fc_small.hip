@@ -399,7 +399,8 @@ extern "C" int niti_fc_i8_fwd_requant(const int8_t* act, const int8_t* w, int8_t
   a.w = const_cast<int8_t*>(w);
   a.out8 = out8;
   a.rq_flags = rq_flags;
-  static int resident = 0;
+  static int resident_of[kDeviceSlots] = {};
+  int& resident = resident_of[device_slot()];
   if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_fwd_requant_kernel), 1024);
   if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "fc_fwd_requant: %lld workgroups do not fit on the device at once (%d)", nb, resident);
   a.kchunk = fwd_chunk(F);
@@ -418,7 +419,8 @@ extern "C" int niti_fc_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8
   if (st != NITI_OK) return st;
   if (err == nullptr || w == nullptr || dx8 == nullptr) return fail(NITI_ERR_INVALID_ARG, "fc_dgrad_requant: null pointer");
   if (!aligned16(w) || !aligned16(dx8)) return fail(NITI_ERR_INVALID_ARG, "fc_dgrad_requant: w and dx8 must be 16-byte aligned");
-  static int resident = 0;
+  static int resident_of[kDeviceSlots] = {};
+  int& resident = resident_of[device_slot()];
   if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_dgrad_requant_kernel));
   if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "fc_dgrad_requant: %lld workgroups do not fit on the device at once (%d)", nb, resident);
   a.err = err;
@@ -440,7 +442,8 @@ extern "C" int niti_fc_i8_wgrad_update(const int8_t* err, const int8_t* act, int
   if (err == nullptr || act == nullptr || w == nullptr) return fail(NITI_ERR_INVALID_ARG, "fc_wgrad_update: null pointer");
   if (reinterpret_cast<uintptr_t>(act) % 4 != 0 || reinterpret_cast<uintptr_t>(w) % 4 != 0 || reinterpret_cast<uintptr_t>(g8_out) % 4 != 0)
     return fail(NITI_ERR_INVALID_ARG, "fc_wgrad_update: act, w and g8_out must be 4-byte aligned");
-  static int resident = 0;
+  static int resident_of[kDeviceSlots] = {};
+  int& resident = resident_of[device_slot()];
   if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_wgrad_update_kernel));
   if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "fc_wgrad_update: %lld workgroups do not fit on the device at once (%d)", nb, resident);
   a.err = err;

@@ -766,7 +766,8 @@ int launch_narrow_geom(const WgradArgs& a, int splits, hipStream_t stream) {
   using G = NGeom<Q, BR, NI>;
   constexpr size_t lds = G::LDS_BYTES;
   auto k = wgrad3x3_narrow_kernel<Q, BR, NI>;
-  static bool attr_set = false;
+  static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
+  bool& attr_set = attr_set_of[device_slot()];
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return fail(NITI_ERR_LAUNCH, "wgrad: cannot reserve %zu bytes of LDS", lds);
@@ -784,7 +785,8 @@ int launch_geom(const WgradArgs& a, int splits, hipStream_t stream) {
   constexpr size_t lds = static_cast<size_t>(STAGES) * G::STAGE_BYTES + 1024;
   static_assert(lds <= 160 * 1024, "stages must fit in LDS");
   auto k = wgrad3x3_kernel<Q, BR, NI, STAGES>;
-  static bool attr_set = false;
+  static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
+  bool& attr_set = attr_set_of[device_slot()];
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return fail(NITI_ERR_LAUNCH, "wgrad: cannot reserve %zu bytes of LDS", lds);
@@ -875,7 +877,8 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   const int nb = wgrad3x3_finish_blocks(Cp, K);
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large for the single-pass finish", K, C);
   if (static_cast<long long>(K) * 9 * C >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large", K, C);
-  static int resident[2] = {0, 0};   // workgroups of 4 / 16 wavefronts the device holds at once
+  static int resident_of[kDeviceSlots][2] = {};   // workgroups of 4 / 16 wavefronts the device holds at once
+  int* const resident = resident_of[device_slot()];
   if (resident[0] == 0) {
     int dev = 0, cus = 0, per4 = 0, per16 = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
