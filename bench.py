@@ -66,7 +66,6 @@ class ConvTriple:
             L["shift_d"] = torch.zeros(1, dtype=torch.int32, device=dev)
             L["shift_w"] = torch.zeros(1, dtype=torch.int32, device=dev)
             self.layers.append(L)
-        self.absmax = torch.zeros(3 * len(LAYERS), dtype=torch.int32, device=dev)
         # zeroed words the single-launch conv + requantisation kernels exchange their tile ranges through
         off = 0
         for L in self.layers:
@@ -78,7 +77,11 @@ class ConvTriple:
             n = ops.wgrad_update_sync_words(BATCH, L["hw"], L["hw"], L["x16"].shape[3], L["k"])
             L["sync_w"] = (off, n)
             off += n
-        self.sync = torch.zeros(max(off, 1), dtype=torch.int32, device=dev)
+        # one buffer, hence one fill per step: the sync words, then (256-byte aligned) the ranges of the two-pass paths
+        sync_words = (max(off, 1) + 63) // 64 * 64
+        self.zeroed = torch.zeros(sync_words + 3 * len(LAYERS), dtype=torch.int32, device=dev)
+        self.sync = self.zeroed[:sync_words]
+        self.absmax = self.zeroed[sync_words:]
         self.ws = ops.scratch(256 << 20, dev)    # shared by all weight-gradient launches
         self.exp0 = torch.zeros(1, dtype=torch.int32, device=dev)
         self.ops_per_step = sum(conv_ops(BATCH, hw, c, k) * (2 if i == 0 else 3) for i, (c, k, hw) in enumerate(LAYERS))
@@ -88,8 +91,7 @@ class ConvTriple:
     def step(self, record=False):
         torch, ops = self.torch, self.ops
         import torch.nn.functional as F
-        self.absmax.zero_()
-        self.sync.zero_()
+        self.zeroed.zero_()
         for i, L in enumerate(self.layers):
             c, k, hw = L["c"], L["k"], L["hw"]
             am = self.absmax[3 * i: 3 * i + 3]
