@@ -30,7 +30,7 @@ enum {
   NITI_ERR_LAUNCH = 4       /* HIP reported a launch error */
 };
 
-/* conv / gemm flags */
+/* conv / gemm flags; a bit that the entry point called does not define is NITI_ERR_INVALID_ARG, not ignored */
 #define NITI_EPI_F32_ROUNDTRIP 1u /* pass every int32 result through fp32 and back, as the
                                      reference's CUTLASS epilogue does
                                      (pytorch/cutlass-extension/cutlassconv_kernel.cu:78-85) */

@@ -79,6 +79,12 @@ static int check_conv_dims(const char* who, int N, int H, int W, int C, int K, i
   return NITI_OK;
 }
 
+// bits outside `allowed` are refused rather than ignored: a caller built against a newer header finds out at once
+static int check_flags(const char* who, unsigned flags, unsigned allowed) {
+  if ((flags & ~allowed) != 0u) return fail(NITI_ERR_INVALID_ARG, "%s: flags=%#x (accepted: %#x)", who, flags, allowed);
+  return NITI_OK;
+}
+
 static bool halo_off() {
   static int v = -1;
   if (v < 0) {
@@ -155,6 +161,7 @@ extern "C" int niti_conv2d_i8_fprop(const int8_t* x, const int8_t* w, int32_t* y
                                     size_t workspace_bytes, void* stream) {
   clear_error();
   int st = check_conv_dims("conv_fprop", N, H, W, C, K, R, S, stride, pad);
+  if (st == NITI_OK) st = check_flags("conv_fprop", flags, NITI_EPI_F32_ROUNDTRIP | NITI_CONV_FILTER_PREPARED);
   if (st != NITI_OK) return st;
   if (x == nullptr || w == nullptr || y == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: null pointer");
   if (!aligned16(x) || !aligned16(w) || !aligned16(y)) return fail(NITI_ERR_INVALID_ARG, "conv_fprop: pointers must be 16-byte aligned");
@@ -187,6 +194,8 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
                                     size_t workspace_bytes, void* stream) {
   clear_error();
   int st = check_conv_dims("conv_dgrad", N, H, W, C, K, R, S, stride, pad);
+  if (st == NITI_OK)
+    st = check_flags("conv_dgrad", flags, NITI_EPI_F32_ROUNDTRIP | NITI_CONV_FILTER_PREPARED | NITI_CONV_FILTER_FORWARD_COPY);
   if (st != NITI_OK) return st;
   if (err == nullptr || w == nullptr || dx == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_dgrad: null pointer");
   if (stride != 1 || R != S || pad > R - 1)
@@ -252,6 +261,8 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
                         size_t workspace_bytes, void* stream, int8_t* pool_out = nullptr) {
   clear_error();
   int st = check_conv_dims(who, N, H, W, C, K, R, S, stride, pad);
+  if (st == NITI_OK)
+    st = check_flags(who, flags, NITI_EPI_F32_ROUNDTRIP | NITI_CONV_FILTER_PREPARED | (dgrad ? NITI_CONV_FILTER_FORWARD_COPY : 0u));
   if (st != NITI_OK) return st;
   if (x == nullptr || w == nullptr || y8 == nullptr || sync == nullptr) return fail(NITI_ERR_INVALID_ARG, "%s: null pointer", who);
   if (!aligned16(x) || !aligned16(w) || !aligned16(y8)) return fail(NITI_ERR_INVALID_ARG, "%s: pointers must be 16-byte aligned", who);
@@ -334,6 +345,7 @@ extern "C" int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_
                                     size_t workspace_bytes, void* stream) {
   clear_error();
   int st = check_conv_dims("conv_wgrad", N, H, W, C, K, R, S, stride, pad);
+  if (st == NITI_OK) st = check_flags("conv_wgrad", flags, NITI_EPI_F32_ROUNDTRIP);
   if (st != NITI_OK) return st;
   if (act == nullptr || err == nullptr || dw == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_wgrad: null pointer");
   if (stride != 1) return fail(NITI_ERR_UNSUPPORTED, "conv_wgrad: stride %d (only 1)", stride);
@@ -386,6 +398,7 @@ extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err,
                                            void* stream) {
   clear_error();
   int st = check_conv_dims("conv_wgrad_update", N, H, W, C, K, R, S, stride, pad);
+  if (st == NITI_OK) st = check_flags("conv_wgrad_update", flags, NITI_EPI_F32_ROUNDTRIP | NITI_CONV_SHIFT_HINT);
   if (st != NITI_OK) return st;
   if (act == nullptr || err == nullptr || w == nullptr || sync == nullptr)
     return fail(NITI_ERR_INVALID_ARG, "conv_wgrad_update: null pointer");
@@ -426,6 +439,7 @@ extern "C" int niti_gemm_i8(int trans_a, int trans_b, const int8_t* a, const int
                             unsigned flags, uint32_t* absmax, void* workspace, size_t workspace_bytes, void* stream) {
   clear_error();
   if (m <= 0 || n <= 0 || k <= 0) return fail(NITI_ERR_INVALID_ARG, "gemm: non-positive extent (m=%d n=%d k=%d)", m, n, k);
+  if (check_flags("gemm", flags, NITI_EPI_F32_ROUNDTRIP) != NITI_OK) return NITI_ERR_INVALID_ARG;
   if (a == nullptr || b == nullptr || c == nullptr) return fail(NITI_ERR_INVALID_ARG, "gemm: null pointer");
   if (!aligned16(c)) return fail(NITI_ERR_INVALID_ARG, "gemm: output must be 16-byte aligned");
   const size_t need = niti_gemm_i8_workspace(trans_a, trans_b, m, n, k);

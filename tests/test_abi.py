@@ -119,6 +119,27 @@ def test_workspace_sizes(lib):
     assert lib.niti_conv2d_i8_wgrad_workspace(0, 7, 9, 40, 24, 3, 3, 1) == 0
 
 
+def test_unknown_flag_bits_are_refused(lib):
+    """Flag words are checked before any pointer is touched: bits the entry point does not define are an error."""
+    conv = (2, 8, 8, 16, 16, 3, 3, 1, 1)      # N H W C K R S stride pad
+    bad = 0x100
+    calls = {
+        "niti_conv2d_i8_fprop": (None, None, None) + conv + (bad, None, None, 0, None),
+        "niti_conv2d_i8_dgrad": (None, None, None) + conv + (bad, None, None, 0, None),
+        "niti_conv2d_i8_wgrad": (None, None, None) + conv + (bad, None, None, 0, None),
+        "niti_conv2d_i8_fprop_requant": (None, None, None) + conv + (bad, 7, 0, 0, 0, 0, None, 0, None, None, None, None, None, 0, None),
+        "niti_conv2d_i8_wgrad_update": (None, None, None, 16) + conv + (bad, 5, 0, 0, 0, None, 0, None, None, None, None, None, None, None,
+                                                                      None, 0, None),
+        "niti_gemm_i8": (0, 1, None, None, None, 4, 4, 16, bad, None, None, 0, None),
+    }
+    for name, args in calls.items():
+        assert getattr(lib, name)(*args) == 1, name                       # NITI_ERR_INVALID_ARG
+        assert b"flags=0x100" in lib.niti_last_error(), (name, lib.niti_last_error())
+    # a forward-copy flag is a data-gradient flag only
+    assert lib.niti_conv2d_i8_fprop(None, None, None, *conv, 4, None, None, 0, None) == 1
+    assert b"flags=0x4" in lib.niti_last_error()
+
+
 def test_package_fails_loudly_without_the_library(tmp_path):
     """The product has no CPU fallback: importing the ops with the shared object missing raises."""
     code = (
