@@ -375,7 +375,13 @@ class TiConv2d(UpdateWeight):
         self.act, self.act_in_exp = input
         dev = self.act.device
         self.act16 = _pad_channels16(self.act).contiguous()      # channel-padded copy, reused by the weight gradient
-        w16 = _pad_channels16(self.weight).contiguous()
+        # With an up-to-date kernel-ready filter copy the padded weights are passed for their shape only: the first
+        # layer then reuses the padded tensor the copy was made from instead of padding the weights again every step.
+        key = (self.weight.data_ptr(), self.weight._version, tuple(self.act16.shape))
+        shape_only = (self.weight.shape[3] % 16 != 0 and getattr(self, "_wprep_key", None) == key
+                      and getattr(self, "_wprep", None) is not None and getattr(self, "_w16_kept", None) is not None)
+        w16 = self._w16_kept if shape_only else _pad_channels16(self.weight).contiguous()
+        self._w16_kept = w16 if self.weight.shape[3] % 16 != 0 else None
         exp_a, exp_b = _exp_tensor(self.act_in_exp, dev), self._wexp()
         pooled = None
         N, H, W, _ = self.act16.shape
@@ -388,6 +394,8 @@ class TiConv2d(UpdateWeight):
             if pooled is not None:      # the pooling layer finds its result ready when it sees this tensor
                 self.pool_after.preset = (fused[0], pooled)
             return fused[0], fused[2]
+        if shape_only:
+            w16 = self._w16_kept = _pad_channels16(self.weight).contiguous()
         am = ops.new_scalar_u32(dev)
         acc = ops.conv2d_fprop(self.act16, w16, self.stride, self.padding, f32_epilogue=F32_EPILOGUE, absmax=am)
         act_out, _, exp_out = _requant(acc, BITWIDTH, ACT_ROUND_METHOD, am, rand, relu=self.fuse_relu,
