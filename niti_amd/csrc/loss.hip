@@ -3,7 +3,9 @@
 // The reference evaluates a base-2 soft-max of the int8 logits in float32 tensor operations, truncates to
 // integers twice on the way and rounds the result to int8 with StoShift(.., 4).  Every float32 operation
 // of that sequence is kept, in the same order and with the same intermediate types (int64 sums of truncated
-// values, float32 products and quotients), so that the result only depends on the device's powf.
+// values, float32 products and quotients).  The one operation whose result differs between math libraries,
+// 2 ** s, is evaluated by a fixed sequence of IEEE double operations (exp2_contract below) that a host can
+// repeat bit for bit, so the whole gradient is reproducible across devices.
 #include "common.h"
 #include "requant_math.h"
 
@@ -26,6 +28,27 @@ struct LossArgs {
 __device__ inline float scaled_logit(int v, float p2, bool up) {
   const float s = static_cast<float>(static_cast<long long>(v) * 47274) / 32768.0f;
   return up ? s * p2 : s / p2;
+}
+
+// 2^s for s >= 0: n = floor(s), x = (s - n) ln2, Horner's rule over 1/k! (k = 18 .. 0) in doubles with one rounded
+// product and one rounded sum per step (no fused multiply-add), result = float(p 2^n).  Truncation error < 2^-60, so
+// this is the correctly rounded float32 power except within ~2^-52 (relative) of a rounding boundary.
+__device__ inline float exp2_contract(float s) {
+  constexpr double c[19] = {
+      0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,  0x1.5555555555555p-3,  0x1.5555555555555p-5,
+      0x1.1111111111111p-7,  0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16, 0x1.71de3a556c734p-19,
+      0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26, 0x1.1eed8eff8d898p-29, 0x1.6124613a86d09p-33, 0x1.93974a8c07c9dp-37,
+      0x1.ae7f3e733b81fp-41, 0x1.ae7f3e733b81fp-45, 0x1.952c77030ad4ap-49, 0x1.6827863b97d97p-53};
+  const double d = static_cast<double>(s);
+  const double n = floor(d);
+  const double x = (d - n) * 0x1.62e42fefa39efp-1;   // contraction is off for this file (pragma above)
+  double p = c[18];
+#pragma unroll
+  for (int k = 17; k >= 0; --k) {
+    p = p * x;
+    p = p + c[k];
+  }
+  return static_cast<float>(ldexp(p, static_cast<int>(n)));
 }
 
 __device__ inline long long wave_sum_i64(long long v) {
@@ -67,7 +90,7 @@ __global__ __launch_bounds__(256) void loss_grad_kernel(const LossArgs a) {
   auto numer = [&](int j) -> float {   // out_grad before the normalisation, as float32
     if (!big) return static_cast<float>(small_term(v[j]));
     const float s = fmaxf(scaled_logit(v[j], p2, up) - off, 0.0f);
-    return powf(2.0f, s) - 1.0f;
+    return exp2_contract(s) - 1.0f;
   };
   long long sum = 0;   // out_grad.sum(1, dtype=int64): truncation of every term (ti_loss.py:31)
   for (int j = lane; j < a.classes; j += 64) sum += big ? static_cast<long long>(numer(j)) : small_term(v[j]);

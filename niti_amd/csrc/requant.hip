@@ -139,14 +139,18 @@ __global__ __launch_bounds__(256) void absmax_f32_kernel(const float* __restrict
 }
 
 // bw = ceil(log2 r); y = int8(clamp(round_half_even(x * 2^(bits - bw)), -128, 127)), float NCHW -> int8 NHWC with the
-// channels zero-padded to cpad; exp_out = bw - bits.  The float operations are the reference's, one by one.
+// channels zero-padded to cpad; exp_out = bw - bits.  The product and the rounding are the reference's float32 operations.
 __global__ __launch_bounds__(256) void quantize_f32_i8_kernel(const float* __restrict__ x, int8_t* __restrict__ y, int64_t pixels,
                                                               int C, int HW, int cpad, const uint32_t* __restrict__ absmax_bits,
                                                               int32_t* exp_out, int bits) {
   const float r = __uint_as_float(*absmax_bits);
-  const float bw = ceilf(log2f(r));
-  const float scale = powf(2.0f, static_cast<float>(bits) - bw);
-  if (blockIdx.x == 0 && threadIdx.x == 0 && exp_out != nullptr) *exp_out = r > 0.0f ? static_cast<int>(bw) - bits : 0;
+  // ceil(log2 r) from the exponent and mantissa of r = m 2^e, 0.5 <= m < 1 (exact; a library log2f rounds k + log2(1 + d)
+  // back to k for the first float32 values above 2^k, k >= 4, and differs between platforms there)
+  int fe = 0;
+  const float fm = frexpf(r, &fe);
+  const int bw = fm == 0.5f ? fe - 1 : fe;
+  const float scale = ldexpf(1.0f, bits - bw);
+  if (blockIdx.x == 0 && threadIdx.x == 0 && exp_out != nullptr) *exp_out = r > 0.0f ? bw - bits : 0;
   const int64_t stride = static_cast<int64_t>(gridDim.x) * blockDim.x;
   for (int64_t p = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x; p < pixels; p += stride) {
     const int64_t n = p / HW, hw = p - n * HW;

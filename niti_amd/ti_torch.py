@@ -259,10 +259,18 @@ def conv2d_weight_int8(input, weight_size, grad_output, stride=1, padding=0, dil
 # ------------------------------------------------------------------------------------------
 # quantisers / initialisers (ti_torch.py:77-99, 334-364)
 # ------------------------------------------------------------------------------------------
+def _ceil_log2(r):
+    """``torch.ceil(torch.log2(r))`` of ti_torch.py:336,348 as exact arithmetic on the float's exponent and mantissa
+    (r = m * 2^e, 0.5 <= m < 1: e - 1 for a power of two, e otherwise), so that every device gives the same integer;
+    a float32 log2 rounds k + log2(1 + d) back to k for the first values above 2^k, k >= 4.  0-d float tensor."""
+    m, e = torch.frexp(r.float())
+    return torch.where(m == 0.5, e - 1, e).to(torch.float32)
+
+
 def weight_quant(input):
     """ti_torch.py:334-339.  Returns (int8 weights on the GPU, exponent as a 0-d float tensor)."""
     input_range = torch.max(torch.abs(input))
-    input_bitwidth = torch.ceil(torch.log2(input_range))
+    input_bitwidth = _ceil_log2(input_range)
     act_exp = input_bitwidth - 7
     round_val = torch.round(input / input_range * (2 ** 7 - 1)).type(torch.int8).to(GPU)
     return round_val, act_exp
@@ -300,7 +308,7 @@ def TiFloatToInt8(input):
     HIP graph (train.StepGraph quantises eagerly and captures forward_int8 + backward)."""
     input = input.to(GPU)
     input_range = torch.max(torch.abs(input))
-    input_bitwidth = torch.ceil(torch.log2(input_range))
+    input_bitwidth = _ceil_log2(input_range)
     act_exp = input_bitwidth - BITWIDTH
     norm_val = input * (2 ** (BITWIDTH - input_bitwidth))
     round_val = torch.round(norm_val)

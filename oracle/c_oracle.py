@@ -31,6 +31,8 @@ def lib():
         _lib.nito_sto_shift1.restype = C.c_int8
         _lib.nito_psto_shift1.restype = C.c_int8
         _lib.nito_absmax.restype = C.c_uint32
+        _lib.nito_exp2_contract.restype = C.c_float
+        _lib.nito_exp2_contract.argtypes = [C.c_float]
     return _lib
 
 
@@ -160,3 +162,30 @@ def maxpool_bwd(y, dy, x, ks=2, stride=2, pad=0, ties="first"):
     dx = torch.empty_like(x)
     lib().nito_maxpool_bwd(_p(y), _p(dy), _p(x), _p(dx), N, H, W, Cc, ks, stride, pad, int(ties == "all"))
     return dx
+
+
+def exp2_contract(s: float) -> float:
+    return float(lib().nito_exp2_contract(float(s)))
+
+
+def ti_loss_pre_round(out_val, out_exp, target):
+    out_val = out_val.contiguous()
+    target = target.to(torch.int64).contiguous()
+    n, classes = out_val.shape
+    pre = torch.empty((n, classes), dtype=torch.int32)
+    lib().nito_ti_loss_pre_round(_p(out_val), n, classes, int(out_exp), _p(target), _p(pre))
+    return pre
+
+
+def float_to_int8(x, bits=7):
+    x = x.to(torch.float32).contiguous()
+    y = torch.empty(x.shape, dtype=torch.int8)
+    e = lib().nito_float_to_int8(_p(x), _p(y), C.c_int64(x.numel()), int(bits))
+    return y, int(e)
+
+
+def weight_quant(w):
+    w = w.to(torch.float32).contiguous()
+    y = torch.empty(w.shape, dtype=torch.int8)
+    e = lib().nito_weight_quant(_p(w), _p(y), C.c_int64(w.numel()))
+    return y, int(e)

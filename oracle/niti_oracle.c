@@ -314,3 +314,112 @@ void nito_maxpool_bwd(const int8_t* y, const int8_t* dy, const int8_t* x, int8_t
   for (size_t i = 0; i < (size_t)N * H * W * C; ++i) dx[i] = (int8_t)acc[i];
   free(acc);
 }
+
+/* ---------------------------------------------------------------- integer cross-entropy gradient (ti_loss.py:5-36) */
+/* 2^s of ti_loss.py:24 as a fixed sequence of IEEE double operations (built with -ffp-contract=off): n = floor(s),
+ * x = (s - n) ln2, Horner's rule over 1/k! (k = 18 .. 0) with one rounded product and one rounded sum per step,
+ * result = (float)(p 2^n).  The HIP kernel runs the same sequence, so host and device agree bit for bit. */
+static const double k_exp2_coef[19] = {
+    0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,  0x1.5555555555555p-3,  0x1.5555555555555p-5,
+    0x1.1111111111111p-7,  0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16, 0x1.71de3a556c734p-19,
+    0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26, 0x1.1eed8eff8d898p-29, 0x1.6124613a86d09p-33, 0x1.93974a8c07c9dp-37,
+    0x1.ae7f3e733b81fp-41, 0x1.ae7f3e733b81fp-45, 0x1.952c77030ad4ap-49, 0x1.6827863b97d97p-53};
+
+float nito_exp2_contract(float s) {
+  const double d = (double)s;
+  const double n = floor(d);
+  const double x = (d - n) * 0x1.62e42fefa39efp-1;
+  volatile double p = k_exp2_coef[18];
+  for (int k = 17; k >= 0; --k) {
+    p = p * x;
+    p = p + k_exp2_coef[k];
+  }
+  return (float)ldexp(p, (int)n);
+}
+
+/* everything before the final StoShift: pre[n][classes] is the int32 tensor of ti_loss.py:35.  Every float
+ * operation is one float32 operation of the reference's tensor sequence, in its order. */
+void nito_ti_loss_pre_round(const int8_t* out, int n, int classes, int out_exp, const int64_t* target, int32_t* pre) {
+  for (int i = 0; i < n; ++i) {
+    const int8_t* v = out + (size_t)i * classes;
+    int32_t* o = pre + (size_t)i * classes;
+    volatile float num[1024];   /* numerators as float32 (volatile: no excess precision, no contraction) */
+    int64_t out_sum = 0;
+    if (classes > 1024) return;
+    if (out_exp > -7) {
+      const float p2 = ldexpf(1.0f, out_exp >= 0 ? out_exp : -out_exp);
+      float mx = -INFINITY;
+      for (int j = 0; j < classes; ++j) {
+        volatile float s = (float)((int64_t)v[j] * 47274) / 32768.0f;     /* :14 */
+        s = out_exp >= 0 ? s * p2 : s / p2;                               /* :15-18 */
+        num[j] = s;
+        if (s > mx) mx = s;
+      }
+      volatile float offset = mx - 10.0f;                                  /* :20-21 */
+      for (int j = 0; j < classes; ++j) {
+        volatile float s = num[j] - offset;                                /* :22 */
+        if (s < 0.0f) s = 0.0f;                                            /* :23 */
+        volatile float pw = nito_exp2_contract(s);
+        num[j] = pw - 1.0f;                                                /* :24 */
+        out_sum += (int64_t)num[j];                                        /* :31 */
+      }
+    } else {
+      for (int j = 0; j < classes; ++j) {
+        const int64_t x = v[j];
+        const int64_t t = ((int64_t)1 << (1 - 2 * out_exp)) + x * ((int64_t)1 << (1 - out_exp)) + x * x;   /* :28-29 */
+        out_sum += t;
+        num[j] = (float)t;   /* :33 multiplies in int64 first; float(2048 t) = 2048 float(t), a power of two */
+      }
+    }
+    const float fsum = (float)out_sum;
+    int64_t tsum = 0;
+    for (int j = 0; j < classes; ++j) {
+      volatile float prod = num[j] * 2048.0f;
+      num[j] = prod / fsum;                                                /* :33 */
+      tsum += (int64_t)num[j];                                             /* :34 */
+    }
+    for (int j = 0; j < classes; ++j) {
+      volatile float g = num[j];
+      if (j == target[i]) g = g - (float)tsum;                             /* :34 */
+      o[j] = (int32_t)g;                                                   /* :35 */
+    }
+  }
+}
+
+/* ---------------------------------------------------------------- float -> int8 quantisers */
+/* ceil(log2 r) of a positive float from its exponent and mantissa (the exact value of ti_torch.py:336,348) */
+int nito_ceil_log2_f32(float r) {
+  int e;
+  const float m = frexpf(r, &e);   /* r = m 2^e, 0.5 <= m < 1 */
+  return m == 0.5f ? e - 1 : e;
+}
+
+/* TiFloatToInt8 (ti_torch.py:341-356) on a flat array; returns the exponent bw - bits (0 for an all-zero input) */
+int nito_float_to_int8(const float* x, int8_t* y, int64_t n, int bits) {
+  float r = 0.0f;
+  for (int64_t i = 0; i < n; ++i) r = fabsf(x[i]) > r ? fabsf(x[i]) : r;
+  if (r == 0.0f) {
+    memset(y, 0, (size_t)n);
+    return 0;
+  }
+  const int bw = nito_ceil_log2_f32(r);
+  const float scale = ldexpf(1.0f, bits - bw);
+  for (int64_t i = 0; i < n; ++i) {
+    float q = nearbyintf(x[i] * scale);   /* round half to even in the default rounding mode */
+    q = q < -128.0f ? -128.0f : (q > 127.0f ? 127.0f : q);
+    y[i] = (int8_t)q;
+  }
+  return bw - bits;
+}
+
+/* weight_quant (ti_torch.py:334-339); returns the exponent */
+int nito_weight_quant(const float* w, int8_t* y, int64_t n) {
+  float r = 0.0f;
+  for (int64_t i = 0; i < n; ++i) r = fabsf(w[i]) > r ? fabsf(w[i]) : r;
+  for (int64_t i = 0; i < n; ++i) {
+    volatile float q = w[i] / r;
+    q = q * 127.0f;
+    y[i] = (int8_t)nearbyintf(q);
+  }
+  return nito_ceil_log2_f32(r) - 7;
+}

@@ -375,9 +375,38 @@ def maxpool_bwd(y, dy, x, kernel_size=2, stride=2, padding=0, ties="first"):
 # --------------------------------------------------------------------------------------
 # integer cross-entropy gradient
 # --------------------------------------------------------------------------------------
-def ti_loss_pre_round(out_val: torch.Tensor, out_exp: int, target: torch.Tensor) -> torch.Tensor:
+# 1/k! for k = 0..18 as the nearest doubles (hex literals: the same bits in niti_oracle.c and in the HIP kernel)
+EXP2_COEF = [float.fromhex(h) for h in (
+    "0x1.0000000000000p+0", "0x1.0000000000000p+0", "0x1.0000000000000p-1", "0x1.5555555555555p-3",
+    "0x1.5555555555555p-5", "0x1.1111111111111p-7", "0x1.6c16c16c16c17p-10", "0x1.a01a01a01a01ap-13",
+    "0x1.a01a01a01a01ap-16", "0x1.71de3a556c734p-19", "0x1.27e4fb7789f5cp-22", "0x1.ae64567f544e4p-26",
+    "0x1.1eed8eff8d898p-29", "0x1.6124613a86d09p-33", "0x1.93974a8c07c9dp-37", "0x1.ae7f3e733b81fp-41",
+    "0x1.ae7f3e733b81fp-45", "0x1.952c77030ad4ap-49", "0x1.6827863b97d97p-53")]
+EXP2_LN2 = float.fromhex("0x1.62e42fefa39efp-1")
+
+
+def exp2_contract(s: torch.Tensor) -> torch.Tensor:
+    """``2 ** s`` of ti_loss.py:24 for a float32 tensor, as a fixed sequence of IEEE double operations, so
+    that host and device agree bit for bit (a library pow differs by an ulp between platforms, which can
+    flip the truncations that follow):  n = floor(s), x = (s - n) * ln2, p = sum x^k / k! by Horner's rule
+    with a separately rounded product and sum per step (no fused multiply-add), result = float32(p * 2^n).
+    The truncation error is below 2^-60, so the result is the correctly rounded float32 power except when
+    the true value lies within about 2^-52 (relative) of a rounding boundary."""
+    d = s.to(torch.float64)
+    n = torch.floor(d)
+    x = (d - n) * EXP2_LN2
+    p = torch.full_like(x, EXP2_COEF[-1])
+    for c in reversed(EXP2_COEF[:-1]):
+        p = p * x
+        p = p + c
+    return torch.ldexp(p, n.to(torch.int32)).to(torch.float32)
+
+
+def ti_loss_pre_round(out_val: torch.Tensor, out_exp: int, target: torch.Tensor, pow2=exp2_contract) -> torch.Tensor:
     """ti_loss.py:6-34: everything before the final StoShift; returns the int32 tensor that
-    StoShift(.., 4) consumes.  fp32 arithmetic exactly as the reference's op sequence."""
+    StoShift(.., 4) consumes.  fp32 arithmetic exactly as the reference's op sequence; ``2 ** s`` of
+    line 24 through ``pow2`` (default: the deterministic statement above; ``lambda s: 2 ** s`` gives the
+    platform's own float pow)."""
     s = out_val.to(torch.int64)
     out_exp = int(out_exp)
     if out_exp > -7:
@@ -390,7 +419,7 @@ def ti_loss_pre_round(out_val: torch.Tensor, out_exp: int, target: torch.Tensor)
         offset = out_max - 10
         s = s - offset.view(-1, 1)
         s = torch.max(s, torch.tensor(0, dtype=torch.int8).to(torch.int64))
-        out_grad = 2 ** s - 1
+        out_grad = pow2(s) - 1
     else:
         e = torch.tensor(out_exp, dtype=torch.int64)
         out_grad = 2 ** (1 - 2 * e) + s * 2 ** (1 - e) + s * s
@@ -403,3 +432,52 @@ def ti_loss_pre_round(out_val: torch.Tensor, out_exp: int, target: torch.Tensor)
 def ti_loss(out_val, out_exp, target, rand, div_mode=FLOOR):
     """ti_loss.py:35-36: int8 error = StoShift(pre_round, 4), exponent 0."""
     return StoShift(ti_loss_pre_round(out_val, out_exp, target), 4, rand, div_mode), 0
+
+
+# --------------------------------------------------------------------------------------
+# float -> int8 quantisers
+# --------------------------------------------------------------------------------------
+def ceil_log2_f32(r: float) -> int:
+    """ceil(log2(r)) of a positive float32 as exact arithmetic on its exponent and mantissa (what
+    ``torch.ceil(torch.log2(r))`` of ti_torch.py:336,348 means mathematically): r = m * 2^e with
+    0.5 <= m < 1 gives e - 1 for m == 0.5 (a power of two) and e otherwise."""
+    m, e = math.frexp(float(np.float32(r)))
+    return e - 1 if m == 0.5 else e
+
+
+def float_to_int8(x: torch.Tensor, bits: int = BITWIDTH, log2_mode: str = "exact") -> Tuple[torch.Tensor, int]:
+    """TiFloatToInt8, ti_torch.py:341-356: r = max|x|, bw = ceil(log2 r), exponent bw - bits,
+    values clamp(round_half_even(x * 2^(bits - bw)), -128, 127) as int8 (same shape as x).
+    log2_mode "exact": ceil_log2_f32 (the contract of the HIP path); "f32": the reference's literal
+    float32 ``ceil(log2(r))`` on this host.  The two differ only for r in the first few float32 values
+    above a power of two >= 16, where float32(k + log2(1 + d)) rounds back to k.
+    An all-zero tensor gives zeros and exponent 0 (the reference's sequence yields NaN there)."""
+    x = x.to(torch.float32)
+    r = torch.max(torch.abs(x))
+    if float(r) == 0.0:
+        return torch.zeros(x.shape, dtype=torch.int8), 0
+    if log2_mode == "exact":
+        bw = ceil_log2_f32(float(r))
+    elif log2_mode == "f32":
+        bw = int(torch.ceil(torch.log2(r)))
+    else:
+        raise ValueError(log2_mode)
+    norm = x * torch.tensor(2.0 ** (bits - bw), dtype=torch.float32)
+    q = torch.clamp(torch.round(norm), -128, 127).to(torch.int8)
+    return q, bw - bits
+
+
+def quantize_input_nhwc(x_nchw: torch.Tensor, bits: int = BITWIDTH) -> Tuple[torch.Tensor, int]:
+    """TiNet.forward, ti_net.py:18-19: TiFloatToInt8 of the float NCHW batch, then permute(0,2,3,1).contiguous()."""
+    q, e = float_to_int8(x_nchw, bits)
+    return q.permute(0, 2, 3, 1).contiguous(), e
+
+
+def weight_quant(w: torch.Tensor, log2_mode: str = "exact") -> Tuple[torch.Tensor, int]:
+    """weight_quant, ti_torch.py:334-339: int8 = round_half_even(w / max|w| * 127) (float32 quotient, then
+    float32 product), exponent ceil(log2(max|w|)) - 7."""
+    w = w.to(torch.float32)
+    r = torch.max(torch.abs(w))
+    bw = ceil_log2_f32(float(r)) if log2_mode == "exact" else int(torch.ceil(torch.log2(r)))
+    q = torch.round(w / r * (2 ** 7 - 1)).to(torch.int8)
+    return q, bw - 7

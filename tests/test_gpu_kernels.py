@@ -748,23 +748,43 @@ def test_maxpool(dev, case):
 
 
 def test_quantize_input(dev):
-    """The input quantiser as two launches against the reference's tensor operations (same device functions, so the
-    results are equal), including ranges at and next to a power of two, where ceil(log2 r) jumps."""
+    """The input quantiser (two launches: range, then quantise + NHWC + channel padding) against the CPU oracle's
+    TiFloatToInt8 + permute, including ranges at and next to a power of two (where ceil(log2 r) jumps), the hand-derived
+    known answers, round-half-even ties and both clamps; the tensor-operation form of the package gives the same."""
+    import json
+    import os
     from niti_amd import ops, ti_torch
+    from oracle import niti_oracle as po
     _say("quantize_input")
     g = torch.Generator().manual_seed(77)
     for shape, top in (((128, 3, 32, 32), None), ((5, 3, 7, 9), 4.0), ((2, 3, 8, 8), 4.000001), ((2, 3, 8, 8), 3.9999998),
-                       ((3, 17, 4, 4), 0.3), ((1, 1, 1, 1), 100.0)):
+                       ((3, 17, 4, 4), 0.3), ((1, 1, 1, 1), 100.0), ((2, 3, 8, 8), 16.000002), ((2, 3, 4, 4), 1e-3),
+                       ((2, 3, 4, 4), 3e4)):
         x = torch.randn(shape, generator=g)
         if top is not None:
             x = x / x.abs().max() * 0.9 * top
             x.view(-1)[min(3, x.numel() - 1)] = -top
+        ref, ref_exp = po.quantize_input_nhwc(x)
         xd = x.to(dev)
-        ref, ref_exp = ti_torch.TiFloatToInt8(xd)
         y, e = ops.quantize_input(xd)
         C = shape[1]
-        assert y.shape[3] == max(16, (C + 3) // 4 * 4) and int(e.cpu()) == int(ref_exp.cpu())
-        assert torch.equal(y[..., :C], ref.permute(0, 2, 3, 1)) and int(y[..., C:].abs().max()) == 0
+        assert y.shape[3] == max(16, (C + 3) // 4 * 4) and int(e.cpu()) == ref_exp, (shape, top)
+        assert torch.equal(y[..., :C].cpu(), ref) and int(y[..., C:].abs().max()) == 0, (shape, top)
+        t, te = ti_torch.TiFloatToInt8(xd)
+        assert int(te.cpu()) == ref_exp and torch.equal(t.permute(0, 2, 3, 1).cpu(), ref), (shape, top)
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "quantize_kat.json")) as f:
+        kat = json.load(f)
+    for c in kat["float_to_int8"]:
+        x = torch.tensor(c["x"], dtype=torch.float32).reshape(1, -1, 1, 1)     # the values as channels of one pixel
+        y, e = ops.quantize_input(x.to(dev))
+        assert y[0, 0, 0, :x.shape[1]].cpu().tolist() == c["q"] and int(e.cpu()) == c["exp"], c["name"]
+    for c in kat["weight_quant"]:
+        q, e = ti_torch.weight_quant(torch.tensor(c["w"], dtype=torch.float32))
+        assert q.cpu().tolist() == c["q"] and int(e.cpu()) == c["exp"], c["name"]
+    w = torch.randn((64, 3, 3, 32), generator=g) * 0.07
+    q, e = ti_torch.weight_quant(w.to(dev))
+    qr, er = po.weight_quant(w)
+    assert torch.equal(q.cpu(), qr) and int(e.cpu()) == er
     y, e = ops.quantize_input(torch.zeros((2, 3, 4, 4), device=dev))
     assert int(y.abs().max()) == 0 and int(e.cpu()) == 0
 
