@@ -166,6 +166,26 @@ int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8
                                  size_t workspace_bytes, void* stream);
 
 /*
+ * niti_conv2d_i8_fprop_requant for callers that cannot allocate device memory or hand in scratch memory: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * arithmetic and the same results as niti_conv2d_i8_fprop_requant; the sync words and the kernel-ready filter copy live
+ * in a device array inside the library (niti_static_scratch_bytes() bytes per GPU the library runs on, about 4.1 MiB,
+ * held until the process ends), which the call clears with a small kernel before use.  It calls no hipMalloc / hipFree
+ * and nothing that allocates.
+ * Limits: a launch of at most 4096 workgroups (as niti_conv2d_i8_fprop_requant) and a filter copy
+ * (niti_conv2d_i8_filter_workspace(.., 0)) of at most 4 MiB unless NITI_CONV_FILTER_PREPARED is passed (then `w` is
+ * the caller's prepared copy); beyond them the call returns NITI_ERR_UNSUPPORTED and launches nothing.
+ * range_out (may be NULL): two words, [0] = max |sum| over the tensor, [1] != 0 if the wait for the other workgroups
+ * ran into its time limit (what words 0 and 1 of `sync` hold after niti_conv2d_i8_fprop_requant).
+ * All calls on one GPU share that GPU's array: calls that overlap on one GPU (two streams, two host threads) race.
+ */
+size_t niti_static_scratch_bytes(void);
+int niti_conv2d_i8_fprop_requant_static(const int8_t* x, const int8_t* w, int8_t* y8, int N, int H, int W, int C, int K, int R,
+                                        int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
+                                        int bw_mode, unsigned rq_flags, int32_t* shift_out, const int32_t* exp_a,
+                                        const int32_t* exp_b, int32_t* exp_out, uint32_t* range_out, void* stream);
+
+/*
  * Weight gradient, replaces the reference's fprop-on-transposed-operands rewrite
  * (ti_torch.py:430-432) and, for the first layer, conv2d_weight_int8 -> group_conv
  * (ti_torch.py:194-233):

@@ -331,6 +331,79 @@ extern "C" int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, 
                       bw_mode, rq_flags, relu_mask, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes, stream);
 }
 
+// ---- forward convolution + requantisation for callers that can neither allocate nor hand in scratch memory --------
+// The sync words and the kernel-ready filter copy of niti_conv2d_i8_fprop_requant live in a device array of this
+// library instead of caller memory.  Each GPU holds its own copy of the array at its own address, looked up once per
+// device; host code only ever uses that address, never the array's name.
+namespace {
+constexpr size_t kStaticSyncWords = 16 + 4096 * static_cast<size_t>(NITI_SLOT_STRIDE);   // = conv3x3_halo_sync_words(4096)
+constexpr size_t kStaticSyncBytes = (kStaticSyncWords * 4 + 255) / 256 * 256;
+constexpr size_t kStaticFilterBytes = NITI_STATIC_FILTER_BYTES;
+static __device__ __align__(256) unsigned char scratch[kStaticSyncBytes + kStaticFilterBytes];
+unsigned char* g_scratch_ptr[kDeviceSlots] = {};
+int g_scratch_dev[kDeviceSlots];
+
+__global__ void copy_words_kernel(const uint32_t* __restrict__ src, uint32_t* __restrict__ dst, int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[i] = src[i];
+}
+
+// address of this device's copy of `scratch` (nullptr + error message on failure)
+unsigned char* static_scratch() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    fail(NITI_ERR_LAUNCH, "static scratch: no current device");
+    return nullptr;
+  }
+  const int slot = device_slot();
+  if (g_scratch_ptr[slot] == nullptr || g_scratch_dev[slot] != dev) {
+    void* p = nullptr;
+    const hipError_t e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      fail(NITI_ERR_LAUNCH, "static scratch: hipGetSymbolAddress: %s", hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[slot] = static_cast<unsigned char*>(p);
+    g_scratch_dev[slot] = dev;
+  }
+  return g_scratch_ptr[slot];
+}
+}  // namespace
+
+extern "C" size_t niti_static_scratch_bytes(void) { return kStaticSyncBytes + kStaticFilterBytes; }
+
+extern "C" int niti_conv2d_i8_fprop_requant_static(const int8_t* x, const int8_t* w, int8_t* y8, int N, int H, int W, int C, int K,
+                                                   int R, int S, int stride, int pad, unsigned flags, int target_bits,
+                                                   int method, int div_mode, int bw_mode, unsigned rq_flags, int32_t* shift_out,
+                                                   const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                                   uint32_t* range_out, void* stream) {
+  clear_error();
+  const char* who = "conv_fprop_requant_static";
+  int st = check_conv_dims(who, N, H, W, C, K, R, S, stride, pad);
+  if (st != NITI_OK) return st;
+  const int nb = fused_blocks(N, H, W, C, K, R, S, stride, pad, 0);
+  if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "%s: shape not covered by the single-launch path", who);
+  const size_t words = conv3x3_halo_sync_words(nb);
+  if (words > kStaticSyncWords)
+    return fail(NITI_ERR_UNSUPPORTED, "%s: %d workgroups need %zu sync words, the static scratch holds %zu", who, nb, words, kStaticSyncWords);
+  const size_t fbytes = (flags & NITI_CONV_FILTER_PREPARED) ? 0 : conv3x3_halo_filter_bytes(C, K);
+  if (fbytes > kStaticFilterBytes)
+    return fail(NITI_ERR_UNSUPPORTED, "%s: the filter copy needs %zu bytes, the static scratch holds %zu (pass a prepared filter)", who,
+                fbytes, kStaticFilterBytes);
+  unsigned char* const base = static_scratch();
+  if (base == nullptr) return NITI_ERR_LAUNCH;
+  uint32_t* const sync = reinterpret_cast<uint32_t*>(base);
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  // the array keeps the previous call's slots: clear them with a kernel (a memset node misbehaves in replayed graphs)
+  st = launch_fill_u32(sync, static_cast<int64_t>(words), 0u, s);
+  if (st != NITI_OK) return st;
+  st = conv_requant(who, 0, x, w, y8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method, div_mode, bw_mode, rq_flags, nullptr,
+                    sync, words, shift_out, exp_a, exp_b, exp_out, base + kStaticSyncBytes, kStaticFilterBytes, stream);
+  if (st != NITI_OK || range_out == nullptr) return st;
+  hipLaunchKernelGGL(copy_words_kernel, dim3(1), dim3(64), 0, s, sync, range_out, 2);
+  return check_launch(who);
+}
+
 extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || pad < 0) return 0;
   const int P = H + 2 * pad - R + 1, Q = W + 2 * pad - S + 1;

@@ -9,6 +9,10 @@
 #ifndef NITI_SLOT_STRIDE
 #define NITI_SLOT_STRIDE 4
 #endif
+// bytes of the kernel-ready filter copy that niti_conv2d_i8_fprop_requant_static can hold in the library's own array
+#ifndef NITI_STATIC_FILTER_BYTES
+#define NITI_STATIC_FILTER_BYTES (4u << 20)
+#endif
 
 namespace niti {
 

@@ -178,6 +178,39 @@ def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_b
                          prepared_filter, shift_hint=shift_hint, pool_out=pool_out)
 
 
+def conv2d_fprop_requant_static(x, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
+                                bw_mode="int", relu=False, y=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
+                                prepared_filter=None, range_out=None):
+    """conv2d_fprop_requant through the entry point that takes no scratch memory from the caller (the library keeps its
+    sync words and filter copy in a device array of its own): only the tensors given here are touched, and when ``y``,
+    ``shift_out`` are passed in nothing is allocated at all.  ``range_out``: int32[2], receives max|sum| and the
+    timed-out flag.  Calls on one GPU must not overlap.  Returns (y, shift_out)."""
+    _chk_dev(x, w, y, shift_out, exp_a, exp_b, exp_out, prepared_filter, range_out)
+    if x.dtype != torch.int8 or w.dtype != torch.int8:
+        raise RuntimeError("conv2d_fprop_requant_static: int8 tensors expected")
+    N, H, W, C = x.shape
+    K, R, S, C2 = w.shape
+    if C2 != C:
+        raise RuntimeError("conv2d_fprop_requant_static: channel mismatch %d vs %d" % (C, C2))
+    P = (H + 2 * padding - R) // stride + 1
+    Q = (W + 2 * padding - S) // stride + 1
+    if y is None:
+        y = torch.empty((N, P, Q, K), dtype=torch.int8, device=x.device)
+    elif y.dtype != torch.int8 or tuple(y.shape) != (N, P, Q, K) or not y.is_contiguous():
+        raise RuntimeError("conv2d_fprop_requant_static: y must be a contiguous int8 [N,P,Q,K] tensor")
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=x.device)
+    if range_out is not None and (range_out.dtype != torch.int32 or range_out.numel() < 2):
+        raise RuntimeError("conv2d_fprop_requant_static: range_out must hold two int32 words")
+    flags = _flags(f32_epilogue) | (L.CONV_FILTER_PREPARED if prepared_filter is not None else 0)
+    st = L.lib().niti_conv2d_i8_fprop_requant_static(
+        _ptr(x), _ptr(prepared_filter if prepared_filter is not None else w), _ptr(y), N, H, W, C, K, R, S, stride, padding, flags,
+        target_bits, L.ROUND[method], L.DIV[div_mode], L.BW[bw_mode], L.RQ_RELU if relu else 0, _ptr(shift_out), _ptr(exp_a),
+        _ptr(exp_b), _ptr(exp_out), _ptr(range_out), _stream(x))
+    L.check(st, "niti_conv2d_i8_fprop_requant_static")
+    return y, shift_out
+
+
 def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
                          prepared_filter=None, relu_mask=None, forward_filter=None, shift_hint=False):
