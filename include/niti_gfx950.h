@@ -66,6 +66,17 @@ const char* niti_last_error(void);
  * int(ceil(log2f((float)r))) under a correctly rounded log2f.  r == 0 gives 0. */
 int niti_bitwidth(uint32_t r, int bw_mode);
 
+/*
+ * Grid-wide waits that gave up.  Every single-launch kernel with a tensor-wide range (niti_conv2d_i8_*_requant,
+ * niti_conv2d_i8_wgrad_update, niti_fc_i8_*) flags a wait that ran into its time limit in word 1 of its own sync words
+ * AND in one word per device inside the library, which stays set until cleared here - so a driver whose sync words are
+ * zeroed again every step can look once per epoch, and before it writes a checkpoint.  Copies that word to *flag_out
+ * (host memory) after everything queued on `stream` so far has run (the call blocks), and zeroes it if clear != 0.
+ * Non-zero means: some output since the last clear is invalid (other work kept part of the device busy).
+ * No counterpart in the reference (its launches never wait for each other).
+ */
+int niti_sync_timeouts(uint32_t* flag_out, int clear, void* stream);
+
 /* dst[0..n) = value */
 int niti_fill_u32(uint32_t* dst, int64_t n, uint32_t value, void* stream);
 

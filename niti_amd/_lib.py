@@ -31,6 +31,7 @@ SIGNATURES = {
     "niti_status_string": (C.c_char_p, [_i]),
     "niti_last_error": (C.c_char_p, []),
     "niti_bitwidth": (_i, [C.c_uint32, _i]),
+    "niti_sync_timeouts": (_i, [_vp, _i, _vp]),
     "niti_fill_u32": (_i, [_vp, _i64, C.c_uint32, _vp]),
     "niti_conv2d_i8_filter_workspace": (_sz, [_i] * 10),
     "niti_conv2d_i8_filter_prepare": (_i, [_vp, _vp, _sz] + [_i] * 10 + [_vp]),

@@ -239,6 +239,39 @@ long long niti::sync_spin_limit() {
   return spin_limit;
 }
 
+// One word per device that every grid-wide wait of the library sets when it gives up.  The sync words of a launch
+// carry the same flag (word 1), but they are the caller's and are zeroed again before the next step; this word stays
+// set until niti_sync_timeouts clears it, so a driver can look once per epoch instead of once per launch.
+namespace {
+static __device__ uint32_t g_timeout_word;
+uint32_t* g_timeout_ptr[kDeviceSlots] = {};
+int g_timeout_dev[kDeviceSlots];
+}  // namespace
+uint32_t* niti::timeout_word() {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) return nullptr;
+  const int slot = device_slot();
+  if (g_timeout_ptr[slot] == nullptr || g_timeout_dev[slot] != dev) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_timeout_word)) != hipSuccess || p == nullptr) return nullptr;
+    g_timeout_ptr[slot] = static_cast<uint32_t*>(p);
+    g_timeout_dev[slot] = dev;
+  }
+  return g_timeout_ptr[slot];
+}
+
+extern "C" int niti_sync_timeouts(uint32_t* flag_out, int clear, void* stream) {
+  clear_error();
+  if (flag_out == nullptr) return fail(NITI_ERR_INVALID_ARG, "sync_timeouts: null pointer");
+  uint32_t* const word = timeout_word();
+  if (word == nullptr) return fail(NITI_ERR_LAUNCH, "sync_timeouts: cannot find the device word");
+  hipStream_t s = static_cast<hipStream_t>(stream);
+  if (hipMemcpyAsync(flag_out, word, sizeof(uint32_t), hipMemcpyDeviceToHost, s) != hipSuccess || hipStreamSynchronize(s) != hipSuccess)
+    return fail(NITI_ERR_LAUNCH, "sync_timeouts: %s", hipGetErrorString(hipGetLastError()));
+  if (clear != 0 && *flag_out != 0u) return launch_fill_u32(word, 1, 0u, s);
+  return NITI_OK;
+}
+
 static int fused_blocks(int N, int H, int W, int C, int K, int R, int S, int stride, int pad, int dgrad) {
   if (halo_off()) return 0;
   if (!dgrad) return conv3x3_halo_requant_blocks(N, H, W, C, K, R, S, stride, pad);
@@ -294,7 +327,7 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
   if (relu_mask != nullptr && !aligned16(relu_mask)) return fail(NITI_ERR_INVALID_ARG, "%s: relu_mask must be 16-byte aligned", who);
   if (pool_out != nullptr && (!aligned16(pool_out) || H % 2 != 0 || W % 2 != 0))
     return fail(NITI_ERR_INVALID_ARG, "%s: pool_out must be 16-byte aligned and the map side even", who);
-  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), shift_out, exp_a, exp_b, exp_out, relu_mask,
+  RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), timeout_word(), shift_out, exp_a, exp_b, exp_out, relu_mask,
                  pool_out};
   return launch_conv3x3_halo_requant(x, wp, y8, N, Hk, Ck, Kk, flags, sync, rq, s);
 }
@@ -494,7 +527,7 @@ extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err,
   if (w_prepared != nullptr && (filter_copy_kind(N, H, W, C, K, R, S, stride, pad, 0) != 2 || reinterpret_cast<uintptr_t>(w_prepared) % 4 != 0))
     return fail(NITI_ERR_UNSUPPORTED, "conv_wgrad_update: w_prepared needs a shape whose forward pass uses a kernel-ready filter copy, 4-byte aligned");
   RequantSpec rq{mu, method, div_mode == NITI_DIV_TRUNC, bw_mode, (flags & NITI_CONV_SHIFT_HINT) ? NITI_RQ_SHIFT_HINT : 0u, sync_spin_limit(),
-                 shift_out, exp_a, exp_b, exp_out, nullptr, nullptr};
+                 timeout_word(), shift_out, exp_a, exp_b, exp_out, nullptr, nullptr};
   return launch_wgrad3x3_update(act, err, w, w_channels, N, H, C, K, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, sync, rq, g8_out,
                                 dw_out, w_prepared, workspace, static_cast<hipStream_t>(stream));
 }

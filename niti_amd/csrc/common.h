@@ -117,8 +117,9 @@ inline size_t slot_words(int blocks) { return static_cast<size_t>((blocks + 15) 
 // Called by a whole wavefront: waits until all nb slots are filled and returns the largest value.  512 slots at a
 // time, eight per lane with the loads in flight together (one trip to memory per look); a lane reads a slot again
 // only while it is still empty, so the reads of the waiting workgroups die down as the slots fill.  Gives up after
-// spin_limit ticks of the 100 MHz clock: *timed_out is set to 1 and the largest value seen so far is returned.
-__device__ inline uint32_t wait_slots(uint32_t* slots, int nb, long long spin_limit, uint32_t* timed_out) {
+// spin_limit ticks of the 100 MHz clock: *timed_out (the launch's own flag) and *sticky (the device-wide word that
+// niti_sync_timeouts reads, may be null) are set to 1 and the largest value seen so far is returned.
+__device__ inline uint32_t wait_slots(uint32_t* slots, int nb, long long spin_limit, uint32_t* timed_out, uint32_t* sticky) {
   constexpr int kLook = 8;
   const int lane = threadIdx.x & 63;
   const long long t0 = wall_clock64();
@@ -141,7 +142,10 @@ __device__ inline uint32_t wait_slots(uint32_t* slots, int nb, long long spin_li
       }
       if (__all(ok)) break;
       if (wall_clock64() - t0 > spin_limit) {
-        if (lane == 0) __hip_atomic_store(timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) {
+          __hip_atomic_store(timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (sticky != nullptr) __hip_atomic_store(sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         gave_up = true;
         break;
       }
@@ -203,6 +207,7 @@ struct RequantSpec {
   int target_bits, method, trunc, bw_mode;
   unsigned flags;          // NITI_RQ_*
   long long spin_limit;    // 100 MHz wall-clock ticks the grid-wide wait may last
+  uint32_t* sticky;        // device-wide word set when a wait gives up (timeout_word()), may be null
   int32_t* shift_out;
   const int32_t* exp_a;
   const int32_t* exp_b;
@@ -212,6 +217,8 @@ struct RequantSpec {
 };
 // wall-clock ticks (100 MHz) a grid-wide wait may last (api.hip)
 long long sync_spin_limit();
+// this device's word that every grid-wide wait sets when it gives up (api.hip); nullptr if it cannot be looked up
+uint32_t* timeout_word();
 int wgrad3x3_finish_blocks(int C, int K);
 size_t wgrad3x3_sync_words(int blocks);
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,

@@ -83,6 +83,7 @@ struct HaloArgs {
   int target_bits, method, trunc, bw_mode;
   unsigned rq_flags;
   long long spin_limit;  // wall-clock ticks (100 MHz) the wait may last
+  uint32_t* sticky;      // device-wide word set when the wait gives up, may be null
   int32_t* shift_out;
   const int32_t* exp_a;
   const int32_t* exp_b;
@@ -97,6 +98,7 @@ constexpr int kSyncSlot0 = 16;
 //              was stored with the final shift; otherwise it computes its tile again and stores it with that shift.
 // With a good prediction (the previous training step's shift) the second launch does nothing but look.
 constexpr unsigned kRqNoWait = 1u << 30, kRqSettle = 1u << 31;
+static_assert(kSlotStride >= 2, "the two-launch form keeps the shift a tile was stored with in the word behind its slot");
 constexpr int kMaxSlots = 4096;
 
 // Q: image width = height; BR: output rows of one image per workgroup; NI: images per workgroup; BR*NI*Q == 256.
@@ -717,7 +719,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (final_range) break;
       // ---- wait for the slots of all workgroups; the maximum over them is the tensor's range
       if (wave == 0) {
-        const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
+        const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1], a.sticky);
         if (lane == 0) red[8] = g != 0u ? g - 1u : 0u;
       }
       __syncthreads();
@@ -885,7 +887,7 @@ __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int
       bmax = wave_max_u32(bmax);
       uint32_t* const slots = a.sync + kSyncSlot0;
       if (lane == 0) __hip_atomic_store(slot_word(slots, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
+      const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1], a.sticky);
       if (lane == 0) words[4] = g != 0u ? g - 1u : 0u;
     }
     __syncthreads();
@@ -1169,6 +1171,7 @@ int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, i
   a.bw_mode = rq.bw_mode;
   a.rq_flags = rq.flags;
   a.spin_limit = rq.spin_limit;
+  a.sticky = rq.sticky;
   a.shift_out = rq.shift_out;
   a.exp_a = rq.exp_a;
   a.exp_b = rq.exp_b;

@@ -33,6 +33,7 @@ struct FcArgs {
   int target_bits, method, trunc, bw_mode;
   unsigned rq_flags;
   long long spin_limit;
+  uint32_t* sticky;   // device-wide word set when the wait gives up, may be null
   int32_t* shift_out;
   const int32_t* exp_a;
   const int32_t* exp_b;
@@ -57,7 +58,7 @@ __device__ inline uint32_t exchange_range(const FcArgs& a, uint32_t bmax) {
   const int nb = gridDim.x;
   uint32_t* const slots = a.sync + kSlot0;
   if (lane == 0) __hip_atomic_store(slot_word(slots, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1]);
+  const uint32_t g = wait_slots(slots, nb, a.spin_limit, &a.sync[1], a.sticky);
   return g != 0u ? g - 1u : 0u;
 }
 
@@ -377,6 +378,7 @@ static int fc_common(const char* who, int which, FcArgs& a, int M, int O, int F,
   a.trunc = div_mode == NITI_DIV_TRUNC ? 1 : 0;
   a.bw_mode = bw_mode;
   a.spin_limit = sync_spin_limit();
+  a.sticky = timeout_word();
   a.shift_out = shift_out;
   a.exp_a = exp_a;
   a.exp_b = exp_b;

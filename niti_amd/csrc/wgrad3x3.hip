@@ -539,6 +539,7 @@ struct FinishArgs {
   int roundtrip, target_bits, method, trunc, bw_mode;
   int predict;         // *shift_out holds a predicted shift on entry
   long long spin_limit;
+  uint32_t* sticky;    // device-wide word set when the wait gives up, may be null
   int32_t* shift_out;
   const int32_t* exp_a;
   const int32_t* exp_b;
@@ -707,7 +708,7 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
     apply(applied, true);
   }
   if (wave == 0) {
-    const uint32_t g = wait_slots(a.sync + kFinishSlot0, gridDim.x, a.spin_limit, &a.sync[1]);
+    const uint32_t g = wait_slots(a.sync + kFinishSlot0, gridDim.x, a.spin_limit, &a.sync[1], a.sticky);
     if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
   }
   __syncthreads();
@@ -912,6 +913,7 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   f.predict = (rq.flags & NITI_RQ_SHIFT_HINT) != 0 ? 1 : 0;
   f.bw_mode = rq.bw_mode;
   f.spin_limit = rq.spin_limit;
+  f.sticky = rq.sticky;
   f.shift_out = rq.shift_out;
   f.exp_a = rq.exp_a;
   f.exp_b = rq.exp_b;

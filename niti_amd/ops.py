@@ -126,8 +126,6 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
         raise L.NitiError("%s: shape not covered by the single-launch path" % entry)
     if sync is None:
         sync = sync_arena.take(words, x.device)
-    if sync is None:
-        sync = torch.zeros(words, dtype=torch.int32, device=x.device)
     elif sync.dtype != torch.int32 or sync.numel() < words:
         raise RuntimeError("%s: sync must be a zeroed int32 tensor of at least %d words" % (entry, words))
     y = torch.empty(out_shape, dtype=torch.int8, device=x.device)
@@ -247,47 +245,73 @@ def scratch(nbytes: int, device) -> torch.Tensor:
 
 class _SyncArena:
     """Zeroed int32 words for the single-launch kernels of one training step: one fill per step instead of one
-    per kernel.  ``reset`` zeroes the whole arena and starts handing out slices from its beginning; ``take``
-    returns the next zeroed slice, or None when the arena has not been reset since it ran out (the caller then
-    allocates its own zeroed words).  Slices are handed out once per reset, so a kernel never sees words another
-    kernel of the same step wrote."""
+    per kernel.  ``reset`` zeroes the arena and starts handing out slices from its beginning; ``take`` returns the
+    next zeroed slice.  Slices are handed out once per reset, so a kernel never sees words another kernel of the
+    same step wrote.  An arena that runs out (or was never reset) grows by another zeroed chunk, which later
+    resets zero as well, so ``timed_out`` covers every slice handed out since the last reset."""
 
     WORDS = 1 << 16
+    MAX_CHUNKS = 8
 
     def __init__(self):
-        self.buf = {}
-        self.off = {}
-        self.taken = {}
+        self.chunks = {}    # device -> list of int32 tensors
+        self.pos = {}       # device -> (chunk index, offset)
+        self.taken = {}     # device -> list of (chunk index, offset)
 
     def reset(self, device):
         key = str(device)
-        if key not in self.buf:
-            self.buf[key] = torch.zeros(self.WORDS, dtype=torch.int32, device=device)
+        if key not in self.chunks:
+            self.chunks[key] = [torch.zeros(self.WORDS, dtype=torch.int32, device=device)]
         else:
-            self.buf[key].zero_()
-        self.off[key] = 0
+            for c in self.chunks[key]:
+                c.zero_()
+        self.pos[key] = (0, 0)
         self.taken[key] = []
 
     def take(self, words, device):
         key = str(device)
-        off = self.off.get(key)
-        if off is None or off + words > self.WORDS:
-            self.off[key] = None
-            return None
-        self.off[key] = off + (words + 31) // 32 * 32
-        self.taken.setdefault(key, []).append(off)
-        return self.buf[key][off:off + words]
+        if key not in self.chunks:
+            self.reset(device)
+        ci, off = self.pos[key]
+        chunks = self.chunks[key]
+        while off + words > chunks[ci].numel():
+            ci, off = ci + 1, 0
+            if ci == len(chunks):
+                if torch.cuda.is_current_stream_capturing():
+                    raise RuntimeError("sync arena: out of words while a graph is being captured; run one step eagerly first")
+                if len(chunks) >= self.MAX_CHUNKS and words <= self.WORDS:
+                    # a caller that never resets: start over (the fill is ordered behind the launches that used the
+                    # words; their flags are gone from here but stay in the device-wide word, see sync_timeouts)
+                    self.reset(device)
+                    ci, off, chunks = 0, 0, self.chunks[key]
+                    break
+                chunks.append(torch.zeros(max(self.WORDS, words), dtype=torch.int32, device=device))
+        self.pos[key] = (ci, off + (words + 31) // 32 * 32)
+        self.taken[key].append((ci, off))
+        return chunks[ci][off:off + words]
 
     def timed_out(self, device) -> bool:
         """True if a single-launch kernel that used a slice since the last reset flagged that its grid-wide wait ran
         into the time limit (its output is then invalid).  Copies the flags to the host: for the end of a step or an
         epoch, not for the inner loop."""
         key = str(device)
-        offs = self.taken.get(key)
-        if not offs:
+        flags = [self.chunks[key][ci][off + 1] for ci, off in self.taken.get(key, [])]
+        if not flags:
             return False
-        idx = torch.tensor([o + 1 for o in offs], dtype=torch.long, device=self.buf[key].device)
-        return bool(self.buf[key][idx].ne(0).any().item())
+        return bool(torch.stack(flags).ne(0).any().item())
+
+
+def sync_timeouts(device=None, clear=True) -> bool:
+    """True if any grid-wide wait of the library's kernels on ``device`` gave up since the flag was last cleared
+    (niti_sync_timeouts): some int8 output or weight update since then was made with a wrong shift.  Unlike
+    ``sync_arena.timed_out`` this survives the arena's resets.  Waits for the device's current stream."""
+    import ctypes
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    flag = ctypes.c_uint32(0)
+    with torch.cuda.device(dev):
+        st = L.lib().niti_sync_timeouts(ctypes.byref(flag), int(clear), torch.cuda.current_stream(dev).cuda_stream)
+    L.check(st, "niti_sync_timeouts")
+    return flag.value != 0
 
 
 sync_arena = _SyncArena()
@@ -337,8 +361,6 @@ def conv2d_wgrad_update(act, err, w, stride=1, padding=1, f32_epilogue=False, mu
         raise L.NitiError("conv2d_wgrad_update: shape not covered by the single-pass path")
     if sync is None:
         sync = sync_arena.take(words, act.device)
-    if sync is None:
-        sync = torch.zeros(words, dtype=torch.int32, device=act.device)
     elif sync.dtype != torch.int32 or sync.numel() < words:
         raise RuntimeError("conv2d_wgrad_update: sync must be a zeroed int32 tensor of at least %d words" % words)
     nbytes = L.lib().niti_conv2d_i8_wgrad_workspace(N, H, W, C, K, R, S, padding)
@@ -485,8 +507,6 @@ def _fc_sync(which, M, O, F, sync, device, who):
         raise L.NitiError("%s: shape not covered by the few-output-features kernels" % who)
     if sync is None:
         sync = sync_arena.take(words, device)
-    if sync is None:
-        sync = torch.zeros(words, dtype=torch.int32, device=device)
     elif sync.dtype != torch.int32 or sync.numel() < words:
         raise RuntimeError("%s: sync must be a zeroed int32 tensor of at least %d words" % (who, words))
     return sync

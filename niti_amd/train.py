@@ -19,7 +19,7 @@ import numpy as np
 import torch
 import torch.nn.functional as F
 
-from . import ti_torch
+from . import ops, ti_torch
 from .ti_vgg import TiVGG_cifar
 
 
@@ -142,7 +142,22 @@ def run_epoch(data_loader, model, training, log_interval=0, epoch=0, use_graph=F
     if count == 0:
         return 0.0, 0.0, 0.0
     loss_avg, top1, top5 = (sums / count).tolist()
+    check_waits(dev)
     return loss_avg, top1, top5
+
+
+class GridWaitTimeout(RuntimeError):
+    """A kernel that exchanges a tensor-wide range between its workgroups gave up waiting for some of them."""
+
+
+def check_waits(dev=None):
+    """Raises if any single-launch kernel since the last check flagged a grid-wide wait that ran into its time limit
+    (other work kept part of the device busy): activations, errors or weight updates since then were rounded with a
+    wrong shift, so the pass is invalid and its weights must not be saved.  One 4-byte read per call; run_epoch calls
+    it at the end of every pass, i.e. before fit() writes a checkpoint."""
+    if ops.sync_timeouts(dev if dev is not None else torch.device(ti_torch.GPU), clear=True):
+        raise GridWaitTimeout("a grid-wide wait of the int8 kernels timed out during this pass: the device was shared with "
+                              "other work; results of the pass are invalid and nothing was saved")
 
 
 def save_checkpoint(state, is_best, path='.', filename='checkpoint.pth.tar', save_all=False):
@@ -248,10 +263,16 @@ def main(argv=None):
     p.add_argument('--init', help='init ckpt')
     p.add_argument('--depth', default=7, type=int)
     p.add_argument('--no-graph', action='store_true', help='issue every launch of a step from Python instead of replaying a HIP graph')
+    p.add_argument('--div-mode', choices=('floor', 'trunc'), default=ti_torch.DIV_MODE,
+                   help="meaning of // on negative numbers in the rounding helpers: floor (torch >= 1.13, default) or "
+                        "trunc (torch <= 1.12, what the reference's published runs used)")
+    p.add_argument('--bw-mode', choices=('int', 'f32'), default=ti_torch.BW_MODE,
+                   help="bit width of a range: exact integer ceil(log2 r) (default) or the reference's float32 evaluation")
     args = p.parse_args(argv)
     logging.basicConfig(level=logging.INFO, format='%(asctime)s %(message)s')
     if args.seed > 0:
         torch.manual_seed(args.seed)
+    ti_torch.DIV_MODE, ti_torch.BW_MODE = args.div_mode, args.bw_mode
     model = TiVGG_cifar(depth=args.depth)
     if args.init:
         load_checkpoint(model, args.init)

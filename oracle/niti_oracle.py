@@ -32,8 +32,15 @@ Pin status per function (what fixes the result, besides the source text):
   maxpool bwd             unique maxima: closed form.  TIES: parity unpinned (cuDNN's rule is
                           closed source); rule chosen here = first maximum in (kh,kw) scan
                           order (= torch CPU), "all" kept as a switchable alternative.
-  ti_loss                 parity unpinned across devices (fp32 pow inside); full-step parity
-                          tests feed the same int8 loss gradient to both sides.
+  ti_loss                 known answers of tests/golden/ti_loss_kat.json (exact rational arithmetic with
+                          explicit float32 rounding, hand-worked rows for both exponent branches) + the
+                          plain-C statement.  ``2 ** s`` follows exp2_contract (a fixed sequence of double
+                          operations = the correctly rounded float32 power on every tested argument); the
+                          reference's own result there depends on its platform's powf by an ulp.
+  float_to_int8 / weight_quant   hand-derived known answers (tests/golden/quantize_kat.json: ranges at and
+                          next to powers of two, half-way ties, both clamps) + the plain-C statement.
+                          ceil(log2 r) is exact arithmetic on the float; the reference's float32 log2
+                          rounds to the lower integer for the first float32 values above 2^k, k >= 4.
 The reference holds no tests, golden vectors or fixtures for any of these.
 """
 from __future__ import annotations

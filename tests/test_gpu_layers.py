@@ -364,6 +364,17 @@ for i in range(4):
     torch.cuda.synchronize()
     flagged += int(sync.cpu()[1] != 0)
 print("FLAGGED", flagged, "ARENA", int(ops.sync_arena.timed_out(dev)))
+# the device-wide word survives the arena's reset, is cleared by a read, and the epoch driver's check raises on it
+ops.sync_arena.reset(dev)
+print("STICKY", int(ops.sync_arena.timed_out(dev)), int(ops.sync_timeouts(dev, clear=False)), int(ops.sync_timeouts(dev)),
+      int(ops.sync_timeouts(dev)))
+from niti_amd import train
+y, sh, sync = ops.conv2d_fprop_requant(x, w)
+try:
+    train.check_waits(dev)
+    print("RAISED 0")
+except train.GridWaitTimeout:
+    print("RAISED 1")
 """
     env = dict(os.environ, NITI_SYNC_TIMEOUT_MS="0.00001")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
@@ -371,3 +382,6 @@ print("FLAGGED", flagged, "ARENA", int(ops.sync_arena.timed_out(dev)))
     assert out.returncode == 0, out.stderr[-2000:]
     line = [l for l in out.stdout.splitlines() if l.startswith("FLAGGED")][0].split()
     assert int(line[1]) >= 1 and int(line[3]) == 1
+    sticky = [l for l in out.stdout.splitlines() if l.startswith("STICKY")][0].split()
+    assert sticky[1:] == ["0", "1", "1", "0"], sticky
+    assert "RAISED 1" in out.stdout
