@@ -86,7 +86,8 @@ class ConvTriple:
         self.exp0 = torch.zeros(1, dtype=torch.int32, device=dev)
         self.ops_per_step = sum(conv_ops(BATCH, hw, c, k) * (2 if i == 0 else 3) for i, (c, k, hw) in enumerate(LAYERS))
         self.main_kernel_ops = []     # algorithmic ops of every launch bracketed by events, in launch order
-        self.events = []
+        self.events = []           # forward and data-gradient launches (the dominant kernel)
+        self.wgrad_events = []     # weight gradient + rounding + update (two kernels per bracket)
 
     def step(self, record=False):
         torch, ops = self.torch, self.ops
@@ -116,7 +117,7 @@ class ConvTriple:
                 acc = ops.conv2d_fprop(L["x16"], w16, 1, 1, f32_epilogue=True, absmax=am[0:1], prepared_filter=wp)
             if record:
                 e1.record()
-                self.events.append((e0, e1, conv_ops(BATCH, hw, c, k)))
+                self.events.append((e0, e1, conv_ops(BATCH, hw, c, k), i, "fprop"))
             if not sn:
                 ops.requant(acc, am[0:1], 7, "round", exp_a=self.exp0, exp_b=self.exp0, exp_out=torch.empty_like(self.exp0))
             # data gradient + error requantisation
@@ -134,11 +135,14 @@ class ConvTriple:
                     dx = ops.conv2d_dgrad(L["err"], L["w"], 1, 1, f32_epilogue=True, absmax=am[1:2], prepared_filter=wt)
                 if record:
                     e1.record()
-                    self.events.append((e0, e1, conv_ops(BATCH, hw, c, k)))
+                    self.events.append((e0, e1, conv_ops(BATCH, hw, c, k), i, "dgrad"))
                 if not sn:
                     ops.requant(dx, am[1:2], 7, "round")
             # weight gradient + gradient rounding + weight update
             so, sn = L["sync_w"]
+            if record:
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record()
             if sn:
                 ops.conv2d_wgrad_update(L["x16"], L["err"], L["w"], 1, 1, f32_epilogue=(i > 0), mu=5, method="psto",
                                         sync=self.sync[so:so + sn], workspace=self.ws, prepared_filter=L["wp"],
@@ -149,6 +153,9 @@ class ConvTriple:
                 if c % 16:
                     dw = dw[..., :c].contiguous()     # zero-padded input channels give zero gradient columns
                 ops.grad_update(dw, L["w"], am[2:3], 5, "psto")
+            if record:
+                e1.record()
+                self.wgrad_events.append((e0, e1, conv_ops(BATCH, hw, c, k), i, "wgrad"))
 
 
 def make_runner(step_fn, warmup, use_graph=True):
@@ -237,6 +244,125 @@ def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH, graph=True):
     return batch / dt, dt * 1e3, mode
 
 
+def _avg_us(fn, reps=20, warm=3):
+    """Average duration of fn() in microseconds over `reps` back-to-back calls, by one HIP event pair on the launch
+    stream around the whole run; a device sleep queued first lets the host run ahead, so the device never idles
+    between the launches."""
+    import torch
+    for _ in range(warm):
+        fn()
+    torch.cuda.synchronize()
+    torch.cuda._sleep(int(2e7))
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(reps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / reps
+
+
+def side_workloads(dev):
+    """The other configurations and bandwidth kernels, each on its own roofline:
+    config0  BASELINE configs[0]: one 128 -> 128 convolution on 128 x 32 x 32 + RoundShift requantisation
+             (ti_torch.py:391-397), as one launch (MFMA roofline) and as the drop-in int32 convolution + separate
+             requantisation (cutlassconv.cpp:57-73: HBM roofline, |x| + |w| + 4|y| bytes);
+    config1  BASELINE configs[1]: fully connected layer 128 x 8192 x 1024, forward / data gradient / weight gradient
+             with StoShift on supplied random integers (ti_torch.py:241-266, int8mm_kernel.cu:8-34), against the HBM
+             roofline with m k + k n + m n bytes per pass;
+    maxpool  2x2 / stride-2 int8 max-pool forward (1.25 |x| bytes) and backward (2.5 |x| bytes)."""
+    import torch
+    from niti_amd import ops
+    g = torch.Generator().manual_seed(1234)
+    out = {}
+    # ---- config 0
+    N, hw, c, k = 128, 32, 128, 128
+    x = torch.randint(-127, 128, (N, hw, hw, c), generator=g, dtype=torch.int8).to(dev)
+    w = torch.randint(-127, 128, (k, 3, 3, c), generator=g, dtype=torch.int8).to(dev)
+    wp = ops.conv_filter_prepare(w, N, hw, hw)
+    words = ops.conv_requant_sync_words(N, hw, hw, c, k)
+    sync = torch.zeros(words, dtype=torch.int32, device=dev)
+    shift = torch.zeros(1, dtype=torch.int32, device=dev)
+    gop = conv_ops(N, hw, c, k) / 1e9
+
+    def fused():
+        sync.zero_()
+        ops.conv2d_fprop_requant(x, w, f32_epilogue=True, sync=sync, prepared_filter=wp, shift_out=shift, shift_hint=True)
+
+    def fill_only():
+        sync.zero_()
+
+    am = torch.zeros(1, dtype=torch.int32, device=dev)
+    y32 = {}
+
+    def dropin_conv():
+        y32["y"] = ops.conv2d_fprop(x, w, 1, 1, f32_epilogue=True, prepared_filter=wp)
+
+    def two_pass():
+        am.zero_()
+        acc = ops.conv2d_fprop(x, w, 1, 1, f32_epilogue=True, absmax=am, prepared_filter=wp)
+        ops.requant(acc, am, 7, "round")
+
+    t_fill = _avg_us(fill_only)
+    t_fused = max(_avg_us(fused) - t_fill, 1e-3)
+    t_conv = _avg_us(dropin_conv)
+    t_two = max(_avg_us(two_pass) - t_fill, 1e-3)
+    y_elems = N * hw * hw * k
+    bytes_dropin = x.numel() + w.numel() + 4 * y_elems
+    out["config0"] = {
+        "workload": "BASELINE configs[0]: conv3x3 128->128 on 128x32x32 + RoundShift requantisation, %.2f GOP" % gop,
+        "fused_us": round(t_fused, 2), "fused_tops": round(gop / t_fused * 1e3, 1),
+        "fused_frac_mfma": round(gop / t_fused * 1e3 / INT8_MFMA_PEAK_TOPS, 4),
+        "dropin_int32_conv_us": round(t_conv, 2), "dropin_gbs": round(bytes_dropin / t_conv * 1e-3, 1),
+        "dropin_frac_hbm": round(bytes_dropin / t_conv * 1e-3 / HBM_PEAK_GBS, 4), "dropin_bytes": bytes_dropin,
+        "two_pass_us": round(t_two, 2), "two_pass_tops": round(gop / t_two * 1e3, 1)}
+    del y32, x, w
+    # ---- config 1
+    M, Fin, O = 128, 8192, 1024
+    A = torch.randint(-127, 128, (M, Fin), generator=g, dtype=torch.int8).to(dev)
+    W = torch.randint(-127, 128, (O, Fin), generator=g, dtype=torch.int8).to(dev)
+    G = torch.randint(-127, 128, (M, O), generator=g, dtype=torch.int8).to(dev)
+    u_f = torch.randint(0, 1 << 20, (M, O), generator=g, dtype=torch.int32).to(dev)
+    u_d = torch.randint(0, 1 << 20, (M, Fin), generator=g, dtype=torch.int32).to(dev)
+    u_w = torch.randint(0, 1 << 20, (O, Fin), generator=g, dtype=torch.int32).to(dev)
+    Wu = W.clone()
+
+    def fc_fwd():
+        am.zero_()
+        ops.requant(ops.gemm(A, W, trans_b=True, absmax=am), am, 7, "sto", rand=u_f)
+
+    def fc_dgrad():
+        am.zero_()
+        ops.requant(ops.gemm(G, W, absmax=am), am, 7, "sto", rand=u_d)
+
+    def fc_wgrad():
+        am.zero_()
+        ops.grad_update(ops.gemm(G, A, trans_a=True, absmax=am), Wu, am, 5, "sto", rand=u_w)
+
+    fc = {"workload": "BASELINE configs[1]: fully connected 128x8192x1024, int32 GEMM + StoShift on supplied random integers; "
+                      "bytes = m k + k n + m n per pass", "gop_per_pass": round(2.0 * M * Fin * O / 1e9, 3)}
+    for name, fn, nbytes in (("fwd", fc_fwd, M * Fin + Fin * O + M * O), ("dgrad", fc_dgrad, M * O + O * Fin + M * Fin),
+                             ("wgrad", fc_wgrad, O * M + M * Fin + O * Fin)):
+        t = max(_avg_us(fn) - t_fill, 1e-3)
+        fc[name + "_us"] = round(t, 2)
+        fc[name + "_gbs"] = round(nbytes / t * 1e-3, 1)
+        fc[name + "_frac_hbm"] = round(nbytes / t * 1e-3 / HBM_PEAK_GBS, 4)
+        fc[name + "_tops"] = round(2.0 * M * Fin * O / t * 1e-6, 1)
+    out["config1"] = fc
+    del A, W, G, u_f, u_d, u_w, Wu
+    # ---- max-pool
+    xp = torch.randint(-127, 128, (128, 32, 32, 128), generator=g, dtype=torch.int8).to(dev)
+    yp = ops.maxpool_fwd(xp)
+    dy = torch.randint(-127, 128, tuple(yp.shape), generator=g, dtype=torch.int8).to(dev)
+    t_f = _avg_us(lambda: ops.maxpool_fwd(xp))
+    t_b = _avg_us(lambda: ops.maxpool_bwd(yp, dy, xp))
+    nb = xp.numel()
+    out["maxpool"] = {"workload": "2x2/stride-2 int8 max-pool on 128x32x32x128",
+                      "fwd_us": round(t_f, 2), "fwd_gbs": round(1.25 * nb / t_f * 1e-3, 1), "fwd_frac_hbm": round(1.25 * nb / t_f * 1e-3 / HBM_PEAK_GBS, 4),
+                      "bwd_us": round(t_b, 2), "bwd_gbs": round(2.5 * nb / t_b * 1e-3, 1), "bwd_frac_hbm": round(2.5 * nb / t_b * 1e-3 / HBM_PEAK_GBS, 4)}
+    return out
+
+
 TRAIN_STEPS = (("train_step", 7, BATCH, "BASELINE configs[3]: VGG-small (6 conv + FC) integer training step, batch 128"),
                ("train_step_vgg13", 13, 256, "BASELINE configs[4]: VGG-13 widths (10 conv + FC) integer training step, batch 256"))
 
@@ -259,6 +385,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train-step", action="store_true")
+    ap.add_argument("--no-side-workloads", action="store_true", help="skip config0 / config1 / max-pool figures")
+    ap.add_argument("--sustained-seconds", type=float, default=1.0,
+                    help="also replay the headline step back to back for at least this long (0: skip)")
     ap.add_argument("--train-steps-only", action="store_true",
                     help="run only the two training-step workloads and print their objects (for kernel traces of a step)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a captured HIP graph")
@@ -300,6 +429,25 @@ def main():
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     tops = wl.ops_per_step / (ms_per_step * 1e-3) / 1e12
+    from niti_amd import ops as _ops
+    if _ops.sync_timeouts(dev):
+        print("bench.py: a grid-wide wait timed out during the timed steps (the GPU was shared with other work); "
+              "no result", file=sys.stderr)
+        return 4
+    # the same step replayed back to back for a second or more: clocks and temperature settle, unlike in the K-step burst
+    sustained = None
+    if args.sustained_seconds > 0:
+        n_rep = max(int(args.sustained_seconds * 1e3 / ms_per_step * 1.15), args.steps)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(n_rep):
+            run()
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        sustained = {"steps": n_rep, "seconds": round(dt, 3), "ms_per_step": round(dt * 1e3 / n_rep, 4),
+                     "tops": round(wl.ops_per_step * n_rep / dt / 1e12, 2)}
+        if _ops.sync_timeouts(dev):
+            sustained["error"] = "a grid-wide wait timed out"
 
     # Dominant kernel: the MFMA implicit-GEMM convolution (forward + data-gradient launches), timed
     # per launch with HIP events on the launch stream over the same K steps run eagerly.  A device
@@ -320,21 +468,36 @@ def main():
         pairs.append((e0, e1))
     torch.cuda.synchronize()
     pair_ms = sorted(e0.elapsed_time(e1) for (e0, e1) in pairs)[len(pairs) // 2]
-    k_ms = sum(max(e0.elapsed_time(e1) - pair_ms, 0.0) for (e0, e1, _) in wl.events)
-    k_ops = sum(o for (_, _, o) in wl.events)
+    k_ms = sum(max(ev[0].elapsed_time(ev[1]) - pair_ms, 0.0) for ev in wl.events)
+    k_ops = sum(ev[2] for ev in wl.events)
     n_launch = len(wl.events)
     achieved = k_ops / (k_ms * 1e-3) / 1e12
+    # per layer and direction: average bracket over the K eager steps (a weight-gradient bracket holds its two kernels)
+    per_layer = []
+    for i, (c, k, hw) in enumerate(LAYERS):
+        row = {"layer": "%d->%d@%d" % (c, k, hw)}
+        for direction, evs in (("fprop", wl.events), ("dgrad", wl.events), ("wgrad", wl.wgrad_events)):
+            sel = [ev for ev in evs if ev[3] == i and ev[4] == direction]
+            if not sel:
+                continue
+            us = sum(max(ev[0].elapsed_time(ev[1]) - pair_ms, 0.0) for ev in sel) * 1e3 / len(sel)
+            t = sel[0][2] / (us * 1e-6) / 1e12
+            row[direction] = {"us": round(us, 2), "tops": round(t, 1), "frac": round(t / INT8_MFMA_PEAK_TOPS, 4)}
+        per_layer.append(row)
     # HBM bytes per launch of this kernel as the counters of an earlier rocprofv3 run gave them (the summary states
     # the figure on a line of its own); null when the summary is not there
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "conv_triple_hbm_traffic.txt")
+    traffic_source = None
     if os.path.exists(tpath):
+        traffic_source = "profiles/conv_triple_hbm_traffic.txt (rocprofv3 FETCH_SIZE / WRITE_SIZE of an earlier run of this command, " \
+                         "scaled by a plain copy; counters cannot be read inside this run)"
         with open(tpath) as f:
             for line in f:
                 if line.startswith("traffic_bytes_per_launch:"):
                     traffic = int(line.split(":", 1)[1].split()[0])
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
-                "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic,
+                "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                 "kernel": "conv3x3_halo_kernel<..., true, *> (convolution + requantisation)", "launches": n_launch,
                 "avg_launch_us": round(k_ms * 1e3 / max(n_launch, 1), 2), "event_pair_overhead_us": round(pair_ms * 1e3, 2),
                 "ops_per_launch_avg": k_ops / max(n_launch, 1),
@@ -350,7 +513,14 @@ def main():
                       "ops_per_step": wl.ops_per_step, "batch": BATCH},
            "launch_mode": mode,
            "pct_int8_mfma_peak": round(100.0 * tops / INT8_MFMA_PEAK_TOPS, 2),
-           "roofline": roofline}
+           "roofline": roofline, "per_layer": per_layer}
+    if sustained is not None:
+        out["sustained"] = sustained
+    if not args.no_side_workloads:
+        try:
+            out.update(side_workloads(dev))
+        except Exception as e:  # the headline line must still be printed
+            out["side_workloads_error"] = str(e)[:300]
     if not args.no_train_step:
         out.update(train_step_objects(dev, max(args.steps, 5), max(args.warmup, 2)))
     if not args.no_cpu_baseline:
