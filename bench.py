@@ -262,6 +262,24 @@ def _avg_us(fn, reps=20, warm=3):
     return e0.elapsed_time(e1) * 1e3 / reps
 
 
+def mfma_probe(dev):
+    """What the matrix units sustain in a register-resident MFMA loop (no LDS, no memory traffic) for constant and for
+    uniform random int8 operands: the shader clock follows the multipliers' power draw, so the second figure - not the
+    datasheet peak - is the ceiling of kernels that multiply random data."""
+    import torch
+    from niti_amd import ops
+    g = torch.Generator().manual_seed(4321)
+    const = torch.ones(1 << 20, dtype=torch.int8, device=dev)
+    rnd = torch.randint(-127, 128, (1 << 20,), generator=g, dtype=torch.int8).to(dev)
+    ops.mfma_probe(const)                              # clocks up
+    ct, cg = ops.mfma_probe(const)
+    rt, rg = ops.mfma_probe(rnd)
+    return {"constant_operands_tops": round(ct, 1), "constant_operands_clock_ghz": round(cg, 2),
+            "random_operands_tops": round(rt, 1), "random_operands_clock_ghz": round(rg, 2),
+            "note": "512 workgroups x 8 wavefronts x 1200 x 12 v_mfma_i32_32x32x32_i8 on register operands; clock = shader "
+                    "cycle counter against the 100 MHz wall clock inside the loop"}
+
+
 def side_workloads(dev):
     """The other configurations and bandwidth kernels, each on its own roofline:
     config0  BASELINE configs[0]: one 128 -> 128 convolution on 128 x 32 x 32 + RoundShift requantisation
@@ -514,6 +532,13 @@ def main():
            "launch_mode": mode,
            "pct_int8_mfma_peak": round(100.0 * tops / INT8_MFMA_PEAK_TOPS, 2),
            "roofline": roofline, "per_layer": per_layer}
+    try:
+        probe = mfma_probe(dev)
+        out["mfma_probe"] = probe
+        roofline["frac_of_random_operand_probe"] = round(achieved / probe["random_operands_tops"], 4)
+        out["pct_of_random_operand_probe"] = round(100.0 * tops / probe["random_operands_tops"], 2)
+    except Exception as e:
+        out["mfma_probe"] = {"error": str(e)[:200]}
     if sustained is not None:
         out["sustained"] = sustained
     if not args.no_side_workloads:

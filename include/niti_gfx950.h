@@ -364,6 +364,18 @@ int niti_loss_grad_i8(const int8_t* out_val, const int32_t* out_exp, const int64
 int niti_group_conv_i8_f32(const int8_t* x, const int8_t* w, float* y, int N, int H, int W, int C, int K, int R,
                            int S, int Cg, int stride, int pad, int dilation, int groups, void* stream);
 
+/*
+ * Measurement aid, no counterpart in the reference: a register-resident int8 MFMA loop (v_mfma_i32_32x32x32_i8, no LDS
+ * and no memory traffic inside the loop) over operand fragments read once from `operands` (operand_bytes >= 128,
+ * 16-byte aligned).  `workgroups` x 8 wavefronts each run `iters` rounds of 12 MFMAs = iters * 12 * 65536 int8
+ * operations per wavefront.  The rate depends on the operand VALUES (the shader clock follows the multipliers' power
+ * draw): time it with events for constant and for random operands to see the ceiling the convolution kernels run
+ * under.  out: workgroups * 512 int32 checksums.  clocks (may be NULL): [0] shader clocks, [1] 100 MHz ticks that
+ * workgroup 0 spent in the loop.
+ */
+int niti_mfma_probe_i8(const int8_t* operands, size_t operand_bytes, int workgroups, int iters, int32_t* out,
+                       int64_t* clocks, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -604,6 +604,32 @@ def loss_grad(out_val, out_exp, target, rand, div_mode="floor"):
     return grad
 
 
+def mfma_probe(operands, workgroups=512, iters=1200):
+    """Times the library's register-resident int8 MFMA loop over the given operand bytes (int8 tensor, >= 128 bytes).
+    Returns (tera-operations per second, shader clock in GHz during the loop): the matrix-unit ceiling for operands
+    with these values."""
+    _chk_dev(operands)
+    if operands.dtype != torch.int8 or not operands.is_contiguous():
+        raise RuntimeError("mfma_probe: contiguous int8 tensor expected")
+    out = torch.empty(workgroups * 512, dtype=torch.int32, device=operands.device)
+    clocks = torch.zeros(2, dtype=torch.int64, device=operands.device)
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+
+    def launch():
+        L.check(L.lib().niti_mfma_probe_i8(_ptr(operands), operands.numel(), workgroups, iters, _ptr(out), _ptr(clocks),
+                                           _stream(operands)), "niti_mfma_probe_i8")
+    for _ in range(3):
+        launch()
+    e0.record()
+    launch()
+    e1.record()
+    torch.cuda.synchronize()
+    ms = e0.elapsed_time(e1)
+    c = clocks.tolist()
+    tops = workgroups * 8 * iters * 12 * 65536.0 / (ms * 1e-3) / 1e12
+    return tops, (c[0] / (c[1] * 10.0) if c[1] else 0.0)
+
+
 def maxpool_fwd(x, kernel_size=2, stride=2, padding=0):
     _chk_dev(x)
     if x.dtype != torch.int8:
