@@ -346,6 +346,29 @@ int niti_fc_i8_wgrad_update(const int8_t* err, const int8_t* act, int8_t* w, int
                             const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
 
 /*
+ * TiLinear of any width (ti_torch.py:241-266) on the matrix cores, each pass as one launch with its requantisation
+ * folded in; replaces int8mm_cuda.int8_mm (int8mm.cpp:9-14, int8mm_kernel.cu:8-34) + the transposing copies around it
+ * (ti_torch.py:246,263,176) + act_calc / err_calc / grad_calc + weight_update.  Operands as the layer stores them:
+ * act [M][F], w [O][F], err [M][O], int8; no operand is re-laid and no int32 product is written to memory.
+ * Rounding: NITI_ROUND_NEAREST, NITI_ROUND_PSEUDO_STOCHASTIC, or NITI_ROUND_STOCHASTIC with `rand` (one int32 per
+ * OUTPUT element - [M][O], [M][F], [O][F] - low `shift` bits used, as in niti_requant_i32_i8; NULL otherwise).
+ * Shapes: forward F % 16 == 0, O % 4 == 0; dgrad O % 32 == 0, F % 32 == 0, O <= 4096; wgrad O % 16 == 0, F % 16 == 0;
+ * 16-byte aligned operands.  niti_linear_i8_sync_words returns 0 for shapes outside that or whose workgroups the
+ * current device does not hold at once (then use niti_gemm_i8 + niti_requant_i32_i8 / niti_grad_update_i8).
+ * sync, shift_out, exp_* as in niti_fc_i8_*.
+ */
+size_t niti_linear_i8_sync_words(int which, int M, int O, int F);
+int niti_linear_i8_fwd_requant(const int8_t* act, const int8_t* w, int8_t* out8, int M, int O, int F, int target_bits, int method,
+                               int div_mode, int bw_mode, unsigned rq_flags, const int32_t* rand, uint32_t* sync, size_t sync_words,
+                               int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
+int niti_linear_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8, int M, int O, int F, int target_bits, int method,
+                                 int div_mode, int bw_mode, const int32_t* rand, uint32_t* sync, size_t sync_words,
+                                 int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
+int niti_linear_i8_wgrad_update(const int8_t* err, const int8_t* act, int8_t* w, int M, int O, int F, int mu, int method,
+                                int div_mode, int bw_mode, const int32_t* rand, uint32_t* sync, size_t sync_words, int8_t* g8_out,
+                                int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* stream);
+
+/*
  * Integer cross-entropy gradient, TiLoss.forward (ti_loss.py:5-36), as one launch: out_val [n][classes] int8 logits
  * with exponent *out_exp (device scalar), target [n] int64 class indices, rand [n][classes] int32 random integers
  * (the low four bits stand in for the reference's torch.randint(0, 16)) -> grad [n][classes] int8 with exponent 0.

@@ -571,6 +571,82 @@ def fc_wgrad_update(err, act, w, mu=5, method="psto", div_mode="floor", bw_mode=
     return g8, shift_out, sync
 
 
+def linear_sync_words(which, M, O, F) -> int:
+    """uint32 words of the sync buffer the any-width TiLinear kernels need for a pass ("forward", "dgrad", "wgrad") on
+    the current device; 0 when the shape is outside them (then: gemm + requant / grad_update)."""
+    return int(L.lib().niti_linear_i8_sync_words({"forward": 0, "dgrad": 1, "wgrad": 2}[which], M, O, F))
+
+
+def _linear_sync(which, M, O, F, sync, device, who):
+    words = linear_sync_words(which, M, O, F)
+    if words == 0:
+        raise L.NitiError("%s: shape not covered by the any-width linear kernels" % who)
+    if sync is None:
+        sync = sync_arena.take(words, device)
+    elif sync.dtype != torch.int32 or sync.numel() < words:
+        raise RuntimeError("%s: sync must be a zeroed int32 tensor of at least %d words" % (who, words))
+    return sync
+
+
+def _chk_rand(rand, shape, who):
+    if rand is not None and (rand.dtype != torch.int32 or tuple(rand.shape) != tuple(shape) or not rand.is_contiguous()):
+        raise RuntimeError("%s: rand must be a contiguous int32 tensor shaped like the output" % who)
+
+
+def linear_fwd_requant(act, w, target_bits=7, method="round", div_mode="floor", bw_mode="int", relu=False, rand=None, sync=None,
+                       shift_out=None, exp_a=None, exp_b=None, exp_out=None):
+    """act_calc(act @ w^T) in one launch for a layer of any width: act [M,F] int8, w [O,F] int8 -> ([M,O] int8, shift,
+    sync).  ``rand`` (int32 [M,O]) for method "sto"."""
+    _chk_dev(act, w, rand, sync, shift_out, exp_a, exp_b, exp_out)
+    M, F = act.shape
+    O = w.shape[0]
+    _chk_rand(rand, (M, O), "linear_fwd_requant")
+    sync = _linear_sync("forward", M, O, F, sync, act.device, "linear_fwd_requant")
+    y = torch.empty((M, O), dtype=torch.int8, device=act.device)
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=act.device)
+    L.check(L.lib().niti_linear_i8_fwd_requant(_ptr(act), _ptr(w), _ptr(y), M, O, F, target_bits, L.ROUND[method], L.DIV[div_mode],
+                                               L.BW[bw_mode], L.RQ_RELU if relu else 0, _ptr(rand), _ptr(sync), sync.numel(),
+                                               _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _stream(act)),
+            "niti_linear_i8_fwd_requant")
+    return y, shift_out, sync
+
+
+def linear_dgrad_requant(err, w, target_bits=7, method="round", div_mode="floor", bw_mode="int", rand=None, sync=None,
+                         shift_out=None, exp_a=None, exp_b=None, exp_out=None):
+    """err_calc(err @ w) in one launch: err [M,O] int8, w [O,F] int8 -> ([M,F] int8, shift, sync)."""
+    _chk_dev(err, w, rand, sync, shift_out, exp_a, exp_b, exp_out)
+    M, O = err.shape
+    F = w.shape[1]
+    _chk_rand(rand, (M, F), "linear_dgrad_requant")
+    sync = _linear_sync("dgrad", M, O, F, sync, err.device, "linear_dgrad_requant")
+    y = torch.empty((M, F), dtype=torch.int8, device=err.device)
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=err.device)
+    L.check(L.lib().niti_linear_i8_dgrad_requant(_ptr(err), _ptr(w), _ptr(y), M, O, F, target_bits, L.ROUND[method], L.DIV[div_mode],
+                                                 L.BW[bw_mode], _ptr(rand), _ptr(sync), sync.numel(), _ptr(shift_out), _ptr(exp_a),
+                                                 _ptr(exp_b), _ptr(exp_out), _stream(err)), "niti_linear_i8_dgrad_requant")
+    return y, shift_out, sync
+
+
+def linear_wgrad_update(err, act, w, mu=5, method="psto", div_mode="floor", bw_mode="int", rand=None, sync=None, want_grad=False,
+                        shift_out=None, exp_a=None, exp_b=None, exp_out=None):
+    """grad_calc(err^T @ act) and the weight update in one launch: err [M,O], act [M,F], w [O,F] int8 updated in place.
+    Returns (int8 gradient or None, shift, sync)."""
+    _chk_dev(err, act, w, rand, sync, shift_out, exp_a, exp_b, exp_out)
+    M, O = err.shape
+    F = act.shape[1]
+    _chk_rand(rand, (O, F), "linear_wgrad_update")
+    sync = _linear_sync("wgrad", M, O, F, sync, err.device, "linear_wgrad_update")
+    g8 = torch.empty((O, F), dtype=torch.int8, device=w.device) if want_grad else None
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=w.device)
+    L.check(L.lib().niti_linear_i8_wgrad_update(_ptr(err), _ptr(act), _ptr(w), M, O, F, mu, L.ROUND[method], L.DIV[div_mode],
+                                                L.BW[bw_mode], _ptr(rand), _ptr(sync), sync.numel(), _ptr(g8), _ptr(shift_out),
+                                                _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _stream(err)), "niti_linear_i8_wgrad_update")
+    return g8, shift_out, sync
+
+
 def pad_last_dim(t, multiple=16):
     """``t`` with zeros appended along its last dimension up to a multiple of ``multiple`` (``t`` itself when it
     already is one): the channel padding of conv2d_int8 (ti_torch.py:182-187) as one launch."""

@@ -552,6 +552,20 @@ class TiLinear(UpdateWeight):
         return (FUSE_CONV_REQUANT and rand is None and _method_name(fn) != "sto" and self.weight.is_contiguous()
                 and (which, M, O, F) not in _fused_refused and ops.fc_sync_words(which, M, O, F) > 0)
 
+    def _wide(self, which, M):
+        """The pass runs as one of the library's any-width kernels (operands as stored, requantisation folded in, random
+        rounding included) when the shape is inside them and the layer has more than a few output features."""
+        O, F = self.weight.shape
+        return (FUSE_CONV_REQUANT and O > 16 and self.weight.is_contiguous() and ("wide", which, M, O, F) not in _fused_refused
+                and ops.linear_sync_words(which, M, O, F) > 0)
+
+    @staticmethod
+    def _sto_rand(fn, rand, shape, dev):
+        """Random integers for a stochastic rounding of a tensor of ``shape`` (the caller's, or drawn here)."""
+        if _method_name(fn) != "sto":
+            return None
+        return rand if rand is not None else torch.randint(0, 2 ** 31 - 1, shape, dtype=torch.int32, device=dev)
+
     def _try(self, which, M, call):
         """``call()``, or None when the device turned out too small to hold the kernel's grid at once."""
         from ._lib import NitiError
@@ -573,6 +587,15 @@ class TiLinear(UpdateWeight):
             act_out, _, _ = ops.fc_fwd_requant(act_in, self.weight, BITWIDTH, _method_name(ACT_ROUND_METHOD), DIV_MODE, BW_MODE,
                                                exp_a=_exp_tensor(exp_in, dev), exp_b=self._wexp(), exp_out=exp_out)
             return act_out, exp_out
+        if self._wide("forward", act_in.shape[0]):
+            exp_out = torch.empty(1, dtype=torch.int32, device=dev)
+            M, O = act_in.shape[0], self.weight.shape[0]
+            done = self._try("wide-forward", M, lambda: ops.linear_fwd_requant(
+                act_in, self.weight, BITWIDTH, _method_name(ACT_ROUND_METHOD), DIV_MODE, BW_MODE,
+                rand=self._sto_rand(ACT_ROUND_METHOD, rand, (M, O), dev), exp_a=_exp_tensor(exp_in, dev), exp_b=self._wexp(),
+                exp_out=exp_out))
+            if done is not None:
+                return done[0], exp_out
         am = ops.new_scalar_u32(dev)
         acc = ops.gemm(act_in, self.weight, trans_b=True, absmax=am)            # act @ W^T, W read as stored
         act_out, _, exp_out = _requant(acc, BITWIDTH, ACT_ROUND_METHOD, am, rand,
@@ -593,6 +616,12 @@ class TiLinear(UpdateWeight):
             done = self._try("dgrad", M, lambda: ops.fc_dgrad_requant(
                 err_in, self.weight, BITWIDTH, _method_name(ERROR_ROUND_METHOD), DIV_MODE, BW_MODE,
                 exp_a=self.err_exp_in, exp_b=self._wexp(), exp_out=new_exp))
+        if done is None and self._wide("dgrad", M):
+            new_exp = torch.empty(1, dtype=torch.int32, device=dev)
+            done = self._try("wide-dgrad", M, lambda: ops.linear_dgrad_requant(
+                err_in, self.weight, BITWIDTH, _method_name(ERROR_ROUND_METHOD), DIV_MODE, BW_MODE,
+                rand=self._sto_rand(ERROR_ROUND_METHOD, rand, (M, self.weight.shape[1]), dev), exp_a=self.err_exp_in,
+                exp_b=self._wexp(), exp_out=new_exp))
         if done is not None:
             err_out, self.err_exp = done[0], new_exp
         else:
@@ -607,6 +636,12 @@ class TiLinear(UpdateWeight):
                 err_in, act, self.weight, GRAD_BITWIDTH, _method_name(GRAD_ROUND_METHOD), DIV_MODE, BW_MODE,
                 want_grad=self.keep_grad, exp_a=_exp_tensor(self.err_exp, dev), exp_b=_exp_tensor(self.act_in_exp, dev),
                 exp_out=self.grad_exp))
+        if done is None and not KEEP_INT32_GRAD and self._wide("wgrad", M):
+            self.grad_exp = torch.empty(1, dtype=torch.int32, device=dev)
+            done = self._try("wide-wgrad", M, lambda: ops.linear_wgrad_update(
+                err_in, act, self.weight, GRAD_BITWIDTH, _method_name(GRAD_ROUND_METHOD), DIV_MODE, BW_MODE,
+                rand=self._sto_rand(GRAD_ROUND_METHOD, grad_rand, tuple(self.weight.shape), dev), want_grad=self.keep_grad,
+                exp_a=_exp_tensor(self.err_exp, dev), exp_b=_exp_tensor(self.act_in_exp, dev), exp_out=self.grad_exp))
         if done is not None:
             self.grad, self.grad_shift, self.grad_int32acc = done[0], done[1], None
         else:

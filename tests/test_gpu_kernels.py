@@ -838,3 +838,64 @@ def test_group_conv_first_layer_wgrad(dev):
     gw = gw.permute(0, 2, 3, 1).contiguous()
     assert gw.dtype == torch.float32
     assert torch.equal(gw, po.conv2d_weight_int8(act, (K, 3, 3, C), err, 1, 1))
+
+
+@pytest.mark.parametrize("case", [(128, 8192, 1024), (40, 256, 64), (300, 512, 96), (16, 64, 32), (64, 320, 32), (128, 1024, 2048),
+                                  (7, 4096, 128)])   # M, F, O
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+def test_linear_any_width(dev, case, div_mode):
+    """TiLinear's three passes as single launches on operands as stored, all rounding methods (stochastic rounding on
+    supplied random integers), against int8mm + act_calc / err_calc / grad_calc / weight_update of the oracle."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    M, F, O = case
+    _say("linear_any_width", case, div_mode)
+    g = torch.Generator().manual_seed(5000 + M + O)
+    act, w, err = ri8(g, M, F), ri8(g, O, F), ri8(g, M, O, lo=-60, hi=60)
+    acc_f = co.gemm(act, w.t().contiguous())            # [M,O]
+    acc_d = co.gemm(err, w)                             # [M,F]
+    acc_w = co.gemm(err.t().contiguous(), act)          # [O,F]
+    assert torch.equal(acc_f, po.int8mm(act, w.t().contiguous()))
+    ad, wd, ed = act.to(dev), w.to(dev), err.to(dev)
+    for method in ("round", "psto", "sto"):
+        uf = torch.randint(0, 1 << 24, (M, O), generator=g, dtype=torch.int32)
+        ud = torch.randint(0, 1 << 24, (M, F), generator=g, dtype=torch.int32)
+        uw = torch.randint(0, 1 << 24, (O, F), generator=g, dtype=torch.int32)
+        sto = method == "sto"
+
+        def low(u, acc, bits):    # the low `shift` bits, as the reference's randint(0, 2^shift) would give
+            s = max(po.bitwidth_int(po.absmax(acc)) - bits, 0)
+            return u & ((1 << s) - 1) if s > 0 else torch.zeros_like(u)
+        if ops.linear_sync_words("forward", M, O, F):
+            ref, e_ref = po.act_calc(acc_f, -5, method, div_mode, rand=low(uf, acc_f, 7) if sto else None)
+            ea = torch.tensor([-5], dtype=torch.int32, device=dev)
+            eo = torch.zeros(1, dtype=torch.int32, device=dev)
+            y, sh, sync = ops.linear_fwd_requant(ad, wd, 7, method, div_mode, rand=uf.to(dev) if sto else None, exp_a=ea, exp_out=eo)
+            sync = sync.cpu()
+            assert int(sync[1]) == 0 and int(sync[0]) == po.absmax(acc_f), method
+            assert torch.equal(y.cpu(), ref) and int(eo.cpu()) == e_ref, method
+            yr, _, _ = ops.linear_fwd_requant(ad, wd, 7, method, div_mode, relu=True, rand=uf.to(dev) if sto else None)
+            assert torch.equal(yr.cpu(), torch.clamp(ref, min=0)), method
+        else:
+            assert O % 4 or F % 16
+        if ops.linear_sync_words("dgrad", M, O, F):
+            ref, sh_ref = po.err_calc(acc_d, method, div_mode, rand=low(ud, acc_d, 7) if sto else None)
+            y, sh, sync = ops.linear_dgrad_requant(ed, wd, 7, method, div_mode, rand=ud.to(dev) if sto else None)
+            sync = sync.cpu()
+            assert int(sync[1]) == 0 and int(sync[0]) == po.absmax(acc_d), method
+            assert int(sh.cpu()) == sh_ref and torch.equal(y.cpu(), ref), method
+        else:
+            assert O % 32 or F % 32
+        if ops.linear_sync_words("wgrad", M, O, F):
+            g8_ref, sh_ref = po.grad_calc(acc_w, 5, method, div_mode, rand=low(uw, acc_w, 5) if sto else None)
+            w_ref = po.weight_update(w, g8_ref)
+            wu = wd.clone()
+            g8, sh, sync = ops.linear_wgrad_update(ed, ad, wu, 5, method, div_mode, rand=uw.to(dev) if sto else None, want_grad=True)
+            sync = sync.cpu()
+            assert int(sync[1]) == 0 and int(sync[0]) == po.absmax(acc_w), method
+            assert int(sh.cpu()) == sh_ref and torch.equal(g8.cpu(), g8_ref) and torch.equal(wu.cpu(), w_ref), method
+        else:
+            assert O % 16 or F % 16
+    assert ops.linear_sync_words("forward", 128, 1024, 8192) > 0 and ops.linear_sync_words("dgrad", 128, 1024, 8192) > 0
+    assert ops.linear_sync_words("wgrad", 128, 1024, 8192) > 0

@@ -125,6 +125,20 @@ def test_linear_layer_fwd_bwd(tt, methods, shape):
     ro = o.backward((err, -2), cfg, rb, rg)
     layer = tt.TiLinear(kin, nout)
     layer.weight, layer.weight_exp, layer.keep_grad = w.to(dev), torch.tensor(-8.0), True
+    from niti_amd import ops
+    gemm_calls = []
+    real_gemm = ops.gemm
+    if nout == 1024:
+        # the wide layer runs as three launches that read the operands as stored: no GEMM into int32, no re-layout
+        ops.gemm = lambda *a, **k: gemm_calls.append(1) or real_gemm(*a, **k)
+    try:
+        _run_linear_layer(tt, layer, x, err, rf, rb, rg, yo, eo, ro, o, dev)
+    finally:
+        ops.gemm = real_gemm
+    assert not gemm_calls
+
+
+def _run_linear_layer(tt, layer, x, err, rf, rb, rg, yo, eo, ro, o, dev):
     y, e = layer.forward((x.to(dev), 1), rf.to(dev))
     assert torch.equal(y.cpu(), yo) and _ei(e) == eo
     r = layer.backward((err.to(dev), -2), rb.to(dev), rg.to(dev))
