@@ -411,6 +411,8 @@ def main():
                     help="also replay the headline step back to back for at least this long (0: skip)")
     ap.add_argument("--train-steps-only", action="store_true",
                     help="run only the two training-step workloads and print their objects (for kernel traces of a step)")
+    ap.add_argument("--side-workloads-only", action="store_true",
+                    help="run only config0 / config1 / max-pool and the MFMA probe and print their objects (for kernel traces)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a captured HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a kernel of known traffic, to scale "
@@ -436,6 +438,12 @@ def main():
             dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.side_workloads_only:
+        out = side_workloads(dev)
+        out["mfma_probe"] = mfma_probe(dev)
+        print(json.dumps(out))
+        return 0
 
     if args.train_steps_only:
         print(json.dumps(train_step_objects(dev, args.steps, args.warmup, not args.eager)))
