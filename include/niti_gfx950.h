@@ -177,6 +177,25 @@ int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8
                                  size_t workspace_bytes, void* stream);
 
 /*
+ * niti_conv2d_i8_dgrad_requant that also runs the backward pass of the 2x2 / stride-2 max-pool in front of the layer:
+ * replaces TiConv2d.backward's data gradient + err_calc (ti_torch.py:403-407), the ReLU mask, and the
+ * TiMaxpool2d.backward -> int8pool_cuda.int8_pool_backward call that follows it in the reference's networks
+ * (ti_torch.py:309-316, int8pool_kernel.cu:82-138; ti_vgg.py:28-35), with the same result as
+ * niti_conv2d_i8_dgrad_requant(.., relu_mask = pooled, ..) followed by niti_maxpool_i8_bwd(pooled, that, pool_in, .., 2, 2,
+ * 0, ties).  N, H, W, C, K describe the convolution (H x W = the pooled map); pooled: [N,H,W,C] int8, the pooling's
+ * output = the layer's input activations; pool_in: [N,2H,2W,C] int8, the pooling's input; dx8_unpooled: [N,2H,2W,C]
+ * int8; all 16-byte aligned.  Elements whose pooled value is not positive get zero (the ReLU in front of the pooling);
+ * the others go to the first position of their window that equals the pooled value (NITI_TIES_FIRST) or to all of them
+ * (NITI_TIES_ALL).  Same coverage as niti_conv2d_i8_dgrad_requant except maps of side 2 (NITI_ERR_UNSUPPORTED).
+ */
+int niti_conv2d_i8_dgrad_requant_unpool(const int8_t* err, const int8_t* w, int8_t* dx8_unpooled, const int8_t* pooled,
+                                        const int8_t* pool_in, int ties, int N, int H, int W, int C, int K, int R, int S, int stride,
+                                        int pad, unsigned flags, int target_bits, int method, int div_mode, int bw_mode,
+                                        unsigned rq_flags, uint32_t* sync, size_t sync_words, int32_t* shift_out,
+                                        const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
+                                        size_t workspace_bytes, void* stream);
+
+/*
  * niti_conv2d_i8_fprop_requant for callers that cannot allocate device memory or hand in scratch memory: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
  * arithmetic and the same results as niti_conv2d_i8_fprop_requant; the sync words and the kernel-ready filter copy live

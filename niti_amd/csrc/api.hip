@@ -291,7 +291,8 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
                         int K, int R, int S, int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
                         int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync, size_t sync_words,
                         int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out, void* workspace,
-                        size_t workspace_bytes, void* stream, int8_t* pool_out = nullptr) {
+                        size_t workspace_bytes, void* stream, int8_t* pool_out = nullptr, const int8_t* pool_x = nullptr,
+                        int ties = -1) {
   clear_error();
   int st = check_conv_dims(who, N, H, W, C, K, R, S, stride, pad);
   if (st == NITI_OK)
@@ -329,6 +330,13 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
     return fail(NITI_ERR_INVALID_ARG, "%s: pool_out must be 16-byte aligned and the map side even", who);
   RequantSpec rq{target_bits, method, div_mode == NITI_DIV_TRUNC, bw_mode, rq_flags, sync_spin_limit(), timeout_word(), shift_out, exp_a, exp_b, exp_out, relu_mask,
                  pool_out};
+  if (pool_x != nullptr) {   // y8 is the [N,2H,2W,C] result of the folded max-pool backward pass
+    if (ties != NITI_TIES_FIRST && ties != NITI_TIES_ALL) return fail(NITI_ERR_INVALID_ARG, "%s: ties=%d", who, ties);
+    if (relu_mask == nullptr || !aligned16(pool_x)) return fail(NITI_ERR_INVALID_ARG, "%s: pooled map and 16-byte aligned pooling input needed", who);
+    rq.pool_x = pool_x;
+    rq.unpool = y8;
+    rq.ties_all = ties == NITI_TIES_ALL ? 1 : 0;
+  }
   return launch_conv3x3_halo_requant(x, wp, y8, N, Hk, Ck, Kk, flags, sync, rq, s);
 }
 
@@ -435,6 +443,21 @@ extern "C" int niti_conv2d_i8_fprop_requant_static(const int8_t* x, const int8_t
   if (st != NITI_OK || range_out == nullptr) return st;
   hipLaunchKernelGGL(copy_words_kernel, dim3(1), dim3(64), 0, s, sync, range_out, 2);
   return check_launch(who);
+}
+
+extern "C" int niti_conv2d_i8_dgrad_requant_unpool(const int8_t* err, const int8_t* w, int8_t* dx8_unpooled, const int8_t* pooled,
+                                                   const int8_t* pool_in, int ties, int N, int H, int W, int C, int K, int R, int S,
+                                                   int stride, int pad, unsigned flags, int target_bits, int method, int div_mode,
+                                                   int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words,
+                                                   int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                                   void* workspace, size_t workspace_bytes, void* stream) {
+  if (pooled == nullptr || pool_in == nullptr) {
+    clear_error();
+    return fail(NITI_ERR_INVALID_ARG, "conv_dgrad_requant_unpool: null pointer");
+  }
+  return conv_requant("conv_dgrad_requant_unpool", 1, err, w, dx8_unpooled, N, H, W, C, K, R, S, stride, pad, flags, target_bits, method,
+                      div_mode, bw_mode, rq_flags, pooled, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace,
+                      workspace_bytes, stream, nullptr, pool_in, ties);
 }
 
 extern "C" size_t niti_conv2d_i8_wgrad_workspace(int N, int H, int W, int C, int K, int R, int S, int pad) {

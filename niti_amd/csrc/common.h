@@ -214,6 +214,10 @@ struct RequantSpec {
   int32_t* exp_out;
   const int8_t* mask;      // conv + requantisation only: optional ReLU-backward mask, laid out like the output
   int8_t* pool;            // forward conv + requantisation only: optional 2x2 / stride-2 maximum of the output
+  // data gradient only: fold in the backward pass of a 2x2 / stride-2 max-pool in front of the layer (mask = pooled map)
+  const int8_t* pool_x = nullptr;   // the pooling's input [N,2H,2W,C]
+  int8_t* unpool = nullptr;         // result [N,2H,2W,C] (the [N,H,W,C] output is then not written)
+  int ties_all = 0;
 };
 // wall-clock ticks (100 MHz) a grid-wide wait may last (api.hip)
 long long sync_spin_limit();

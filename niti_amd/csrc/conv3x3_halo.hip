@@ -80,6 +80,13 @@ struct HaloArgs {
   long long y8_bytes;
   int8_t* pool;       // optional [N,Q/2,Q/2,K] int8: 2x2 / stride-2 maximum of y8 (the max-pool that follows the layer)
   long long pool_bytes;
+  // data gradient through a 2x2 / stride-2 max-pool in front of the layer: `mask` is the pooled map (this launch's
+  // result is the gradient with respect to it), pool_x the pooling's input [N,2Q,2Q,K]; the rounded, masked result
+  // goes to the position(s) of each window that equal the pooled value, into unpool [N,2Q,2Q,K], and y8 is not written
+  const int8_t* pool_x;
+  int8_t* unpool;
+  long long unpool_bytes;
+  int ties_all;
   int target_bits, method, trunc, bw_mode;
   unsigned rq_flags;
   long long spin_limit;  // wall-clock ticks (100 MHz) the wait may last
@@ -687,10 +694,41 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
           for (int q = 0; q < 4; ++q) v[q] &= static_cast<int>(positive_bytes(static_cast<uint32_t>(mk[q])));
         }
-        // the 128-channel tile writes 64 bytes per pixel and wavefront: streaming stores start the write-back of the
-        // 16 MiB result while the kernel still runs (measured 2 us per launch); the 32-byte pieces of the 64-channel
-        // tile are slower that way
-        __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, NWF == 2 ? 2 : 0);
+        if (a.unpool != nullptr) {
+          // max-pool backward folded in (mk holds the pooled values): the window of pooled pixel m in the pooling's input
+          const __amdgpu_buffer_rsrc_t rxp = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.pool_x), 0, a.unpool_bytes, 0x00020000);
+          const __amdgpu_buffer_rsrc_t ru = __builtin_amdgcn_make_buffer_rsrc(a.unpool, 0, a.unpool_bytes, 0x00020000);
+          const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
+          const auto mk = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
+          const int n = m / (Q * Q), rem = m - n * (Q * Q);
+          const int pp = rem / Q, pq = rem - pp * Q;
+          const int rowb = 2 * Q * a.K;
+          const int base = ((n * 2 * Q + 2 * pp) * 2 * Q + 2 * pq) * a.K + ch;
+          int wo[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) wo[k] = off == kOob ? kOob : base + (k >> 1) * rowb + (k & 1) * a.K;
+          v4i xw[4], ow[4];
+#pragma unroll
+          for (int k = 0; k < 4; ++k) xw[k] = __builtin_amdgcn_raw_buffer_load_b128(rxp, wo[k], 0, 0);
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            uint32_t taken = 0;   // bytes whose gradient an earlier position of the window (scan order) already received
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              const uint32_t eq = equal_bytes(static_cast<uint32_t>(xw[k][q]), static_cast<uint32_t>(mk[q]));
+              const uint32_t keep = a.ties_all != 0 ? eq : eq & ~taken;
+              ow[k][q] = static_cast<int>(static_cast<uint32_t>(v[q]) & keep);
+              taken |= eq;
+            }
+          }
+#pragma unroll
+          for (int k = 0; k < 4; ++k) __builtin_amdgcn_raw_buffer_store_b128(ow[k], ru, wo[k], 0, 0);
+        } else {
+          // the 128-channel tile writes 64 bytes per pixel and wavefront: streaming stores start the write-back of the
+          // 16 MiB result while the kernel still runs (measured 2 us per launch); the 32-byte pieces of the 64-channel
+          // tile are slower that way
+          __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, NWF == 2 ? 2 : 0);
+        }
       }
       if (a.pool != nullptr) {
         // The max-pool behind this layer, from the rounded values still in the patch: the wavefront's 64 pixels are a
@@ -1163,6 +1201,15 @@ int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, i
   a.y8_bytes = static_cast<long long>(N) * H * H * K;
   a.pool = rq.pool;
   a.pool_bytes = static_cast<long long>(N) * (H / 2) * (H / 2) * K;
+  a.pool_x = rq.pool_x;
+  a.unpool = rq.unpool;
+  a.unpool_bytes = 4 * a.y8_bytes;
+  a.ties_all = rq.ties_all;
+  if (a.unpool != nullptr) {
+    if (H == 2) return fail(NITI_ERR_UNSUPPORTED, "conv_requant: the max-pool backward pass is not folded in on 2 x 2 maps");
+    if (a.mask == nullptr || a.pool_x == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_requant: unpooling needs the pooled map and the pooling's input");
+    if (a.unpool_bytes >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "conv_requant: unpooled map of 2 GiB or more");
+  }
   if (a.pool != nullptr && H == 2)
     return fail(NITI_ERR_UNSUPPORTED, "conv_requant: the pooled output is not available on 2 x 2 maps");
   a.target_bits = rq.target_bits;

@@ -151,13 +151,6 @@ __global__ __launch_bounds__(256) void maxpool_bwd_kernel(const PoolArgs a) {
   }
 }
 
-// 0xFF in every byte where a and b agree
-__device__ inline uint32_t equal_bytes(uint32_t a, uint32_t b) {
-  const uint32_t z = a ^ b;
-  const uint32_t nz = (((z & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | z) & 0x80808080u;   // bit 7 of the bytes that differ
-  return ((nz ^ 0x80808080u) >> 7) * 0xFFu;
-}
-
 // The layers' case: 2 x 2 windows, stride 2, no padding, even H and W, C % 16 == 0.  Windows do not overlap, so a
 // lane owns one window x 16 channels: six 16-byte loads, byte-parallel compares, four 16-byte stores.
 template <bool kAll>

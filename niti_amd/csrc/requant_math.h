@@ -95,6 +95,13 @@ __host__ __device__ inline uint32_t positive_bytes(uint32_t m) {
   return (pos >> 7) * 0xFFu;
 }
 
+// 0xFF in every byte where a and b agree
+__host__ __device__ inline uint32_t equal_bytes(uint32_t a, uint32_t b) {
+  const uint32_t z = a ^ b;
+  const uint32_t nz = (((z & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | z) & 0x80808080u;   // bit 7 of the bytes that differ
+  return ((nz ^ 0x80808080u) >> 7) * 0xFFu;
+}
+
 // the larger of four signed bytes, byte by byte: each byte in the high half of a 16-bit lane keeps its order there
 __device__ inline uint32_t max_i8x4(uint32_t a, uint32_t b) {
   typedef short s2_t __attribute__((ext_vector_type(2)));

@@ -114,10 +114,18 @@ def conv_requant_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1, dgrad=
 
 def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epilogue, target_bits, method, div_mode,
                   bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None, forward_filter=None,
-                  shift_hint=False, pool_out=None):
+                  shift_hint=False, pool_out=None, unpool=None):
     _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask, forward_filter)
     if relu_mask is not None and (relu_mask.dtype != torch.int8 or tuple(relu_mask.shape) != tuple(out_shape)):
         raise RuntimeError("%s: relu_mask must be int8 and shaped like the output" % entry)
+    if unpool is not None:      # (pooling input [N,2H,2W,C], tie rule): the result is written at that size
+        pool_in, ties = unpool
+        _chk_dev(x, pool_in)
+        n_, h_, w_, c_ = out_shape
+        if relu_mask is None or pool_in.dtype != torch.int8 or tuple(pool_in.shape) != (n_, 2 * h_, 2 * w_, c_) or not pool_in.is_contiguous():
+            raise RuntimeError("%s: unpool needs relu_mask (the pooled map) and a contiguous int8 [N,2H,2W,C] pooling input" % entry)
+        entry = "niti_conv2d_i8_dgrad_requant_unpool"
+        out_shape = tuple(pool_in.shape)
     if x.dtype != torch.int8 or w.dtype != torch.int8:
         raise RuntimeError("%s: int8 tensors expected" % entry)
     N, H, W, C, K, R, S = dims
@@ -147,7 +155,11 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
     tail = (_ptr(sync), sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes, _stream(x))
     if pool_out is not None:    # the entry with the pooled output takes it right after the output
         head = head[:3] + (_ptr(pool_out),) + head[3:]
-    st = getattr(L.lib(), entry)(*(head + ((_ptr(relu_mask),) if dgrad else ()) + tail))
+    if unpool is not None:
+        head = head[:3] + (_ptr(relu_mask), _ptr(unpool[0]), L.TIES[unpool[1]]) + head[3:]
+        st = getattr(L.lib(), entry)(*(head + tail))
+    else:
+        st = getattr(L.lib(), entry)(*(head + ((_ptr(relu_mask),) if dgrad else ()) + tail))
     L.check(st, entry)
     return y, shift_out, sync
 
@@ -211,8 +223,10 @@ def conv2d_fprop_requant_static(x, w, stride=1, padding=1, f32_epilogue=False, t
 
 def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None, relu_mask=None, forward_filter=None, shift_hint=False):
+                         prepared_filter=None, relu_mask=None, forward_filter=None, shift_hint=False, unpool=None):
     """conv2d_dgrad + requant as one launch: err [N,P,Q,K] int8, w [K,R,S,C] int8 -> ([N,H,W,C] int8, shift, sync).
+    ``unpool`` = (pool_in [N,2H,2W,C] int8, "first" | "all") with ``relu_mask`` = the pooled map: the backward pass of
+    the 2x2 / stride-2 max-pool in front of the layer is folded in and the result has pool_in's shape.
     ``relu_mask`` (int8 [N,H,W,C]): results whose mask element is not positive are stored as zero, after range
     and rounding were taken from the unmasked sums (the backward pass of a ReLU in front of the layer).
     ``forward_filter``: the copy the forward pass reads, in place of ``prepared_filter`` (see conv2d_dgrad)."""
@@ -224,7 +238,7 @@ def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target
     W = Q - 2 * padding + S - 1
     return _conv_requant("niti_conv2d_i8_dgrad_requant", True, err, w, (N, H, W, C), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, False, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter, relu_mask, forward_filter, shift_hint)
+                         prepared_filter, relu_mask, forward_filter, shift_hint, unpool=unpool)
 
 
 _scratch = {}

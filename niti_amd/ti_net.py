@@ -37,6 +37,9 @@ class TiNet(Module):
             if j < len(layers) and isinstance(layers[j], ti_torch.TiConv2d) and not layers[j].first_layer:
                 layers[j].relu_below = True
                 l.bwd_folded = True
+                if j == i + 2 and (layers[i + 1].kernel_size, layers[i + 1].stride, layers[i + 1].padding) == (2, 2, 0):
+                    # ... and the data gradient writes its result through that max-pool's backward pass as well
+                    layers[j].pool_below = layers[i + 1]
             elif j == i + 2:
                 # ReLU -> max-pool -> anything else: the pooling's backward pass applies the mask to its own output
                 layers[i + 1].relu_below = True

@@ -190,14 +190,14 @@ _fused_refused = set()       # (dgrad, input shape, filter shape, stride, paddin
 
 
 def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None, prepared_filter=None,
-                        forward_filter=None, shift_state=None, pool_out=None):
+                        forward_filter=None, shift_state=None, pool_out=None, unpool=None):
     """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
     exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
     single-launch kernel, or more workgroups than the device holds at once."""
     method = _method_name(fn)
     if not FUSE_CONV_REQUANT or method == "sto" or rand is not None:
         return None
-    key = (dgrad, tuple(x.shape), tuple(w.shape), stride, padding)
+    key = (dgrad, tuple(x.shape), tuple(w.shape), stride, padding, unpool is not None)
     if key in _fused_refused:
         return None
     N = x.shape[0]
@@ -212,6 +212,8 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
     kw = dict(relu=relu, prepared_filter=prepared_filter) if not dgrad else dict(relu_mask=relu_mask, forward_filter=forward_filter)
     if pool_out is not None:
         kw.update(pool_out=pool_out)
+    if unpool is not None:
+        kw.update(unpool=unpool)
     if shift_state is not None:     # the tensor's shift of the previous step: the kernel's prediction for this one
         kw.update(shift_out=shift_state, shift_hint=True)
     try:
@@ -378,6 +380,7 @@ class TiConv2d(UpdateWeight):
         self.fuse_relu = False
         self.relu_below = False
         self.pool_after = None      # the 2x2 / stride-2 TiMaxpool2d behind this layer's (fused) ReLU, if its forward is folded in
+        self.pool_below = None      # the 2x2 / stride-2 TiMaxpool2d in front of this layer, if its backward pass is folded in
 
     def forward(self, input, rand=None):
         self.act, self.act_in_exp = input
@@ -463,6 +466,16 @@ class TiConv2d(UpdateWeight):
 
     def _data_gradient(self, err_in, rand, mask, forward_filter):
         """err_calc(conv_dgrad(err_in, weight)) (ti_torch.py:422-427), the ReLU mask applied; -> (int8 error, exponent)."""
+        pool = self.pool_below
+        if (pool is not None and mask is not None and err_in.shape[1] > 2 and getattr(pool, "act_out", None) is not None
+                and pool.act_out.data_ptr() == mask.data_ptr() and pool.act_in.is_contiguous()):
+            # the max-pool in front of this layer: its backward pass is written by this launch's epilogue
+            fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
+                                        False, self.err_exp_in, self._wexp(), relu_mask=mask, forward_filter=forward_filter,
+                                        shift_state=self._shift_state("err", err_in.device), unpool=(pool.act_in, POOL_TIES))
+            if fused is not None:
+                pool.bwd_done = fused[0]
+                return fused[0], fused[2]
         fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
                                     False, self.err_exp_in, self._wexp(), relu_mask=mask, forward_filter=forward_filter,
                                     shift_state=self._shift_state("err", err_in.device))
@@ -685,6 +698,7 @@ class TiMaxpool2d(Module):
         self.padding = padding
         self.relu_below = False     # the ReLU in front of this layer leaves its backward pass to this layer
         self.preset = None          # (input tensor, pooled tensor) left by the convolution that computed both
+        self.bwd_done = None        # the error tensor a convolution behind this layer has already routed through it
 
     def forward(self, input):
         self.act_in, exp_in = input
@@ -698,6 +712,9 @@ class TiMaxpool2d(Module):
 
     def backward(self, input):
         err_in, err_exp = input
+        done, self.bwd_done = self.bwd_done, None
+        if done is not None and done is err_in:
+            return input        # the data gradient behind this layer wrote its result through this pooling already
         err_out = ops.maxpool_bwd(self.act_out, err_in.contiguous(), self.act_in, self.kernel_size, self.stride,
                                   self.padding, POOL_TIES, relu=self.relu_below)
         return err_out, err_exp

@@ -899,3 +899,41 @@ def test_linear_any_width(dev, case, div_mode):
             assert O % 16 or F % 16
     assert ops.linear_sync_words("forward", 128, 1024, 8192) > 0 and ops.linear_sync_words("dgrad", 128, 1024, 8192) > 0
     assert ops.linear_sync_words("wgrad", 128, 1024, 8192) > 0
+
+
+@pytest.mark.parametrize("case", [(4, 8, 16, 32), (8, 16, 128, 64), (2, 16, 48, 80), (16, 4, 64, 128), (8, 32, 32, 16), (1024, 16, 48, 32),
+                                  (264, 16, 16, 272)])   # N, Q (pooled map), C, K; the last two: 512-pixel tiles, two-launch form
+def test_conv_dgrad_requant_unpool(dev, case):
+    """Data gradient + err_calc + ReLU mask + the backward pass of the 2x2 max-pool in front of the layer in one launch,
+    against the oracle's three steps; windows with several equal maxima under both tie rules."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_dgrad_requant_unpool", case)
+    g = torch.Generator().manual_seed(990 + C + K)
+    e, w = ri8(g, N, Q, Q, K), ri8(g, K, 3, 3, C)
+    pool_in = ri8(g, N, 2 * Q, 2 * Q, C, lo=-3, hi=5)            # few distinct values: many ties, many non-positive maxima
+    pooled = po.maxpool_fwd(pool_in)
+    acc = co.conv_dgrad(e, w, Q, Q, 1, 1)
+    ed, wd, pd, xd = e.to(dev), w.to(dev), pooled.to(dev), pool_in.to(dev)
+    for method in ("round", "psto"):
+        dx, sh_ref = po.err_calc(acc, method)
+        dx = torch.where(pooled > 0, dx, torch.zeros_like(dx))
+        for ties in ("first", "all"):
+            ref = co.maxpool_bwd(pooled, dx, pool_in, 2, 2, 0, ties)
+            y, sh, sync = ops.conv2d_dgrad_requant(ed, wd, 1, 1, method=method, relu_mask=pd, unpool=(xd, ties))
+            assert tuple(y.shape) == tuple(pool_in.shape) and int(sync.cpu()[1]) == 0
+            assert int(sh.cpu()) == sh_ref and int(sync.cpu()[0]) == po.absmax(acc)
+            assert torch.equal(y.cpu(), ref), (method, ties)
+        # the forward filter copy as the filter operand, and a wrong shift prediction (stores twice)
+        so = torch.tensor([max(sh_ref - 2, 0)], dtype=torch.int32, device=dev)
+        y, sh, _ = ops.conv2d_dgrad_requant(ed, wd, 1, 1, method=method, relu_mask=pd, unpool=(xd, "first"),
+                                            forward_filter=ops.conv_filter_prepare(wd, N, Q, Q), shift_out=so, shift_hint=True)
+        assert int(so.cpu()) == sh_ref and torch.equal(y.cpu(), co.maxpool_bwd(pooled, dx, pool_in, 2, 2, 0, "first")), method
+    # maps of side 2 keep the separate pooling pass
+    from niti_amd._lib import NitiError
+    with pytest.raises(NitiError):
+        ops.conv2d_dgrad_requant(torch.zeros((32, 2, 2, 32), dtype=torch.int8, device=dev), torch.zeros((32, 3, 3, 32), dtype=torch.int8, device=dev),
+                                 relu_mask=torch.zeros((32, 2, 2, 32), dtype=torch.int8, device=dev),
+                                 unpool=(torch.zeros((32, 4, 4, 32), dtype=torch.int8, device=dev), "first"))

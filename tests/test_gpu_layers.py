@@ -383,7 +383,8 @@ ops.sync_arena.reset(dev)
 print("STICKY", int(ops.sync_arena.timed_out(dev)), int(ops.sync_timeouts(dev, clear=False)), int(ops.sync_timeouts(dev)),
       int(ops.sync_timeouts(dev)))
 from niti_amd import train
-y, sh, sync = ops.conv2d_fprop_requant(x, w)
+for i in range(8):      # whether a launch runs into the one-tick limit depends on timing: several tries
+    y, sh, sync = ops.conv2d_fprop_requant(x, w)
 try:
     train.check_waits(dev)
     print("RAISED 0")
