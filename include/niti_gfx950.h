@@ -398,6 +398,53 @@ int niti_loss_grad_i8(const int8_t* out_val, const int32_t* out_exp, const int64
                       int8_t* grad, int n, int classes, int div_mode, void* stream);
 
 /*
+ * Random integers drawn inside the kernels.  The reference draws a dropout mask (ti_torch.py:444) and the random
+ * integers of the loss gradient's StoShift (ti_loss.py:35, ti_torch.py:88-90) with torch.randint on the device, a
+ * launch each; the entry points below that take `rng` draw them themselves.  rng: four uint32 words in device memory,
+ * {key0, key1, step, 0}, which the caller initialises once (any key, step 0) and the kernels advance: every launch
+ * that draws adds 1 to `step` when its last workgroup is done.  Word i of stream s in a launch that finds step t is
+ * output word (i & 3) of Philox4x32-10 with counter {i >> 2, s, t, 0} and key {key0, key1} (stream 1: dropout, a
+ * feature is kept when bit 0 of its word is set; stream 2: loss gradient, logit i uses the low four bits of word i).
+ * niti_rng_words_u32 writes the first n words of a stream that a launch would draw in the state's present step (it
+ * does not advance the state): what a test or a replaying host needs to predict a kernel's draws.
+ * niti_loss_grad_i8_rng is niti_loss_grad_i8 with the random integers drawn from rng.
+ */
+int niti_rng_words_u32(const uint32_t* rng, uint32_t stream_id, uint32_t* out, size_t n, void* stream);
+int niti_loss_grad_i8_rng(const int8_t* out_val, const int32_t* out_exp, const int64_t* target, uint32_t* rng, int8_t* grad,
+                          int n, int classes, int div_mode, void* stream);
+
+/*
+ * The classifier at the end of a network in two launches: TiDropout.forward + TiLinear.forward (+ TiLoss.forward when
+ * the targets are known), then TiLinear.backward + TiDropout.backward (ti_vgg.py:37-40, ti_torch.py:241-266, :439-455,
+ * ti_loss.py:5-36; in the reference about sixty tensor-operation launches, with the passes above nine).
+ * niti_head_i8_forward: out8 [M][O] = act_calc((act * mask) @ w^T) as niti_fc_i8_fwd_requant, with
+ *   dropout 0: no mask; 1: drop_mask [F] (bytes 0 / 1) is read; 2: the mask is drawn from rng and written to drop_mask;
+ *   exp_bias is added to *exp_out (TiDropout adds 1 to the exponent);
+ *   target [M] int64 or null: with it loss_grad [M][O] receives what niti_loss_grad_i8 gives for the logits just
+ *   written (their exponent being *exp_out), with loss_rand [M][O] or, when that is null, draws from rng.
+ * niti_head_i8_backward: err [M][O] (exponent *exp_err) ->
+ *   dx8 [M][F] = err_calc(err @ w) * mask, *err_exp_out = shift + *exp_err + *exp_w (ti_torch.py:258-260);
+ *   w = clip(w - grad_calc(err^T @ (act * mask), grad_bits)) in place (ti_torch.py:262-263, :16-21), g8_out [O][F]
+ *   optionally the rounded gradient, *grad_exp_out = its shift + *err_exp_out + *exp_act + exp_act_bias.
+ *   act is the tensor in front of the dropout; drop_mask may be null.  M <= 256, O <= 16, F a multiple of 64.
+ * Both need every workgroup resident (NITI_ERR_UNSUPPORTED otherwise) and zeroed sync words
+ * (niti_head_i8_sync_words(backward, ...), 0 = shape not covered): word 0 range (backward: of the data gradient),
+ * word 1 time-out flag, word 2 (backward) range of the weight gradient.  Rounding NITI_ROUND_NEAREST or
+ * NITI_ROUND_PSEUDO_STOCHASTIC.
+ */
+size_t niti_head_i8_sync_words(int backward, int M, int O, int F);
+int niti_head_i8_forward(const int8_t* act, const int8_t* w, int8_t* out8, int M, int O, int F, int dropout, int8_t* drop_mask,
+                         uint32_t* rng, int exp_bias, const int64_t* target, const int32_t* loss_rand, int8_t* loss_grad,
+                         int target_bits, int method, int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync,
+                         size_t sync_words, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                         void* stream);
+int niti_head_i8_backward(const int8_t* err, const int8_t* act, const int8_t* drop_mask, int8_t* w, int8_t* dx8, int M, int O,
+                          int F, int err_bits, int err_method, int grad_bits, int grad_method, int div_mode, int bw_mode,
+                          uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out, int32_t* grad_shift_out,
+                          const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act, int exp_act_bias,
+                          int32_t* err_exp_out, int32_t* grad_exp_out, void* stream);
+
+/*
  * Grouped int8 convolution with float32 output, replaces int8conv_cuda.group_conv
  * (pytorch/int8conv-extension/int8conv.cpp:35-44, int8conv_kernel.cu:248-334):
  * x: [N,H,W,G*Cg] int8, w: [K,R,S,Cg] int8 (K % G == 0, filter k belongs to group k/(K/G)),

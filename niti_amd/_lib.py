@@ -72,6 +72,13 @@ SIGNATURES = {
     "niti_linear_i8_dgrad_requant": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp]),
     "niti_linear_i8_wgrad_update": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "niti_loss_grad_i8": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "niti_loss_grad_i8_rng": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _vp]),
+    "niti_rng_words_u32": (_i, [_vp, _u, _vp, _sz, _vp]),
+    "niti_head_i8_sync_words": (_sz, [_i] * 4),
+    "niti_head_i8_forward": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _i, _i, _i, _i, _u, _vp, _sz,
+                                  _vp, _vp, _vp, _vp, _vp]),
+    "niti_head_i8_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp,
+                                   _vp, _vp, _vp, _i, _vp, _vp, _vp]),
     "niti_mfma_probe_i8": (_i, [_vp, _sz, _i, _i, _vp, _vp, _vp]),
     "niti_group_conv_i8_f32": (_i, [_vp, _vp, _vp] + [_i] * 12 + [_vp]),
 }

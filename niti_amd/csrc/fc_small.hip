@@ -9,11 +9,18 @@
 //   wgrad     g[o][f]  = sum_m err[m][o] act[m][f]  -> grad_calc -> w = clip(w - g): a lane owns 4 consecutive f,
 //             the four wavefronts of a workgroup each take a quarter of the samples (four at a time through
 //             v_dot4_i32_i8 after a 4 x 4 byte transposition) and are added through LDS.
-// All three keep their int32 sums in registers across the tensor-wide range: every workgroup publishes its
+// The classifier at the end of a network (ti_vgg.py:37-40: TiFlat, TiDropout, TiLinear; then TiLoss) takes two launches
+// of the same code: the forward kernel can also apply the dropout mask to the activations it reads (drawing the mask
+// itself) and, when the targets are known, evaluate the loss gradient of the logits it has just rounded (a tile's 16
+// samples are complete in its workgroup); fc_head_bwd_kernel does data gradient, dropout backward, weight gradient
+// and weight update for a slab of 64 input features per workgroup.
+// All of them keep their int32 sums in registers across the tensor-wide range: every workgroup publishes its
 // largest magnitude in a slot of its own and reads all slots (all workgroups resident - checked by the host - and
 // the wait bounded by a wall-clock limit), as the convolution kernels do.
 #include "common.h"
+#include "loss_math.h"
 #include "requant_math.h"
+#include "rng.h"
 
 namespace niti {
 namespace {
@@ -38,6 +45,14 @@ struct FcArgs {
   const int32_t* exp_a;
   const int32_t* exp_b;
   int32_t* exp_out;
+  // classifier head, forward only
+  int dropout;               // 0 none, 1 mask given, 2 mask drawn from rng and written to mask
+  int8_t* mask;              // [F] 0 / 1 per input feature
+  uint32_t* rng;             // generator state (rng.h)
+  int exp_bias;              // added to the output exponent (the dropout's + 1)
+  const int64_t* target;     // [M] or null: with it the loss gradient of the rounded logits is written as well
+  const int32_t* loss_rand;  // [M][O] low four bits used, or null (then drawn from rng)
+  int8_t* loss_grad;         // [M][O]
 };
 
 __device__ inline int round_to_i8(int x, int shift, bool psto, bool trunc) {
@@ -49,7 +64,7 @@ __device__ inline void write_scalars(const FcArgs& a, uint32_t gmax, int shift) 
   const int sh = shift > 0 ? shift : 0;
   a.sync[0] = gmax;
   if (a.shift_out != nullptr) *a.shift_out = sh;
-  if (a.exp_out != nullptr) *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+  if (a.exp_out != nullptr) *a.exp_out = sh + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0) + a.exp_bias;
 }
 
 // Called by wavefront 0 of every workgroup with the workgroup's largest magnitude: returns the largest over the grid.
@@ -64,11 +79,42 @@ __device__ inline uint32_t exchange_range(const FcArgs& a, uint32_t bmax) {
 
 // ---- forward ------------------------------------------------------------------------------------------
 // One workgroup of 16 wavefronts per tile of 16 samples; wavefront w reduces over features [w * kchunk, (w+1) * kchunk).
+// kHead: dropout on the activations (mask bytes 0x00 / 0xFF in dynamic LDS, F bytes) and the loss gradient.
+template <bool kHead>
 __global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
   __shared__ int part[16][256];
+  __shared__ __attribute__((aligned(16))) int8_t logits[16][16];   // kHead: the tile's rounded logits
+  extern __shared__ __attribute__((aligned(16))) unsigned char keep[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int mt = blockIdx.x;
+  const bool drop = kHead && a.dropout != 0;
+  const bool draws = kHead && (a.dropout == 2 || (a.target != nullptr && a.loss_rand == nullptr));
+  RngDraw draw{};
+  if (draws) draw = rng_read(a.rng);
+  if (drop) {
+    for (int k = threadIdx.x * 8; k < a.F; k += 1024 * 8) {   // F is a multiple of 16
+      uint32_t m[2];
+      if (a.dropout == 2) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          uint32_t w4[4];
+          rng_words4(draw, kRngStreamDropout, static_cast<uint32_t>(k / 4 + h), w4);
+          m[h] = (w4[0] & 1u) | ((w4[1] & 1u) << 8) | ((w4[2] & 1u) << 16) | ((w4[3] & 1u) << 24);
+        }
+        if (mt == 0) {
+          *reinterpret_cast<uint32_t*>(a.mask + k) = m[0];
+          *reinterpret_cast<uint32_t*>(a.mask + k + 4) = m[1];
+        }
+      } else {
+        m[0] = *reinterpret_cast<const uint32_t*>(a.mask + k);
+        m[1] = *reinterpret_cast<const uint32_t*>(a.mask + k + 4);
+      }
+      *reinterpret_cast<uint32_t*>(keep + k) = m[0] * 255u;      // bytes 0 / 1 -> 0x00 / 0xFF
+      *reinterpret_cast<uint32_t*>(keep + k + 4) = m[1] * 255u;
+    }
+    __syncthreads();
+  }
   const int row = lane & 15, kg = lane >> 4;           // operand row (sample / output feature), 16-byte piece of a 64-step
   const int m = mt * 16 + row;
   const int k0 = wave * a.kchunk;
@@ -86,6 +132,7 @@ __global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
       const bool in = k < k1;                             // F is a multiple of 16: a piece is inside or outside
       fa[u] = (va && in) ? *reinterpret_cast<const v4i*>(pa + k) : zero;
       fw[u] = (vw && in) ? *reinterpret_cast<const v4i*>(pw + k) : zero;
+      if (drop && in) fa[u] &= *reinterpret_cast<const v4i*>(keep + k);
     }
 #pragma unroll
     for (int u = 0; u < 4; ++u) acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[u], fw[u], acc, 0, 0, 0);
@@ -113,13 +160,63 @@ __global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int mm = mt * 16 + 4 * (lane >> 4) + i;
+      int r = 0;
       if (mm < a.M && o < a.O) {
-        int r = round_to_i8(acc[i], shift, psto, trunc);
+        r = round_to_i8(acc[i], shift, psto, trunc);
         if (relu && r < 0) r = 0;
         a.out8[static_cast<long long>(mm) * a.O + o] = static_cast<int8_t>(r);
       }
+      if (kHead) logits[4 * (lane >> 4) + i][o] = static_cast<int8_t>(r);
+    }
+    if (kHead && lane == 0) part[0][0] = (shift > 0 ? shift : 0) + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0) + a.exp_bias;
+  }
+  if (!kHead) return;
+  if (a.target != nullptr) {
+    // ti_loss.py:5-36 for the tile's samples: sixteen lanes per sample (one per class), four samples per wavefront
+    __syncthreads();
+    if (wave < 4) {
+      const int e = part[0][0];
+      const int srow = wave * 4 + (lane >> 4), j = lane & 15;
+      const int row = mt * 16 + srow;
+      const bool valid = row < a.M && j < a.O;
+      const int v = logits[srow][j];
+      const bool big = e > -7, up = e >= 0;
+      const float p2 = exp2f(static_cast<float>(up ? e : -e));   // exact power of two
+      auto group_sum = [](long long x) {
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) {
+          const int lo = __shfl_xor(static_cast<int>(x & 0xFFFFFFFFLL), off, 64);
+          const int hi = __shfl_xor(static_cast<int>(x >> 32), off, 64);
+          x += (static_cast<long long>(hi) << 32) | static_cast<unsigned int>(lo);
+        }
+        return x;
+      };
+      float nm;             // out_grad before the normalisation, as float32
+      long long term;       // its truncation (ti_loss.py:31)
+      if (big) {
+        const float sc = scaled_logit(v, p2, up);
+        float mx = valid ? sc : -INFINITY;
+#pragma unroll
+        for (int off = 8; off > 0; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off, 64));
+        nm = exp2_contract(fmaxf(sc - (mx - 10.0f), 0.0f)) - 1.0f;
+        term = static_cast<long long>(nm);
+      } else {
+        term = loss_small_term(v, e);
+        nm = static_cast<float>(term);
+      }
+      const float fsum = static_cast<float>(group_sum(valid ? term : 0LL));
+      float g = nm * 2048.0f / fsum;
+      const long long tsum = group_sum(valid ? static_cast<long long>(g) : 0LL);   // ti_loss.py:34
+      if (valid) {
+        if (j == a.target[row]) g = g - static_cast<float>(tsum);
+        const int x = static_cast<int>(g);   // .type(torch.int32)
+        const long long idx = static_cast<long long>(row) * a.O + j;
+        const int u = a.loss_rand != nullptr ? a.loss_rand[idx] & 15 : static_cast<int>(rng_word(draw, kRngStreamLoss, static_cast<uint32_t>(idx)) & 15u);
+        a.loss_grad[idx] = static_cast<int8_t>(round_one<NITI_ROUND_STOCHASTIC>(x, 4, a.trunc != 0, u));
+      }
     }
   }
+  if (draws && threadIdx.x == 0) rng_arrive(a.rng, gridDim.x, draw);
 }
 
 // ---- data gradient ------------------------------------------------------------------------------------
@@ -312,6 +409,256 @@ __global__ __launch_bounds__(256) void fc_wgrad_update_kernel(const FcArgs a) {
   }
 }
 
+// ---- classifier head, backward: data gradient + dropout backward + weight gradient + update -----------------------
+// ti_torch.py:255-266 followed by ti_torch.py:452-455 in one launch.  A workgroup owns a slab of 64 input features:
+// it stages the error rows (all samples, 16 bytes each), the slab of the weights as stored and the slab of the
+// activations with the dropout mask applied (what the forward pass multiplied), then
+//   dx[m][f] = sum_o err[m][o] w[o][f]   sixteen wavefronts x 16 samples, four MFMAs each,
+//   g[o][f]  = sum_m err[m][o] act[m][f] four wavefronts x 16 features, an MFMA per 64 samples,
+// (v_mfma_i32_16x16x64_i8; weights and activations are transposed on their way into LDS),
+// exchanges both ranges, rounds, masks and stores dx, and applies w = clip(w - g) to its slab.
+constexpr int kHeadSlab = 64;
+constexpr int kHeadMaxM = 256;     // a lane holds four samples x 16 features of the data gradient
+
+struct HeadBwdArgs {
+  const int8_t* err;    // [M][O]
+  const int8_t* act;    // [M][F], before the dropout
+  const int8_t* mask;   // [F] 0 / 1, or null
+  int8_t* w;            // [O][F], updated in place
+  int8_t* dx8;          // [M][F]
+  int8_t* g8;           // [O][F] rounded gradient, or null
+  uint32_t* sync;       // 0 data-gradient range, 1 wait gave up, 2 weight-gradient range, kSlot0.. a slot of two words per workgroup
+  int M, O, F;
+  int err_bits, err_method, grad_bits, grad_method, trunc, bw_mode;
+  long long spin_limit;
+  uint32_t* sticky;
+  int32_t* err_shift_out;
+  int32_t* grad_shift_out;
+  const int32_t* exp_err;
+  const int32_t* exp_w;
+  const int32_t* exp_act;
+  int exp_act_bias;
+  int32_t* err_exp_out;
+  int32_t* grad_exp_out;
+};
+
+__device__ inline int byte_of(uint32_t w, int b) { return static_cast<int>(static_cast<int8_t>((w >> (8 * b)) & 0xFFu)); }
+
+// 4 x 4 byte transposition: in[j] holds bytes 0..3 of row j; out[b] holds byte b of rows 0..3
+__device__ inline void transpose4x4_bytes(const uint32_t (&in)[4], uint32_t (&out)[4]) {
+  const uint32_t lo01 = __builtin_amdgcn_perm(in[1], in[0], 0x05010400u), hi01 = __builtin_amdgcn_perm(in[1], in[0], 0x07030602u);
+  const uint32_t lo23 = __builtin_amdgcn_perm(in[3], in[2], 0x05010400u), hi23 = __builtin_amdgcn_perm(in[3], in[2], 0x07030602u);
+  out[0] = __builtin_amdgcn_perm(lo23, lo01, 0x05040100u);
+  out[1] = __builtin_amdgcn_perm(lo23, lo01, 0x07060302u);
+  out[2] = __builtin_amdgcn_perm(hi23, hi01, 0x05040100u);
+  out[3] = __builtin_amdgcn_perm(hi23, hi01, 0x07060302u);
+}
+
+constexpr int kHeadGroups = kHeadMaxM / 4;     // groups of four samples
+constexpr int kHeadActPitch = kHeadGroups + 4; // words per feature row of the transposed activations (16-byte rows, banks spread)
+
+// wait_slots for slots that hold two values: workgroup b stores (data-gradient maximum + 1) | (weight-gradient
+// maximum + 1) << 32 as one 8-byte word at slot b.  Called by a whole wavefront; nb <= 4096.
+__device__ inline void wait_slot_pairs(uint32_t* slots, int nb, long long spin_limit, uint32_t* timed_out, uint32_t* sticky,
+                                       uint32_t& max_lo, uint32_t& max_hi) {
+  const int lane = threadIdx.x & 63;
+  const long long t0 = wall_clock64();
+  uint32_t glo = 0, ghi = 0;
+  bool gave_up = false;
+  for (int base = 0; base < nb && !gave_up; base += 64) {
+    unsigned long long v = base + lane < nb ? 0ULL : 1ULL;
+    for (;;) {
+      if (v == 0ULL)
+        v = __hip_atomic_load(reinterpret_cast<unsigned long long*>(slot_word(slots, base + lane)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (__all(v != 0ULL)) break;
+      if (wall_clock64() - t0 > spin_limit) {
+        if (lane == 0) {
+          __hip_atomic_store(timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (sticky != nullptr) __hip_atomic_store(sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        gave_up = true;
+        break;
+      }
+      __builtin_amdgcn_s_sleep(4);
+    }
+    if (base + lane < nb) {
+      const uint32_t lo = static_cast<uint32_t>(v), hi = static_cast<uint32_t>(v >> 32);
+      glo = lo > glo ? lo : glo;
+      ghi = hi > ghi ? hi : ghi;
+    }
+  }
+  max_lo = wave_max_u32(glo);
+  max_hi = wave_max_u32(ghi);
+}
+
+__global__ __launch_bounds__(1024) void fc_head_bwd_kernel(const HeadBwdArgs a) {
+  // both products run on v_mfma_i32_16x16x64_i8, whose operands are rows with the reduction index in consecutive bytes
+  __shared__ __attribute__((aligned(16))) uint32_t err_s[kHeadMaxM * 4];               // [m][o]: 16 bytes per sample
+  __shared__ __attribute__((aligned(16))) uint32_t err_t[kMaxOut * kHeadGroups];       // [o][m]
+  __shared__ __attribute__((aligned(16))) uint32_t act_t[kHeadSlab * kHeadActPitch];   // [f][m], masked
+  __shared__ __attribute__((aligned(16))) uint32_t w_t[kHeadSlab * 4];                 // [f][o]: 16 bytes per input feature
+  __shared__ __attribute__((aligned(16))) uint32_t keep_s[kHeadSlab / 4];              // dropout mask of the slab as 0x00 / 0xFF bytes
+  __shared__ uint32_t wmax_d[16], wmax_w[16], gshare[2];
+  const int t = threadIdx.x, lane = t & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+  const int f0 = blockIdx.x * kHeadSlab;
+  const v4i zero = {0, 0, 0, 0};
+  if (t < 256) {
+    const int piece = t & 3, mgroup = t >> 2;     // 16-byte piece of the slab, group of four samples
+    v4i mk = {-1, -1, -1, -1};
+    if (a.mask != nullptr) {
+      const v4i m = *reinterpret_cast<const v4i*>(a.mask + f0 + piece * 16);
+#pragma unroll
+      for (int d = 0; d < 4; ++d) mk[d] = static_cast<int>(static_cast<uint32_t>(m[d]) * 255u);   // bytes 0 / 1 -> 0x00 / 0xFF
+    }
+    v4i av[4];      // samples 4 mgroup .. + 3, features f0 + 16 piece .. + 15
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int m = 4 * mgroup + j;
+      av[j] = m < a.M ? *reinterpret_cast<const v4i*>(a.act + static_cast<long long>(m) * a.F + f0 + piece * 16) : zero;
+    }
+    uint32_t win[4] = {0u, 0u, 0u, 0u};
+    if (t < 64) {   // weights: output features 4 (t / 16) .. + 3, input features f0 + 4 (t % 16) .. + 3
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        win[j] = 4 * (t >> 4) + j < a.O ? *reinterpret_cast<const uint32_t*>(a.w + static_cast<long long>(4 * (t >> 4) + j) * a.F + f0 + 4 * (t & 15)) : 0u;
+    }
+    uint32_t eb[kMaxOut];   // error row of sample t, all loads in flight together
+#pragma unroll
+    for (int o = 0; o < kMaxOut; ++o)
+      eb[o] = (t < a.M && o < a.O) ? static_cast<uint32_t>(a.err[static_cast<long long>(t) * a.O + o]) & 0xFFu : 0u;
+    if (t < 4) *reinterpret_cast<v4i*>(keep_s + 4 * t) = mk;
+    if (t < 64) {
+      uint32_t out[4];
+      transpose4x4_bytes(win, out);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) w_t[(4 * (t & 15) + b) * 4 + (t >> 4)] = out[b];
+    }
+    uint32_t wd[4] = {0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int o = 0; o < kMaxOut; ++o) wd[o >> 2] |= eb[o] << (8 * (o & 3));
+    *reinterpret_cast<v4i*>(err_s + t * 4) = v4i{static_cast<int>(wd[0]), static_cast<int>(wd[1]), static_cast<int>(wd[2]), static_cast<int>(wd[3])};
+#pragma unroll
+    for (int d = 0; d < 4; ++d) {   // activations, masked, transposed: word d of the four rows -> features 4 d .. 4 d + 3
+      const uint32_t in[4] = {static_cast<uint32_t>(av[0][d] & mk[d]), static_cast<uint32_t>(av[1][d] & mk[d]),
+                              static_cast<uint32_t>(av[2][d] & mk[d]), static_cast<uint32_t>(av[3][d] & mk[d])};
+      uint32_t out[4];
+      transpose4x4_bytes(in, out);
+#pragma unroll
+      for (int b = 0; b < 4; ++b) act_t[(16 * piece + 4 * d + b) * kHeadActPitch + mgroup] = out[b];
+    }
+  }
+  __syncthreads();
+  {               // err_t[o][g] from err_s: one word per thread (16 output features x 64 groups)
+    const int o = t >> 6, g = t & 63;
+    uint32_t word = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) word |= ((err_s[(4 * g + j) * 4 + (o >> 2)] >> (8 * (o & 3))) & 0xFFu) << (8 * j);
+    err_t[o * kHeadGroups + g] = word;
+  }
+  // data gradient: wavefront w takes samples 16 w .. + 15; per block of 16 features one MFMA whose reduction (the
+  // output features) fills the first quarter of its 64 steps.  dacc[blk][i]: feature 16 blk + 4 (lane / 16) + i of
+  // sample 16 w + lane % 16
+  const int row = lane & 15, kg = lane >> 4;
+  v4i dacc[4];
+  {
+    const v4i eop = kg == 0 ? *reinterpret_cast<const v4i*>(err_s + (16 * wave + row) * 4) : zero;
+#pragma unroll
+    for (int blk = 0; blk < 4; ++blk) {
+      const v4i wop = kg == 0 ? *reinterpret_cast<const v4i*>(w_t + (16 * blk + row) * 4) : zero;
+      dacc[blk] = __builtin_amdgcn_mfma_i32_16x16x64_i8(wop, eop, zero, 0, 0, 0);
+    }
+  }
+  __syncthreads();   // err_t is complete
+  // weight gradient: wavefront w < 4 takes features 16 w .. + 15, 64 samples per MFMA.  gacc[i]: output feature
+  // 4 (lane / 16) + i, feature 16 w + lane % 16
+  v4i gacc = zero;
+  if (wave < 4) {
+    const int steps = (a.M + 63) >> 6;
+    for (int ks = 0; ks < steps; ++ks) {
+      const v4i eop = *reinterpret_cast<const v4i*>(err_t + row * kHeadGroups + ks * 16 + kg * 4);
+      const v4i aop = *reinterpret_cast<const v4i*>(act_t + (16 * wave + row) * kHeadActPitch + ks * 16 + kg * 4);
+      gacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(eop, aop, gacc, 0, 0, 0);
+    }
+  }
+  uint32_t dmax = 0, gmaxl = 0;
+#pragma unroll
+  for (int blk = 0; blk < 4; ++blk)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t u = uabs(dacc[blk][i]);     // rows beyond M are sums of zeros
+      dmax = u > dmax ? u : dmax;
+    }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const uint32_t u = uabs(gacc[i]);
+    gmaxl = u > gmaxl ? u : gmaxl;
+  }
+  dmax = wave_max_u32(dmax);
+  gmaxl = wave_max_u32(gmaxl);
+  if (lane == 0) {
+    wmax_d[wave] = dmax;
+    wmax_w[wave] = gmaxl;
+  }
+  __syncthreads();
+  if (wave == 0) {
+    const uint32_t bd = wave_max_u32(lane < 16 ? wmax_d[lane] : 0u);
+    const uint32_t bw = wave_max_u32(lane < 16 ? wmax_w[lane] : 0u);
+    uint32_t* const slots = a.sync + kSlot0;
+    if (lane == 0)
+      __hip_atomic_store(reinterpret_cast<unsigned long long*>(slot_word(slots, blockIdx.x)),
+                         static_cast<unsigned long long>(bd + 1u) | (static_cast<unsigned long long>(bw + 1u) << 32), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    uint32_t gd = 0, gw = 0;
+    wait_slot_pairs(slots, gridDim.x, a.spin_limit, &a.sync[1], a.sticky, gd, gw);
+    if (lane == 0) {
+      gshare[0] = gd != 0u ? gd - 1u : 0u;
+      gshare[1] = gw != 0u ? gw - 1u : 0u;
+    }
+  }
+  __syncthreads();
+  const uint32_t range_d = gshare[0], range_w = gshare[1];
+  const int shift_d = bitwidth_of(range_d, a.bw_mode) - a.err_bits;
+  const int shift_w = bitwidth_of(range_w, a.bw_mode) - a.grad_bits;
+  if (blockIdx.x == 0 && t == 0) {
+    const int sd = shift_d > 0 ? shift_d : 0, sw = shift_w > 0 ? shift_w : 0;
+    a.sync[0] = range_d;
+    a.sync[2] = range_w;
+    const int e_err = sd + (a.exp_err != nullptr ? *a.exp_err : 0) + (a.exp_w != nullptr ? *a.exp_w : 0);   // ti_torch.py:260
+    if (a.err_shift_out != nullptr) *a.err_shift_out = sd;
+    if (a.grad_shift_out != nullptr) *a.grad_shift_out = sw;
+    if (a.err_exp_out != nullptr) *a.err_exp_out = e_err;
+    if (a.grad_exp_out != nullptr) *a.grad_exp_out = sw + e_err + (a.exp_act != nullptr ? *a.exp_act : 0) + a.exp_act_bias;   // ti_torch.py:18
+  }
+  const bool trunc = a.trunc != 0;
+  const bool psto_d = a.err_method == NITI_ROUND_PSEUDO_STOCHASTIC, psto_w = a.grad_method == NITI_ROUND_PSEUDO_STOCHASTIC;
+  {
+    const int m = 16 * wave + row;
+    if (m < a.M) {
+#pragma unroll
+      for (int blk = 0; blk < 4; ++blk) {
+        const uint32_t r4 = pack4_i8(round_to_i8(dacc[blk][0], shift_d, psto_d, trunc), round_to_i8(dacc[blk][1], shift_d, psto_d, trunc),
+                                     round_to_i8(dacc[blk][2], shift_d, psto_d, trunc), round_to_i8(dacc[blk][3], shift_d, psto_d, trunc));
+        *reinterpret_cast<uint32_t*>(a.dx8 + static_cast<long long>(m) * a.F + f0 + 16 * blk + 4 * kg) = r4 & keep_s[4 * blk + kg];   // ti_torch.py:454
+      }
+    }
+  }
+  if (wave < 4) {
+    const int f = 16 * wave + row;
+    const uint32_t wold = w_t[f * 4 + kg];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int o = 4 * kg + i;
+      if (o < a.O) {
+        const int r = round_to_i8(gacc[i], shift_w, psto_w, trunc);
+        const long long at = static_cast<long long>(o) * a.F + f0 + f;
+        a.w[at] = static_cast<int8_t>(clip127(byte_of(wold, i) - r));
+        if (a.g8 != nullptr) a.g8[at] = static_cast<int8_t>(r);
+      }
+    }
+  }
+}
+
 int resident_blocks(const void* kernel, int threads = 256) {
   int dev = 0, cus = 0, per_cu = 0;
   if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
@@ -403,10 +750,10 @@ extern "C" int niti_fc_i8_fwd_requant(const int8_t* act, const int8_t* w, int8_t
   a.rq_flags = rq_flags;
   static int resident_of[kDeviceSlots] = {};
   int& resident = resident_of[device_slot()];
-  if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_fwd_requant_kernel), 1024);
+  if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_fwd_requant_kernel<false>), 1024);
   if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "fc_fwd_requant: %lld workgroups do not fit on the device at once (%d)", nb, resident);
   a.kchunk = fwd_chunk(F);
-  hipLaunchKernelGGL(fc_fwd_requant_kernel, dim3(static_cast<unsigned>(nb)), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
+  hipLaunchKernelGGL(fc_fwd_requant_kernel<false>, dim3(static_cast<unsigned>(nb)), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
   return check_launch("fc_fwd_requant");
 }
 
@@ -454,4 +801,123 @@ extern "C" int niti_fc_i8_wgrad_update(const int8_t* err, const int8_t* act, int
   a.out8 = g8_out;
   hipLaunchKernelGGL(fc_wgrad_update_kernel, dim3(static_cast<unsigned>(nb)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
   return check_launch("fc_wgrad_update");
+}
+
+// ---- classifier head ------------------------------------------------------------------------------------------
+static long long head_bwd_blocks(int M, int O, int F) {
+  if (M <= 0 || O <= 0 || F <= 0 || O > kMaxOut || M > kHeadMaxM || F % kHeadSlab != 0) return 0;
+  const long long nb = F / kHeadSlab;
+  return nb <= 4096 ? nb : 0;
+}
+
+extern "C" size_t niti_head_i8_sync_words(int backward, int M, int O, int F) {
+  if (!backward) return niti_fc_i8_sync_words(NITI_FC_FORWARD, M, O, F);
+  const long long nb = head_bwd_blocks(M, O, F);
+  if (nb == 0) return 0;
+  return static_cast<size_t>(kSlot0) + slot_words(static_cast<int>(nb));
+}
+
+extern "C" int niti_head_i8_forward(const int8_t* act, const int8_t* w, int8_t* out8, int M, int O, int F, int dropout,
+                                    int8_t* drop_mask, uint32_t* rng, int exp_bias, const int64_t* target, const int32_t* loss_rand,
+                                    int8_t* loss_grad, int target_bits, int method, int div_mode, int bw_mode, unsigned rq_flags,
+                                    uint32_t* sync, size_t sync_words, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b,
+                                    int32_t* exp_out, void* stream) {
+  FcArgs a{};
+  long long nb = 0;
+  const int st = fc_common("head_forward", NITI_FC_FORWARD, a, M, O, F, target_bits, method, div_mode, bw_mode, sync, sync_words,
+                           shift_out, exp_a, exp_b, exp_out, &nb);
+  if (st != NITI_OK) return st;
+  if (act == nullptr || w == nullptr || out8 == nullptr) return fail(NITI_ERR_INVALID_ARG, "head_forward: null pointer");
+  if (!aligned16(act) || !aligned16(w)) return fail(NITI_ERR_INVALID_ARG, "head_forward: operands must be 16-byte aligned");
+  if (dropout < 0 || dropout > 2) return fail(NITI_ERR_INVALID_ARG, "head_forward: dropout=%d (0 none, 1 mask given, 2 mask drawn)", dropout);
+  if (dropout != 0 && (drop_mask == nullptr || reinterpret_cast<uintptr_t>(drop_mask) % 4 != 0))
+    return fail(NITI_ERR_INVALID_ARG, "head_forward: the dropout mask must be a 4-byte aligned array of F bytes");
+  if (dropout != 0 && F > 32768) return fail(NITI_ERR_UNSUPPORTED, "head_forward: dropout over more than 32768 features");
+  if (target != nullptr && loss_grad == nullptr) return fail(NITI_ERR_INVALID_ARG, "head_forward: targets without a place for the loss gradient");
+  if ((dropout == 2 || (target != nullptr && loss_rand == nullptr)) && rng == nullptr)
+    return fail(NITI_ERR_INVALID_ARG, "head_forward: random draws asked for without a generator state");
+  if (static_cast<long long>(M) * O > 0x7FFFFFFFLL) return fail(NITI_ERR_UNSUPPORTED, "head_forward: more than 2^31 logits");
+  a.act = act;
+  a.w = const_cast<int8_t*>(w);
+  a.out8 = out8;
+  a.rq_flags = rq_flags;
+  a.dropout = dropout;
+  a.mask = drop_mask;
+  a.rng = rng;
+  a.exp_bias = exp_bias;
+  a.target = target;
+  a.loss_rand = loss_rand;
+  a.loss_grad = loss_grad;
+  const size_t lds = dropout != 0 ? static_cast<size_t>(F) : 0;
+  static int resident_of[kDeviceSlots] = {};
+  int& resident = resident_of[device_slot()];
+  if (resident == 0) {
+    // counted with the largest mask the kernel takes, so the answer holds for every call
+    int dev = 0, cus = 0, per_cu = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, reinterpret_cast<const void*>(fc_fwd_requant_kernel<true>), 1024, 32768) == hipSuccess)
+      resident = cus * per_cu;
+  }
+  if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "head_forward: %lld workgroups do not fit on the device at once (%d)", nb, resident);
+  a.kchunk = fwd_chunk(F);
+  hipLaunchKernelGGL(fc_fwd_requant_kernel<true>, dim3(static_cast<unsigned>(nb)), dim3(1024), lds, static_cast<hipStream_t>(stream), a);
+  return check_launch("head_forward");
+}
+
+extern "C" int niti_head_i8_backward(const int8_t* err, const int8_t* act, const int8_t* drop_mask, int8_t* w, int8_t* dx8, int M, int O,
+                                     int F, int err_bits, int err_method, int grad_bits, int grad_method, int div_mode, int bw_mode,
+                                     uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out, int32_t* grad_shift_out,
+                                     const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act, int exp_act_bias,
+                                     int32_t* err_exp_out, int32_t* grad_exp_out, void* stream) {
+  clear_error();
+  if (M <= 0 || O <= 0 || F <= 0) return fail(NITI_ERR_INVALID_ARG, "head_backward: non-positive extent");
+  if (err == nullptr || act == nullptr || w == nullptr || dx8 == nullptr || sync == nullptr) return fail(NITI_ERR_INVALID_ARG, "head_backward: null pointer");
+  if (err_bits < 1 || err_bits > 7 || grad_bits < 1 || grad_bits > 7)
+    return fail(NITI_ERR_INVALID_ARG, "head_backward: err_bits=%d grad_bits=%d outside 1..7", err_bits, grad_bits);
+  for (const int method : {err_method, grad_method})
+    if (method != NITI_ROUND_NEAREST && method != NITI_ROUND_PSEUDO_STOCHASTIC)
+      return fail(NITI_ERR_UNSUPPORTED, "head_backward: rounding method %d needs random input; use the separate passes", method);
+  if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "head_backward: div_mode=%d", div_mode);
+  if (bw_mode != NITI_BW_INT && bw_mode != NITI_BW_F32) return fail(NITI_ERR_INVALID_ARG, "head_backward: bw_mode=%d", bw_mode);
+  const long long nb = head_bwd_blocks(M, O, F);
+  if (nb == 0)
+    return fail(NITI_ERR_UNSUPPORTED, "head_backward: M=%d O=%d F=%d outside the kernel (M <= %d, O <= %d, F a multiple of %d); use the separate passes",
+                M, O, F, kHeadMaxM, kMaxOut, kHeadSlab);
+  if (!aligned16(act) || !aligned16(w) || !aligned16(dx8) || (drop_mask != nullptr && !aligned16(drop_mask)))
+    return fail(NITI_ERR_INVALID_ARG, "head_backward: act, w, dx8 and the mask must be 16-byte aligned");
+  const size_t need = niti_head_i8_sync_words(1, M, O, F);
+  if (sync_words < need) return fail(NITI_ERR_WORKSPACE, "head_backward: needs %zu zeroed sync words, got %zu", need, sync_words);
+  static int resident_of[kDeviceSlots] = {};
+  int& resident = resident_of[device_slot()];
+  if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_head_bwd_kernel), 1024);
+  if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "head_backward: %lld workgroups do not fit on the device at once (%d)", nb, resident);
+  HeadBwdArgs a{};
+  a.err = err;
+  a.act = act;
+  a.mask = drop_mask;
+  a.w = w;
+  a.dx8 = dx8;
+  a.g8 = g8_out;
+  a.sync = sync;
+  a.M = M;
+  a.O = O;
+  a.F = F;
+  a.err_bits = err_bits;
+  a.err_method = err_method;
+  a.grad_bits = grad_bits;
+  a.grad_method = grad_method;
+  a.trunc = div_mode == NITI_DIV_TRUNC ? 1 : 0;
+  a.bw_mode = bw_mode;
+  a.spin_limit = sync_spin_limit();
+  a.sticky = timeout_word();
+  a.err_shift_out = err_shift_out;
+  a.grad_shift_out = grad_shift_out;
+  a.exp_err = exp_err;
+  a.exp_w = exp_w;
+  a.exp_act = exp_act;
+  a.exp_act_bias = exp_act_bias;
+  a.err_exp_out = err_exp_out;
+  a.grad_exp_out = grad_exp_out;
+  hipLaunchKernelGGL(fc_head_bwd_kernel, dim3(static_cast<unsigned>(nb)), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
+  return check_launch("head_backward");
 }

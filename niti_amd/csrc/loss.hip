@@ -7,7 +7,9 @@
 // 2 ** s, is evaluated by a fixed sequence of IEEE double operations (exp2_contract below) that a host can
 // repeat bit for bit, so the whole gradient is reproducible across devices.
 #include "common.h"
+#include "loss_math.h"
 #include "requant_math.h"
+#include "rng.h"
 
 namespace niti {
 namespace {
@@ -16,40 +18,11 @@ struct LossArgs {
   const int8_t* out;       // [n][classes] logits
   const int32_t* out_exp;  // exponent of the logits (device scalar)
   const int64_t* target;   // [n]
-  const int32_t* rand;     // [n][classes], low four bits used
+  const int32_t* rand;     // [n][classes], low four bits used; null: drawn from rng
+  uint32_t* rng;           // generator state (rng.h), used when rand is null
   int8_t* grad;            // [n][classes]
   int n, classes, trunc;
 };
-
-// no fused multiply-add: the reference runs every operation as a kernel of its own
-#pragma clang fp contract(off)
-
-// ti_loss.py:10-24 for one logit: 2^max(s - offset, 0) - 1 with s = v * 47274 / 2^15 * 2^e
-__device__ inline float scaled_logit(int v, float p2, bool up) {
-  const float s = static_cast<float>(static_cast<long long>(v) * 47274) / 32768.0f;
-  return up ? s * p2 : s / p2;
-}
-
-// 2^s for s >= 0: n = floor(s), x = (s - n) ln2, Horner's rule over 1/k! (k = 18 .. 0) in doubles with one rounded
-// product and one rounded sum per step (no fused multiply-add), result = float(p 2^n).  Truncation error < 2^-60, so
-// this is the correctly rounded float32 power except within ~2^-52 (relative) of a rounding boundary.
-__device__ inline float exp2_contract(float s) {
-  constexpr double c[19] = {
-      0x1.0000000000000p+0,  0x1.0000000000000p+0,  0x1.0000000000000p-1,  0x1.5555555555555p-3,  0x1.5555555555555p-5,
-      0x1.1111111111111p-7,  0x1.6c16c16c16c17p-10, 0x1.a01a01a01a01ap-13, 0x1.a01a01a01a01ap-16, 0x1.71de3a556c734p-19,
-      0x1.27e4fb7789f5cp-22, 0x1.ae64567f544e4p-26, 0x1.1eed8eff8d898p-29, 0x1.6124613a86d09p-33, 0x1.93974a8c07c9dp-37,
-      0x1.ae7f3e733b81fp-41, 0x1.ae7f3e733b81fp-45, 0x1.952c77030ad4ap-49, 0x1.6827863b97d97p-53};
-  const double d = static_cast<double>(s);
-  const double n = floor(d);
-  const double x = (d - n) * 0x1.62e42fefa39efp-1;   // contraction is off for this file (pragma above)
-  double p = c[18];
-#pragma unroll
-  for (int k = 17; k >= 0; --k) {
-    p = p * x;
-    p = p + c[k];
-  }
-  return static_cast<float>(ldexp(p, static_cast<int>(n)));
-}
 
 __device__ inline long long wave_sum_i64(long long v) {
 #pragma unroll
@@ -67,6 +40,8 @@ __global__ __launch_bounds__(256) void loss_grad_kernel(const LossArgs a) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= a.n) return;
+  RngDraw draw{};
+  if (a.rand == nullptr) draw = rng_read(a.rng);
   const int8_t* v = a.out + static_cast<long long>(row) * a.classes;
   const int e = *a.out_exp;
   const bool big = e > -7;
@@ -105,8 +80,10 @@ __global__ __launch_bounds__(256) void loss_grad_kernel(const LossArgs a) {
     if (j == t) g = g - static_cast<float>(tsum);
     const int x = static_cast<int>(g);   // .type(torch.int32)
     const long long idx = static_cast<long long>(row) * a.classes + j;
-    a.grad[idx] = static_cast<int8_t>(round_one<NITI_ROUND_STOCHASTIC>(x, 4, trunc, a.rand[idx] & 15));
+    const int u = a.rand != nullptr ? a.rand[idx] & 15 : static_cast<int>(rng_word(draw, kRngStreamLoss, static_cast<uint32_t>(idx)) & 15u);
+    a.grad[idx] = static_cast<int8_t>(round_one<NITI_ROUND_STOCHASTIC>(x, 4, trunc, u));
   }
+  if (a.rand == nullptr && threadIdx.x == 0) rng_arrive(a.rng, gridDim.x, draw);   // the first row of a workgroup always exists
 }
 
 }  // namespace
@@ -114,14 +91,60 @@ __global__ __launch_bounds__(256) void loss_grad_kernel(const LossArgs a) {
 
 using namespace niti;
 
-extern "C" int niti_loss_grad_i8(const int8_t* out_val, const int32_t* out_exp, const int64_t* target, const int32_t* rand,
-                                 int8_t* grad, int n, int classes, int div_mode, void* stream) {
+static int loss_launch(const int8_t* out_val, const int32_t* out_exp, const int64_t* target, const int32_t* rand, uint32_t* rng,
+                       int8_t* grad, int n, int classes, int div_mode, void* stream) {
   clear_error();
-  if (out_val == nullptr || out_exp == nullptr || target == nullptr || rand == nullptr || grad == nullptr)
+  if (out_val == nullptr || out_exp == nullptr || target == nullptr || (rand == nullptr && rng == nullptr) || grad == nullptr)
     return fail(NITI_ERR_INVALID_ARG, "loss_grad: null pointer");
   if (n <= 0 || classes <= 0) return fail(NITI_ERR_INVALID_ARG, "loss_grad: n=%d classes=%d", n, classes);
+  if (static_cast<long long>(n) * classes > 0x7FFFFFFFLL) return fail(NITI_ERR_UNSUPPORTED, "loss_grad: more than 2^31 logits");
   if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "loss_grad: div_mode=%d", div_mode);
-  const LossArgs a{out_val, out_exp, target, rand, grad, n, classes, div_mode == NITI_DIV_TRUNC ? 1 : 0};
+  const LossArgs a{out_val, out_exp, target, rand, rng, grad, n, classes, div_mode == NITI_DIV_TRUNC ? 1 : 0};
   hipLaunchKernelGGL(loss_grad_kernel, dim3((n + 3) / 4), dim3(256), 0, static_cast<hipStream_t>(stream), a);
   return check_launch("loss_grad");
+}
+
+extern "C" int niti_loss_grad_i8(const int8_t* out_val, const int32_t* out_exp, const int64_t* target, const int32_t* rand,
+                                 int8_t* grad, int n, int classes, int div_mode, void* stream) {
+  if (rand == nullptr) {
+    clear_error();
+    return fail(NITI_ERR_INVALID_ARG, "loss_grad: null pointer");
+  }
+  return loss_launch(out_val, out_exp, target, rand, nullptr, grad, n, classes, div_mode, stream);
+}
+
+extern "C" int niti_loss_grad_i8_rng(const int8_t* out_val, const int32_t* out_exp, const int64_t* target, uint32_t* rng,
+                                     int8_t* grad, int n, int classes, int div_mode, void* stream) {
+  if (rng == nullptr) {
+    clear_error();
+    return fail(NITI_ERR_INVALID_ARG, "loss_grad: null pointer");
+  }
+  return loss_launch(out_val, out_exp, target, nullptr, rng, grad, n, classes, div_mode, stream);
+}
+
+// ---- the generator's words, for callers that want to see what a kernel will draw --------------------------------
+namespace niti {
+namespace {
+__global__ __launch_bounds__(256) void rng_words_kernel(const uint32_t* state, uint32_t stream_id, uint32_t* out, long long n) {
+  const RngDraw d = rng_read(state);
+  const long long q = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;   // a lane writes four words
+  if (4 * q >= n) return;
+  uint32_t w[4];
+  rng_words4(d, stream_id, static_cast<uint32_t>(q), w);
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    if (4 * q + i < n) out[4 * q + i] = w[i];
+}
+}  // namespace
+}  // namespace niti
+
+extern "C" int niti_rng_words_u32(const uint32_t* rng, uint32_t stream_id, uint32_t* out, size_t n, void* stream) {
+  clear_error();
+  if (rng == nullptr || (out == nullptr && n != 0)) return fail(NITI_ERR_INVALID_ARG, "rng_words: null pointer");
+  if (n == 0) return NITI_OK;
+  if (n > (1ULL << 34)) return fail(NITI_ERR_UNSUPPORTED, "rng_words: a stream has 2^34 words");
+  const long long quads = static_cast<long long>((n + 3) / 4);
+  hipLaunchKernelGGL(rng_words_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                     rng, stream_id, out, static_cast<long long>(n));
+  return check_launch("rng_words");
 }

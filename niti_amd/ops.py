@@ -694,6 +694,146 @@ def loss_grad(out_val, out_exp, target, rand, div_mode="floor"):
     return grad
 
 
+def loss_grad_rng(out_val, out_exp, target, rng, div_mode="floor"):
+    """``loss_grad`` with the random integers drawn in the kernel from the generator state ``rng`` (see rng_state)."""
+    _chk_dev(out_val, out_exp, target, rng)
+    if out_val.dtype != torch.int8 or out_val.dim() != 2 or not out_val.is_contiguous():
+        raise RuntimeError("loss_grad_rng: contiguous int8 [n, classes] logits expected")
+    if out_exp.dtype != torch.int32 or target.dtype != torch.int64 or target.numel() != out_val.shape[0] or not target.is_contiguous():
+        raise RuntimeError("loss_grad_rng: int32 exponent and int64 targets [n] expected")
+    _check_rng(rng, "loss_grad_rng")
+    n, classes = out_val.shape
+    grad = torch.empty_like(out_val)
+    L.check(L.lib().niti_loss_grad_i8_rng(_ptr(out_val), _ptr(out_exp), _ptr(target), _ptr(rng), _ptr(grad), n, classes,
+                                          L.DIV[div_mode], _stream(out_val)), "niti_loss_grad_i8_rng")
+    return grad
+
+
+RNG_STREAM = {"dropout": 1, "loss": 2}
+_rng_states = {}
+
+
+def _check_rng(rng, who):
+    if rng.dtype != torch.int32 or rng.numel() != 4 or not rng.is_contiguous() or not rng.is_cuda:
+        raise RuntimeError("%s: the generator state is a contiguous int32 tensor of 4 words on the GPU" % who)
+
+
+def rng_state(device=None, key=None):
+    """Generator state for the kernels that draw their own random integers (dropout mask, loss gradient rounding):
+    int32[4] = {key0, key1, step, 0}.  Without ``key`` returns the device's shared state, created on first use with
+    a key taken from torch's default CPU generator (so ``torch.manual_seed`` fixes the sequence); with ``key`` (an
+    int, 64 bits used) a fresh state at step 0.  Creating a state copies to the device: not under graph capture."""
+    dev = torch.device("cuda", torch.cuda.current_device()) if device is None else torch.device(device)
+    if dev.index is None:
+        dev = torch.device("cuda", torch.cuda.current_device())
+    if key is None:
+        if str(dev) not in _rng_states:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("rng_state: first use under graph capture; run one step eagerly first")
+            k = int(torch.empty((), dtype=torch.int64).random_().item())
+            _rng_states[str(dev)] = rng_state(dev, k)
+        return _rng_states[str(dev)]
+    words = [key & 0xFFFFFFFF, (key >> 32) & 0xFFFFFFFF, 0, 0]
+    return torch.tensor([w - (1 << 32) if w >= (1 << 31) else w for w in words], dtype=torch.int32).to(dev)
+
+
+def rng_words(rng, stream, n):
+    """The first ``n`` words (int32 tensor, to be read as unsigned) of stream "dropout" / "loss" that a kernel launched
+    now would draw from ``rng``; the state is not advanced."""
+    _check_rng(rng, "rng_words")
+    out = torch.empty(n, dtype=torch.int32, device=rng.device)
+    L.check(L.lib().niti_rng_words_u32(_ptr(rng), RNG_STREAM[stream] if isinstance(stream, str) else int(stream), _ptr(out), n,
+                                       _stream(rng)), "niti_rng_words_u32")
+    return out
+
+
+def head_sync_words(which, M, O, F) -> int:
+    """uint32 sync words of the classifier-head kernels ("forward" / "backward"); 0 = shape not covered."""
+    return int(L.lib().niti_head_i8_sync_words(1 if which == "backward" else 0, M, O, F))
+
+
+def head_forward(act, w, target_bits=7, method="round", div_mode="floor", bw_mode="int", relu=False, dropout=None,
+                 drop_mask=None, rng=None, exp_bias=0, target=None, loss_rand=None, sync=None, shift_out=None, exp_a=None,
+                 exp_b=None, exp_out=None):
+    """Classifier forward in one launch (niti_head_i8_forward): act_calc((act * mask) @ w^T) for act [M,F], w [O,F],
+    O <= 16.  ``dropout``: None, "given" (``drop_mask`` int8 [F] of 0 / 1 is read) or "draw" (the mask is drawn from
+    ``rng`` and written to ``drop_mask``, allocated here when None).  With ``target`` (int64 [M]) the loss gradient
+    of the logits is computed as well, rounded with ``loss_rand`` (int32 [M,O]) or with draws from ``rng``.
+    Returns (out8 [M,O], drop_mask or None, loss gradient [M,O] or None, shift, sync)."""
+    _chk_dev(act, w, sync, shift_out, exp_a, exp_b, exp_out, drop_mask, rng, target, loss_rand)
+    if act.dtype != torch.int8 or w.dtype != torch.int8 or act.dim() != 2 or w.dim() != 2 or act.shape[1] != w.shape[1]:
+        raise RuntimeError("head_forward: int8 act [M,F] and w [O,F] expected")
+    if not act.is_contiguous() or not w.is_contiguous():
+        raise RuntimeError("head_forward: contiguous operands expected")
+    M, F = act.shape
+    O = w.shape[0]
+    mode = {None: 0, "given": 1, "draw": 2}[dropout]
+    if mode == 2 and drop_mask is None:
+        drop_mask = torch.empty(F, dtype=torch.int8, device=act.device)
+    if mode != 0 and (drop_mask is None or drop_mask.dtype != torch.int8 or drop_mask.numel() != F or not drop_mask.is_contiguous()):
+        raise RuntimeError("head_forward: drop_mask must be a contiguous int8 tensor of F elements")
+    if rng is not None:
+        _check_rng(rng, "head_forward")
+    loss_grad_out = None
+    if target is not None:
+        if target.dtype != torch.int64 or target.numel() != M or not target.is_contiguous():
+            raise RuntimeError("head_forward: int64 targets [M] expected")
+        if loss_rand is not None and (loss_rand.dtype != torch.int32 or tuple(loss_rand.shape) != (M, O) or not loss_rand.is_contiguous()):
+            raise RuntimeError("head_forward: loss_rand must be a contiguous int32 [M,O] tensor")
+        loss_grad_out = torch.empty((M, O), dtype=torch.int8, device=act.device)
+    words = head_sync_words("forward", M, O, F)
+    if words == 0:
+        raise L.NitiError("head_forward: shape not covered by the few-output-features kernels")
+    if sync is None:
+        sync = sync_arena.take(words, act.device)
+    elif sync.dtype != torch.int32 or sync.numel() < words:
+        raise RuntimeError("head_forward: sync must be a zeroed int32 tensor of at least %d words" % words)
+    out = torch.empty((M, O), dtype=torch.int8, device=act.device)
+    if shift_out is None:
+        shift_out = torch.empty(1, dtype=torch.int32, device=act.device)
+    st = L.lib().niti_head_i8_forward(_ptr(act), _ptr(w), _ptr(out), M, O, F, mode, _ptr(drop_mask) if mode else None, _ptr(rng),
+                                      int(exp_bias), _ptr(target), _ptr(loss_rand), _ptr(loss_grad_out), target_bits,
+                                      L.ROUND[method], L.DIV[div_mode], L.BW[bw_mode], L.RQ_RELU if relu else 0, _ptr(sync),
+                                      sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _stream(act))
+    L.check(st, "niti_head_i8_forward")
+    return out, (drop_mask if mode else None), loss_grad_out, shift_out, sync
+
+
+def head_backward(err, act, w, err_bits=7, err_method="psto", grad_bits=5, grad_method="psto", div_mode="floor", bw_mode="int",
+                  drop_mask=None, want_grad=False, sync=None, exp_err=None, exp_w=None, exp_act=None, exp_act_bias=0,
+                  err_exp_out=None, grad_exp_out=None):
+    """Classifier backward in one launch (niti_head_i8_backward): err [M,O], act [M,F] (in front of the dropout),
+    w [O,F] (updated in place), ``drop_mask`` int8 [F] of 0 / 1 or None.  Returns (dx8 [M,F] with the mask applied,
+    rounded gradient [O,F] or None, err shift, grad shift, sync)."""
+    _chk_dev(err, act, w, drop_mask, sync, exp_err, exp_w, exp_act, err_exp_out, grad_exp_out)
+    if (err.dtype != torch.int8 or act.dtype != torch.int8 or w.dtype != torch.int8 or err.dim() != 2 or act.dim() != 2
+            or w.dim() != 2 or err.shape[0] != act.shape[0] or tuple(w.shape) != (err.shape[1], act.shape[1])):
+        raise RuntimeError("head_backward: int8 err [M,O], act [M,F], w [O,F] expected")
+    if not (err.is_contiguous() and act.is_contiguous() and w.is_contiguous()):
+        raise RuntimeError("head_backward: contiguous operands expected")
+    M, O = err.shape
+    F = act.shape[1]
+    if drop_mask is not None and (drop_mask.dtype != torch.int8 or drop_mask.numel() != F or not drop_mask.is_contiguous()):
+        raise RuntimeError("head_backward: drop_mask must be a contiguous int8 tensor of F elements")
+    words = head_sync_words("backward", M, O, F)
+    if words == 0:
+        raise L.NitiError("head_backward: shape not covered (M <= 256, O <= 16, F a multiple of 64)")
+    if sync is None:
+        sync = sync_arena.take(words, err.device)
+    elif sync.dtype != torch.int32 or sync.numel() < words:
+        raise RuntimeError("head_backward: sync must be a zeroed int32 tensor of at least %d words" % words)
+    dx = torch.empty((M, F), dtype=torch.int8, device=err.device)
+    g8 = torch.empty_like(w) if want_grad else None
+    shifts = torch.empty(2, dtype=torch.int32, device=err.device)
+    st = L.lib().niti_head_i8_backward(_ptr(err), _ptr(act), _ptr(drop_mask), _ptr(w), _ptr(dx), M, O, F, err_bits,
+                                       L.ROUND[err_method], grad_bits, L.ROUND[grad_method], L.DIV[div_mode], L.BW[bw_mode],
+                                       _ptr(sync), sync.numel(), _ptr(g8), _ptr(shifts[0:1]), _ptr(shifts[1:2]), _ptr(exp_err),
+                                       _ptr(exp_w), _ptr(exp_act), int(exp_act_bias), _ptr(err_exp_out), _ptr(grad_exp_out),
+                                       _stream(err))
+    L.check(st, "niti_head_i8_backward")
+    return dx, g8, shifts[0:1], shifts[1:2], sync
+
+
 def mfma_probe(operands, workgroups=512, iters=1200):
     """Times the library's register-resident int8 MFMA loop over the given operand bytes (int8 tensor, >= 128 bytes).
     Returns (tera-operations per second, shader clock in GHz during the loop): the matrix-unit ceiling for operands

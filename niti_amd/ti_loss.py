@@ -9,16 +9,20 @@ class TiLoss(Module):
     """ti_loss.py:5-36: base-2 soft-max approximation of the cross-entropy gradient, rounded to int8
     with StoShift(.., 4).  One launch of the library's kernel, which keeps the reference's float32
     operation sequence per sample (``2 ** s`` by a fixed sequence of double operations, see exp2_f32); the ``out_exp > -7`` case split happens on the device, so there is no
-    host synchronisation.  ``rand`` (int32 in [0,16), one per logit) replaces the device random draw
-    when given."""
+    host synchronisation.  ``rand`` (int32 in [0,16), one per logit) replaces the random integers the kernel
+    otherwise draws itself (Philox4x32-10 on a small state in device memory, ops.rng_state)."""
+
+    rng = None      # RngBox of the network; without one the device's shared generator state is used
 
     def forward(self, out_val, out_exp, target, rand=None):
         dev = out_val.device
         e = ti_torch._exp_tensor(out_exp, dev)
-        if rand is None:
-            rand = torch.randint(0, 16, out_val.shape, dtype=torch.int32, device=dev)
-        self.out_grad = ops.loss_grad(out_val.contiguous(), e, target.to(torch.int64).contiguous(),
-                                      rand.to(torch.int32).contiguous(), ti_torch.DIV_MODE)
+        if rand is None:    # the kernel draws the random integers itself
+            state = self.rng.state(dev) if self.rng is not None else ops.rng_state(dev)
+            self.out_grad = ops.loss_grad_rng(out_val.contiguous(), e, target.to(torch.int64).contiguous(), state, ti_torch.DIV_MODE)
+        else:
+            self.out_grad = ops.loss_grad(out_val.contiguous(), e, target.to(torch.int64).contiguous(),
+                                          rand.to(torch.int32).contiguous(), ti_torch.DIV_MODE)
         return self.out_grad, 0
 
 

@@ -12,6 +12,11 @@ class TiNet(Module):
     def __init__(self):
         super().__init__()
         self.loss = TiLoss()
+        self.rng = ti_torch.RngBox()      # random draws made inside the kernels (dropout mask, loss gradient rounding)
+        self.loss.rng = self.rng
+        # the classifier TiLinear whose forward launch can evaluate the loss gradient (kept out of the module tree: it
+        # already is a member of forward_layers)
+        self.__dict__["_head"] = None
 
     def fuse(self):
         """Fold each TiReLU that directly follows a TiConv2d into that layer's requantisation."""
@@ -44,12 +49,23 @@ class TiNet(Module):
                 # ReLU -> max-pool -> anything else: the pooling's backward pass applies the mask to its own output
                 layers[i + 1].relu_below = True
                 l.bwd_folded = True
+        # [TiDropout ->] TiLinear with few outputs at the end: the classifier's launches apply the dropout mask (and
+        # draw it), and its forward launch evaluates the loss gradient when forward() is given the targets
+        if layers and isinstance(layers[-1], ti_torch.TiLinear) and layers[-1].weight.shape[0] <= 16:
+            self.__dict__["_head"] = layers[-1]
+            self._head.rng = self.rng
+            if len(layers) > 1 and isinstance(layers[-2], ti_torch.TiDropout):
+                # plain attributes, not sub-modules: the two layers refer to each other
+                layers[-1].__dict__["drop_below"] = layers[-2]
+                layers[-2].__dict__["head"] = layers[-1]
         return self
 
-    def forward(self, x):
-        """ti_net.py:17-23: float NCHW batch -> (int8 logits, exponent)."""
+    def forward(self, x, target=None):
+        """ti_net.py:17-23: float NCHW batch -> (int8 logits, exponent).  ``target`` (not in the reference): the
+        class indices that backward() will be called with; the classifier's forward launch then computes the loss
+        gradient as well and backward(target) with the same tensor starts from it."""
         x_data, x_exp = self.quantize_input(x)
-        return self.forward_int8(x_data, x_exp)
+        return self.forward_int8(x_data, x_exp, target)
 
     @staticmethod
     def quantize_input(x):
@@ -62,9 +78,13 @@ class TiNet(Module):
         x_data, x_exp = ti_torch.TiFloatToInt8(x)
         return x_data.permute(0, 2, 3, 1).contiguous(), x_exp
 
-    def forward_int8(self, x_data, x_exp=0):
+    def forward_int8(self, x_data, x_exp=0, target=None, loss_rand=None):
         """Same as forward() for a batch that already is int8 NHWC with exponent ``x_exp``."""
         ops.sync_arena.reset(x_data.device)     # one fill for the range-exchange words of the whole step
+        if self._head is not None:
+            self._head.next_target = None
+            if target is not None and ti_torch.TRAINING and target.dtype == torch.int64 and target.is_contiguous() and target.is_cuda:
+                self._head.next_target = (target, loss_rand)
         self.out, self.out_exp = self.forward_layers((x_data, x_exp))
         return self.out, self.out_exp
 
@@ -75,7 +95,13 @@ class TiNet(Module):
 
     def backward(self, target, loss_rand=None):
         """ti_net.py:25-32."""
-        x = self.loss(self.out, self.out_exp, target, loss_rand)
+        done = self._head.loss_grad if self._head is not None else None
+        if done is not None and done[0] is target and loss_rand is None:
+            self._head.loss_grad = None
+            self.loss.out_grad = done[1]        # the classifier's forward launch has evaluated TiLoss already
+            x = (done[1], 0)
+        else:
+            x = self.loss(self.out, self.out_exp, target, loss_rand)
         return self.backward_from(x)
 
     def backward_from(self, x):

@@ -557,6 +557,22 @@ class TiLinear(UpdateWeight):
         super().__init__()
         self._init_weight(torch.Size([out_features, in_features]))
         self.last_layer = last_layer
+        self.__dict__["drop_below"] = None   # the TiDropout in front of this layer whose masking this layer's kernels take over
+        self.rng = None             # RngBox of the network (dropout mask / loss rounding drawn inside the kernels)
+        self.next_target = None     # (targets, random integers or None): evaluate the loss gradient in the next forward
+        self.loss_grad = None       # (targets, loss gradient) left by that forward
+        self._dropped = None        # dropout mask the last forward applied itself
+
+    def _head(self, which, M, methods, rands):
+        """The pass runs as one of the classifier-head kernels (dropout, loss gradient, both backward products and the
+        update folded in) when the shape is inside them and no rounding needs random input."""
+        O, F = self.weight.shape
+        return (FUSE_CONV_REQUANT and all(r is None for r in rands) and all(_method_name(m) != "sto" for m in methods)
+                and self.weight.is_contiguous() and ("head", which, M, O, F) not in _fused_refused
+                and ops.head_sync_words(which, M, O, F) > 0)
+
+    def _rng_state(self, dev):
+        return self.rng.state(dev) if self.rng is not None else ops.rng_state(dev)
 
     def _one_launch(self, which, M, fn, rand):
         """The pass runs as one of the library's kernels for few output features (operands read as stored,
@@ -595,6 +611,30 @@ class TiLinear(UpdateWeight):
         act_in, exp_in = input
         act_in = act_in.contiguous()
         dev = act_in.device
+        drop, self._dropped, self.loss_grad = self.drop_below, None, None
+        pending = drop is not None and drop.pending is not None and drop.pending[0] is input[0]
+        want_loss, self.next_target = self.next_target, None
+        if (pending or want_loss is not None) and self._head("forward", act_in.shape[0], (ACT_ROUND_METHOD,), (rand,)):
+            M = act_in.shape[0]
+            exp_out = torch.empty(1, dtype=torch.int32, device=dev)
+            given = drop.pending[1] if pending else None
+            draws = (pending and given is None) or (want_loss is not None and want_loss[1] is None)
+            done = self._try("head-forward", M, lambda: ops.head_forward(
+                act_in, self.weight, BITWIDTH, _method_name(ACT_ROUND_METHOD), DIV_MODE, BW_MODE,
+                dropout=None if not pending else ("draw" if given is None else "given"), drop_mask=given,
+                rng=self._rng_state(dev) if draws else None, exp_bias=1 if pending else 0,
+                target=want_loss[0] if want_loss is not None else None, loss_rand=want_loss[1] if want_loss is not None else None,
+                exp_a=_exp_tensor(exp_in, dev), exp_b=self._wexp(), exp_out=exp_out))
+            if done is not None:
+                if pending:
+                    drop.drop_mask = self._dropped = done[1]
+                    drop.pending = None
+                if want_loss is not None:
+                    self.loss_grad = (want_loss[0], done[2])
+                return done[0], exp_out
+        if pending:   # the dropout left its work to this layer, which cannot take it: do it now
+            act_in, exp_in = drop.apply_now(act_in, exp_in)
+            self.act_in = (act_in, exp_in)
         if self._one_launch("forward", act_in.shape[0], ACT_ROUND_METHOD, rand):
             exp_out = torch.empty(1, dtype=torch.int32, device=dev)
             act_out, _, _ = ops.fc_fwd_requant(act_in, self.weight, BITWIDTH, _method_name(ACT_ROUND_METHOD), DIV_MODE, BW_MODE,
@@ -623,6 +663,22 @@ class TiLinear(UpdateWeight):
         act = act.contiguous()
         M = err_in.shape[0]
         self.err_exp_in = _exp_tensor(err_exp, dev)
+        mask = self._dropped     # the forward pass read ``act`` through this mask: act_in is the tensor in front of the dropout
+        if not KEEP_INT32_GRAD and self._head("backward", M, (ERROR_ROUND_METHOD, GRAD_ROUND_METHOD), (rand, grad_rand)):
+            exps = torch.empty(2, dtype=torch.int32, device=dev)
+            done = self._try("head-backward", M, lambda: ops.head_backward(
+                err_in, act, self.weight, BITWIDTH, _method_name(ERROR_ROUND_METHOD), GRAD_BITWIDTH, _method_name(GRAD_ROUND_METHOD),
+                DIV_MODE, BW_MODE, drop_mask=mask, want_grad=self.keep_grad, exp_err=self.err_exp_in, exp_w=self._wexp(),
+                exp_act=_exp_tensor(self.act_in_exp, dev), exp_act_bias=1 if mask is not None else 0,
+                err_exp_out=exps[0:1], grad_exp_out=exps[1:2]))
+            if done is not None:
+                self.err_exp, self.grad_exp = exps[0:1], exps[1:2]
+                self.grad, self.grad_shift, self.grad_int32acc = done[1], done[3], None
+                if mask is not None:
+                    self.drop_below.bwd_done = done[0]     # masked already
+                return done[0], self.err_exp
+        if mask is not None:     # the separate passes want the masked activations and their exponent
+            act, self.act_in_exp = ops.mask_features(act, mask, _exp_tensor(self.act_in_exp, dev), 1)
         done = None
         if self._one_launch("dgrad", M, ERROR_ROUND_METHOD, rand):
             new_exp = torch.empty(1, dtype=torch.int32, device=dev)
@@ -736,18 +792,38 @@ class TiFlat(Module):
 
 class TiDropout(Module):
     """ti_torch.py:439-455: one keep/drop decision per feature (not per sample), exponent + 1.
-    ``mask`` (int8 0/1 per feature) can be supplied for reproducible runs."""
+    ``mask`` (int8 0/1 per feature) can be supplied for reproducible runs.  With ``head`` set (TiNet.fuse: the
+    TiLinear that follows) the masking is left to that layer's kernels, which also draw the mask."""
+
+    def __init__(self):
+        super().__init__()
+        self.__dict__["head"] = None   # the TiLinear behind this layer that applies the mask in its own launches
+        self.pending = None      # (activation tensor, given mask or None) handed to that layer
+        self.bwd_done = None     # the error tensor that layer has already masked
 
     def forward(self, input, mask=None):
         if TRAINING:
             act_in, exp_in = input
-            if mask is None:
-                mask = torch.randint(low=0, high=2, size=(act_in.size(1),), dtype=torch.int8, device=act_in.device)
-            self.drop_mask = mask.to(act_in.device)
-            if self._one_launch(act_in):
-                return ops.mask_features(act_in, self.drop_mask, _exp_tensor(exp_in, act_in.device), 1)
-            return act_in * self.drop_mask, _exp_tensor(exp_in, act_in.device) + 1
+            if mask is not None:
+                mask = mask.to(act_in.device)
+            if (self.head is not None and FUSE_CONV_REQUANT and act_in.is_cuda and act_in.dtype == torch.int8 and act_in.dim() == 2
+                    and act_in.is_contiguous() and (mask is None or (mask.dtype == torch.int8 and mask.is_contiguous()))):
+                self.pending = (act_in, mask)
+                return input
+            return self.apply_now(act_in, exp_in, mask)
+        self.pending = None
         return input
+
+    def apply_now(self, act_in, exp_in, mask=None):
+        if mask is None and self.pending is not None:
+            mask = self.pending[1]
+        self.pending = None
+        if mask is None:
+            mask = torch.randint(low=0, high=2, size=(act_in.size(1),), dtype=torch.int8, device=act_in.device)
+        self.drop_mask = mask.to(act_in.device)
+        if self._one_launch(act_in):
+            return ops.mask_features(act_in, self.drop_mask, _exp_tensor(exp_in, act_in.device), 1)
+        return act_in * self.drop_mask, _exp_tensor(exp_in, act_in.device) + 1
 
     def _one_launch(self, t):
         m = self.drop_mask
@@ -756,6 +832,25 @@ class TiDropout(Module):
 
     def backward(self, input):
         err_in, err_exp = input
+        done, self.bwd_done = self.bwd_done, None
+        if done is not None and done is err_in:
+            return input        # the layer behind this one masked its data gradient already
         if self._one_launch(err_in):
             return ops.mask_features(err_in, self.drop_mask), err_exp
         return err_in * self.drop_mask, err_exp
+
+
+class RngBox:
+    """The generator state (ops.rng_state) of one network, created on first use with a key drawn from torch's default
+    CPU generator: two networks built after the same ``torch.manual_seed`` draw the same sequence."""
+
+    def __init__(self):
+        self._state = {}
+
+    def state(self, device):
+        key = str(device)
+        if key not in self._state:
+            if torch.cuda.is_current_stream_capturing():
+                raise RuntimeError("RngBox: first use under graph capture; run one step eagerly first")
+            self._state[key] = ops.rng_state(device, int(torch.empty((), dtype=torch.int64).random_().item()))
+        return self._state[key]

@@ -51,7 +51,7 @@ def _add_metrics(output, output_exp, target, sums):
 
 def _one_step(model, training, inputs, target, sums):
     """Forward (+ backward when training) on one batch of float images."""
-    output, output_exp = model(inputs)
+    output, output_exp = model(inputs, target if training else None)
     _add_metrics(output, output_exp, target, sums)
     if training:
         model.backward(target)
@@ -77,7 +77,7 @@ class StepGraph:
         self.side = torch.cuda.Stream()
 
     def _step(self):
-        self.model.forward_int8(self.x8, self.x_exp)
+        self.model.forward_int8(self.x8, self.x_exp, self.target if self.training else None)
         if self.training:
             self.model.backward(self.target)
 

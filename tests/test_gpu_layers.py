@@ -220,7 +220,29 @@ def test_training_step(tt, name, cfg_list, N):
     yo, eo = onet.forward_int8(x, 0)
     y, e = net.forward_int8(x.to(dev), 0)
     assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+    # a complete step with the targets known at forward time: the classifier's forward launch evaluates the loss
+    # gradient, backward(target) starts from it
     from niti_amd import ops
+    onet.backward(target, loss_rand)
+    tgt = target.to(dev)
+    calls = []
+    orig_loss = ops.loss_grad
+    ops.loss_grad = lambda *a, **k: calls.append("loss") or orig_loss(*a, **k)
+    try:
+        y, e = net.forward_int8(x.to(dev), 0, tgt, loss_rand.to(dev))
+        assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+        net.backward(tgt)
+    finally:
+        ops.loss_grad = orig_loss
+    assert calls == []
+    from oracle import niti_oracle as po
+    if not bool((po.ti_loss_pre_round(yo, eo, target) == -2 ** 31).any()):
+        # (for exponents far from zero the reference's own formula, ti_loss.py:14-31, divides 0 by 0 and converts the NaN
+        # to an integer, which host and device do differently: nothing to compare there)
+        assert torch.equal(net.loss.out_grad.cpu(), onet.loss_err)
+        for i, (a, b) in enumerate(zip(gl, ol)):
+            assert torch.equal(a.weight.cpu(), b.weight), "updated weight of layer %d (second step)" % i
+            assert _ei(a.grad_exp) == b.grad_exp
     assert not ops.sync_arena.timed_out(dev), "a single-launch kernel gave up waiting for its workgroups"
 
 
