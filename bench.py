@@ -225,7 +225,8 @@ def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH, graph=True):
         if hasattr(l, "weight"):
             l.weight = torch.randint(-127, 128, tuple(l.weight.shape), generator=g, dtype=torch.int8).to(dev)
             l.weight_exp = torch.tensor(-8.0)
-    x = torch.randint(-127, 128, (batch, 32, 32, 3), generator=g, dtype=torch.int8).to(dev)
+    # the batch as the input quantiser delivers it (ops.quantize_input): int8 NHWC with the 3 channels zero-padded to 16
+    x = torch.nn.functional.pad(torch.randint(-127, 128, (batch, 32, 32, 3), generator=g, dtype=torch.int8), (0, 13)).to(dev)
     target = torch.randint(0, 10, (batch,), generator=g).to(dev)
     ti_torch.TRAINING = True
     ti_torch.GRAD_BITWIDTH = 5
