@@ -228,6 +228,10 @@ size_t wgrad3x3_sync_words(int blocks);
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
                            bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
                            void* workspace, hipStream_t stream);
+// one-launch weight gradient + update for 4 x 4 and 2 x 2 maps (wgrad_small.hip); sync words as for the finishing kernel
+bool wgrad_small_supported(int N, int H, int C, int K, int w_channels);
+int launch_wgrad_small_update(const int8_t* act, const int8_t* err, int8_t* w, int N, int H, int C, int K, bool roundtrip,
+                              uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep, hipStream_t stream);
 int conv3x3_halo_requant_blocks(int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
 size_t conv3x3_halo_sync_words(int blocks);
 int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, int N, int H, int C, int K, unsigned flags,

@@ -878,6 +878,12 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   const int nb = wgrad3x3_finish_blocks(Cp, K);
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large for the single-pass finish", K, C);
   if (static_cast<long long>(K) * 9 * C >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large", K, C);
+  {
+    // few pixels, many weights: nothing to split, one launch does it all (NITI_WGRAD_SMALL=0 pins the kernel pair below)
+    const char* e = getenv("NITI_WGRAD_SMALL");
+    if ((e == nullptr || e[0] != '0') && wgrad_small_supported(N, H, C, K, w_channels))
+      return launch_wgrad_small_update(act, err, w, N, H, C, K, roundtrip, sync, rq, g8, dw, wprep, stream);
+  }
   static int resident_of[kDeviceSlots][2] = {};   // workgroups of 4 / 16 wavefronts the device holds at once
   int* const resident = resident_of[device_slot()];
   if (resident[0] == 0) {
