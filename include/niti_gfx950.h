@@ -161,8 +161,7 @@ int niti_conv2d_i8_fprop_requant(const int8_t* x, const int8_t* w, int8_t* y8, i
  * niti_conv2d_i8_fprop_requant that also writes the 2x2 / stride-2 maximum of its output: the TiMaxpool2d.forward ->
  * int8pool_cuda.int8_pool call that follows the layer (and its ReLU) in the reference's networks (ti_torch.py:302-307,
  * int8pool_kernel.cu:28-80; ti_vgg.py:28-35), taken from the rounded values before they leave the kernel.
- * pool_out: [N,H/2,W/2,K] int8, 16-byte aligned.  Same coverage as niti_conv2d_i8_fprop_requant except maps of side 2
- * (NITI_ERR_UNSUPPORTED: use niti_maxpool_i8_fwd on y8).
+ * pool_out: [N,H/2,W/2,K] int8, 16-byte aligned.  Same coverage as niti_conv2d_i8_fprop_requant.
  */
 int niti_conv2d_i8_fprop_requant_pool(const int8_t* x, const int8_t* w, int8_t* y8, int8_t* pool_out, int N, int H, int W, int C,
                                       int K, int R, int S, int stride, int pad, unsigned flags, int target_bits, int method,
@@ -186,7 +185,7 @@ int niti_conv2d_i8_dgrad_requant(const int8_t* err, const int8_t* w, int8_t* dx8
  * output = the layer's input activations; pool_in: [N,2H,2W,C] int8, the pooling's input; dx8_unpooled: [N,2H,2W,C]
  * int8; all 16-byte aligned.  Elements whose pooled value is not positive get zero (the ReLU in front of the pooling);
  * the others go to the first position of their window that equals the pooled value (NITI_TIES_FIRST) or to all of them
- * (NITI_TIES_ALL).  Same coverage as niti_conv2d_i8_dgrad_requant except maps of side 2 (NITI_ERR_UNSUPPORTED).
+ * (NITI_TIES_ALL).  Same coverage as niti_conv2d_i8_dgrad_requant.
  */
 int niti_conv2d_i8_dgrad_requant_unpool(const int8_t* err, const int8_t* w, int8_t* dx8_unpooled, const int8_t* pooled,
                                         const int8_t* pool_in, int ties, int N, int H, int W, int C, int K, int R, int S, int stride,

@@ -956,9 +956,48 @@ __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int
         uint32_t v = pack4_i8(r[0], r[1], r[2], r[3]);
         const int c = ch + 8 * g;
         const int off = (n < a.N && c < a.K) ? static_cast<int>(row + c) : kOob;
-        if (a.mask != nullptr)   // ReLU backward of the layer below, folded in: its output is this layer's input
-          v &= positive_bytes(static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b32(rm, off, 0, 0)));
-        __builtin_amdgcn_raw_buffer_store_b32(v, ry, off, 0, 0);
+        uint32_t mk = 0;
+        if (a.mask != nullptr) {   // ReLU backward of the layer below, folded in: its output is this layer's input
+          mk = static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b32(rm, off, 0, 0));
+          v &= positive_bytes(mk);
+        }
+        if (a.unpool != nullptr) {
+          // max-pool backward folded in (mk holds the pooled values): the window of this pixel in the pooling's 4 x 4 input
+          const __amdgpu_buffer_rsrc_t rxp = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.pool_x), 0, a.unpool_bytes, 0x00020000);
+          const __amdgpu_buffer_rsrc_t ru = __builtin_amdgcn_make_buffer_rsrc(a.unpool, 0, a.unpool_bytes, 0x00020000);
+          const int base = ((n * 4 + 2 * py) * 4 + 2 * px) * a.K + c;
+          int wo[4];
+          uint32_t xw[4];
+#pragma unroll
+          for (int q = 0; q < 4; ++q) wo[q] = off == kOob ? kOob : base + (q >> 1) * 4 * a.K + (q & 1) * a.K;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) xw[q] = static_cast<uint32_t>(__builtin_amdgcn_raw_buffer_load_b32(rxp, wo[q], 0, 0));
+          uint32_t taken = 0;   // bytes whose gradient an earlier position of the window (scan order) already received
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const uint32_t eq = equal_bytes(xw[q], mk);
+            const uint32_t keep = a.ties_all != 0 ? eq : eq & ~taken;
+            taken |= eq;
+            __builtin_amdgcn_raw_buffer_store_b32(v & keep, ru, wo[q], 0, 0);
+          }
+        } else {
+          __builtin_amdgcn_raw_buffer_store_b32(v, ry, off, 0, 0);
+        }
+        if (a.pool != nullptr) reinterpret_cast<uint32_t*>(red)[(p * 4 + g) * 64 + lane] = v;   // the sums parked here have been read
+      }
+    }
+    if (a.pool != nullptr) {
+      // the 2 x 2 max-pool behind this layer leaves one pixel: wavefront g takes the maximum over the four pixels for
+      // its group of channels
+      __syncthreads();
+      if (rh == 0) {
+        const uint32_t* pv = reinterpret_cast<const uint32_t*>(red);
+        const int g = p;
+        const uint32_t mx = max_i8x4(max_i8x4(pv[(0 * 4 + g) * 64 + lane], pv[(1 * 4 + g) * 64 + lane]),
+                                     max_i8x4(pv[(2 * 4 + g) * 64 + lane], pv[(3 * 4 + g) * 64 + lane]));
+        const __amdgpu_buffer_rsrc_t rp = __builtin_amdgcn_make_buffer_rsrc(a.pool, 0, a.pool_bytes, 0x00020000);
+        const int c = ch + 8 * g;
+        __builtin_amdgcn_raw_buffer_store_b32(mx, rp, (n < a.N && c < a.K) ? n * a.K + c : kOob, 0, 0);
       }
     }
     if (blockIdx.x == 0 && tid == 0) {
@@ -1206,12 +1245,9 @@ int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, i
   a.unpool_bytes = 4 * a.y8_bytes;
   a.ties_all = rq.ties_all;
   if (a.unpool != nullptr) {
-    if (H == 2) return fail(NITI_ERR_UNSUPPORTED, "conv_requant: the max-pool backward pass is not folded in on 2 x 2 maps");
     if (a.mask == nullptr || a.pool_x == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_requant: unpooling needs the pooled map and the pooling's input");
     if (a.unpool_bytes >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "conv_requant: unpooled map of 2 GiB or more");
   }
-  if (a.pool != nullptr && H == 2)
-    return fail(NITI_ERR_UNSUPPORTED, "conv_requant: the pooled output is not available on 2 x 2 maps");
   a.target_bits = rq.target_bits;
   a.method = rq.method;
   a.trunc = rq.trunc;

@@ -396,7 +396,7 @@ class TiConv2d(UpdateWeight):
         exp_a, exp_b = _exp_tensor(self.act_in_exp, dev), self._wexp()
         pooled = None
         N, H, W, _ = self.act16.shape
-        if self.pool_after is not None and self.fuse_relu and self.stride == 1 and self.padding == 1 and H == W and H >= 4 and H % 2 == 0:
+        if self.pool_after is not None and self.fuse_relu and self.stride == 1 and self.padding == 1 and H == W and H >= 2 and H % 2 == 0:
             pooled = torch.empty((N, H // 2, W // 2, self.weight.shape[0]), dtype=torch.int8, device=dev)
         fused = _conv_requant_fused(False, self.act16, w16, self.stride, self.padding, ACT_ROUND_METHOD, rand,
                                     self.fuse_relu, exp_a, exp_b, prepared_filter=self._forward_filter(w16),
@@ -467,7 +467,7 @@ class TiConv2d(UpdateWeight):
     def _data_gradient(self, err_in, rand, mask, forward_filter):
         """err_calc(conv_dgrad(err_in, weight)) (ti_torch.py:422-427), the ReLU mask applied; -> (int8 error, exponent)."""
         pool = self.pool_below
-        if (pool is not None and mask is not None and err_in.shape[1] > 2 and getattr(pool, "act_out", None) is not None
+        if (pool is not None and mask is not None and err_in.shape[1] >= 2 and getattr(pool, "act_out", None) is not None
                 and pool.act_out.data_ptr() == mask.data_ptr() and pool.act_in.is_contiguous()):
             # the max-pool in front of this layer: its backward pass is written by this launch's epilogue
             fused = _conv_requant_fused(True, err_in, self.weight, self.stride, self.padding, ERROR_ROUND_METHOD, rand,
