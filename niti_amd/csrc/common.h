@@ -228,6 +228,13 @@ size_t wgrad3x3_sync_words(int blocks);
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
                            bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
                            void* workspace, hipStream_t stream);
+// one-launch weight gradient + update of the first layer (wgrad_first.hip); its accumulation buffer are extra zeroed sync
+// words behind the finishing kernel's
+size_t wgrad_first_extra_words(int H, int C, int K);
+bool wgrad_first_supported(int N, int H, int C, int K, int w_channels);
+int launch_wgrad_first_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int K, bool roundtrip,
+                              uint32_t* sync, int32_t* accum, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
+                              hipStream_t stream);
 // one-launch weight gradient + update for 4 x 4 and 2 x 2 maps (wgrad_small.hip); sync words as for the finishing kernel
 bool wgrad_small_supported(int N, int H, int C, int K, int w_channels);
 int launch_wgrad_small_update(const int8_t* act, const int8_t* err, int8_t* w, int N, int H, int C, int K, bool roundtrip,

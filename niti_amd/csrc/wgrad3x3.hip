@@ -879,6 +879,14 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   if (nb == 0) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large for the single-pass finish", K, C);
   if (static_cast<long long>(K) * 9 * C >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: gradient of %d x 9 x %d too large", K, C);
   {
+    // the first layer: one launch with integer atomics and a last-arriver finish (NITI_WGRAD_FIRST=0 pins the pair below)
+    const char* e = getenv("NITI_WGRAD_FIRST");
+    if ((e == nullptr || e[0] != '0') && wgrad_first_supported(N, H, C, K, w_channels)) {
+      int32_t* const accum = reinterpret_cast<int32_t*>(sync + wgrad3x3_sync_words(wgrad3x3_finish_blocks(C, K)));
+      return launch_wgrad_first_update(act, err, w, w_channels, N, K, roundtrip, sync, accum, rq, g8, dw, wprep, stream);
+    }
+  }
+  {
     // few pixels, many weights: nothing to split, one launch does it all (NITI_WGRAD_SMALL=0 pins the kernel pair below)
     const char* e = getenv("NITI_WGRAD_SMALL");
     if ((e == nullptr || e[0] != '0') && wgrad_small_supported(N, H, C, K, w_channels))

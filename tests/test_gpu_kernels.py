@@ -454,7 +454,8 @@ def test_conv_wgrad_arrangements(dev, case, wgrad_arrangement):
 
 
 @pytest.mark.parametrize("case", [(4, 32, 16, 32), (8, 16, 128, 64), (6, 8, 80, 144), (64, 8, 64, 256), (16, 16, 256, 128),
-                                  (2, 8, 16, 16), (4, 8, 3, 16), (8, 32, 3, 128), (32, 8, 512, 512), (16, 4, 64, 128), (64, 4, 512, 256), (64, 2, 128, 64), (256, 2, 512, 512)])
+                                  (2, 8, 16, 16), (4, 8, 3, 16), (8, 32, 3, 128), (32, 8, 512, 512), (16, 4, 64, 128), (64, 4, 512, 256), (64, 2, 128, 64), (256, 2, 512, 512),
+                                  (3, 32, 3, 64), (2, 32, 3, 32), (2, 32, 3, 256), (5, 32, 2, 64), (1, 32, 1, 128)])
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 def test_conv_wgrad_update(dev, case, div_mode):
     """wgrad + grad_calc + weight update in one call against the oracle's three steps."""
