@@ -44,6 +44,10 @@ struct WfArgs {
   int32_t* exp_out;
 };
 
+template <int N>
+__device__ inline void wf_wait_vmcnt() {
+  __builtin_amdgcn_s_waitcnt((N & 15) | (((N >> 4) & 3) << 14) | 0x0F70);
+}
 __device__ inline void wf_sync() {
   asm volatile("" ::: "memory");
   __builtin_amdgcn_s_barrier();
@@ -59,7 +63,9 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
   constexpr int PP = K / 16;             // 16-byte pieces per pixel of the error tile
   constexpr int SWZ = PP >= 8 ? 7 : PP - 1;
   constexpr int PPI = 1024 / K;          // pixels per staging instruction
-  constexpr int BUF = 256 * K > 32768 ? 256 * K : 32768;   // error tile of 8 rows; later the wavefronts' parked sums
+  constexpr int NBUF = K <= 128 ? 4 : 2;                   // error tiles of 8 rows in LDS
+  constexpr int BUF = 256 * K;                             // the wavefronts' sums are parked across them at the end (32 KB)
+  static_assert(NBUF * BUF >= 32768, "room for the parked sums");
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   int8_t* const planes = smem;
   int8_t* const ebuf = smem + kWfXBytes;
@@ -71,18 +77,10 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
   const int kb = wave % KB, pg = wave / KB;
   const int n = blockIdx.x;
 
-  // ---- the image's channel planes, zero border
-  for (int i = tid; i < kWfXBytes / 4; i += 512) reinterpret_cast<uint32_t*>(planes)[i] = 0u;
-  __syncthreads();
+  // the image's pixels (the first dword of each holds the channels), requested ahead of the error tiles
+  uint32_t xv[2];
 #pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int pix = tid + 512 * h;
-    const uint32_t v = *reinterpret_cast<const uint32_t*>(a.act + (static_cast<long long>(n) * 1024 + pix) * 16);
-    const int at = ((pix >> 5) + 1) * kWfPitch + (pix & 31) + 1;
-#pragma unroll
-    for (int c = 0; c < 3; ++c)
-      if (c < a.Cw) planes[c * kWfPlane + at] = static_cast<int8_t>((v >> (8 * c)) & 0xFFu);
-  }
+  for (int h = 0; h < 2; ++h) xv[h] = *reinterpret_cast<const uint32_t*>(a.act + (static_cast<long long>(n) * 1024 + tid + 512 * h) * 16);
 
   // ---- error tile staging: an instruction fills PPI pixels x K bytes; pieces swizzled by the pixel (bank spread)
   const __amdgpu_buffer_rsrc_t rerr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.err), 0, a.err_bytes, 0x00020000);
@@ -117,12 +115,31 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
   v16i acc;
 #pragma unroll
   for (int e = 0; e < 16; ++e) acc[e] = 0;
-  issue(0, 0);
-  for (int piece8 = 0; piece8 < 4; ++piece8) {
-    __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0): this piece has landed
+  // all four pieces of the image are requested at once where they fit (one memory latency instead of four)
+  if (NBUF == 4) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) issue(q, q);
+  } else {
+    issue(0, 0);
+  }
+  // ---- the image's channel planes with a border of zeros, while the error tiles are on their way
+  for (int i = tid; i < kWfXBytes / 4; i += 512) reinterpret_cast<uint32_t*>(planes)[i] = 0u;
+  __syncthreads();
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int pix = tid + 512 * h;
+    const int at = ((pix >> 5) + 1) * kWfPitch + (pix & 31) + 1;
+#pragma unroll
+    for (int c = 0; c < 3; ++c)
+      if (c < a.Cw) planes[c * kWfPlane + at] = static_cast<int8_t>((xv[h] >> (8 * c)) & 0xFFu);
+  }
+  static_for<4>([&](auto piecec) {
+    constexpr int piece8 = decltype(piecec)::value;
+    if (NBUF == 4) wf_wait_vmcnt<(3 - piece8) * KB>();     // this piece has landed (loads complete in order)
+    else wf_wait_vmcnt<0>();
     wf_sync();                                             // ... for every wavefront, and the other buffer has been read
-    if (piece8 + 1 < 4) issue(piece8 + 1, (piece8 + 1) & 1);
-    const unsigned ebase = lds0 + static_cast<unsigned>(kWfXBytes + (piece8 & 1) * BUF);
+    if (NBUF != 4 && piece8 + 1 < 4) issue(piece8 + 1, (piece8 + 1) & 1);
+    const unsigned ebase = lds0 + static_cast<unsigned>(kWfXBytes + (piece8 % NBUF) * BUF);
 #pragma unroll
     for (int i = 0; i < RW; ++i) {
       const int r = pg * RW + i;                           // image row inside the piece
@@ -145,7 +162,7 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
       if (!live) fb = v4i{0, 0, 0, 0};
       acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, fb, acc, 0, 0, 0);
     }
-  }
+  });
   // ---- add the row groups through LDS, then into the accumulation buffer.  acc[4 g + e]: output channel
   // kb * 32 + 8 g + 4 lk + e, column lane % 32
   __syncthreads();   // every wavefront is done with the error tiles
@@ -241,7 +258,7 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
 template <int KB>
 int wf_launch(const WfArgs& a, hipStream_t stream) {
   constexpr int K = KB * 32;
-  constexpr size_t lds = static_cast<size_t>(kWfXBytes) + 2 * static_cast<size_t>(256 * K > 32768 ? 256 * K : 32768);
+  constexpr size_t lds = static_cast<size_t>(kWfXBytes) + static_cast<size_t>(K <= 128 ? 4 : 2) * 256 * K;
   auto k = wgrad_first_kernel<KB>;
   static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
   bool& attr_set = attr_set_of[device_slot()];
