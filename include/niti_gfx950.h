@@ -240,6 +240,10 @@ int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int 
  * 16 or 32, C % 16 == 0, K % 16 == 0, N*H*W % 128 == 0, even N for side 8, N*H*W % 256 == 0 for sides 2 and 4) with
  * K*9*C <= 4M, rounding
  * NITI_ROUND_NEAREST or NITI_ROUND_PSEUDO_STOCHASTIC.  niti_conv2d_i8_wgrad_update_sync_words returns 0 otherwise.
+ * Two kinds of layer run as a single launch instead of the kernel pair: the first layer (side 32, C == 16 with
+ * w_channels <= 3, K 32 / 64 / 128 / 256: a workgroup per image adds its sums with integer atomics into extra zeroed
+ * sync words, the last workgroup to arrive rounds and updates - no workgroup waits for another) and layers on maps of
+ * side 2 and 4 with C % 32 == 0, K % 32 == 0 (a workgroup owns 32 x 32 channels x 9 taps over all pixels).
  *
  * act: [N,H,W,C] int8 (C may include zero channel padding); err: [N,H,W,K] int8; w: [K,3,3,w_channels] int8,
  * updated in place, w_channels <= C (gradient columns beyond w_channels are padding and are dropped).
