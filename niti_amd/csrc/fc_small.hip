@@ -459,6 +459,7 @@ constexpr int kHeadActPitch = kHeadGroups + 4; // words per feature row of the t
 
 // wait_slots for slots that hold two values: workgroup b stores (data-gradient maximum + 1) | (weight-gradient
 // maximum + 1) << 32 as one 8-byte word at slot b.  Called by a whole wavefront; nb <= 4096.
+static_assert(kSlotStride % 2 == 0, "a slot must hold an 8-byte aligned pair of words");
 __device__ inline void wait_slot_pairs(uint32_t* slots, int nb, long long spin_limit, uint32_t* timed_out, uint32_t* sticky,
                                        uint32_t& max_lo, uint32_t& max_hi) {
   const int lane = threadIdx.x & 63;
