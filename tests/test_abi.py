@@ -93,6 +93,28 @@ def test_argument_validation_without_a_gpu(lib):
     assert st == 1
     st = lib.niti_gemm_i8(0, 1, p, p, p, 0, 4, 4, 0, null, null, 0, null)
     assert st == 1
+    # classifier head and the generator's words: refused before any HIP call
+    st = lib.niti_head_i8_forward(p, p, p, 16, 10, 64, 3, null, null, 0, null, null, null, 7, 0, 0, 0, 0, p, 4096, null, null, null, null, null)
+    assert st == 1 and b"dropout" in lib.niti_last_error()                                        # dropout mode 3
+    st = lib.niti_head_i8_forward(p, p, p, 16, 10, 64, 2, p, null, 1, null, null, null, 7, 0, 0, 0, 0, p, 4096, null, null, null, null, null)
+    assert st == 1 and b"generator" in lib.niti_last_error()                                      # a drawn mask without a state
+    st = lib.niti_head_i8_forward(p, p, p, 16, 10, 64, 0, null, null, 0, p, null, null, 7, 0, 0, 0, 0, p, 4096, null, null, null, null, null)
+    assert st == 1 and b"loss gradient" in lib.niti_last_error()                                  # targets without an output
+    st = lib.niti_head_i8_forward(p, p, p, 16, 17, 64, 0, null, null, 0, null, null, null, 7, 0, 0, 0, 0, p, 4096, null, null, null, null, null)
+    assert st == 2                                                                                # 17 output features
+    st = lib.niti_head_i8_backward(p, p, null, p, p, 300, 10, 64, 7, 2, 5, 2, 0, 0, p, 4096, null, null, null, null, null, null, 0, null, null, null)
+    assert st == 2 and b"M <= 256" in lib.niti_last_error()
+    st = lib.niti_head_i8_backward(p, p, null, p, p, 16, 10, 64, 7, 1, 5, 2, 0, 0, p, 4096, null, null, null, null, null, null, 0, null, null, null)
+    assert st == 2 and b"random" in lib.niti_last_error()                                         # stochastic rounding
+    st = lib.niti_head_i8_backward(p, p, null, p, p, 16, 10, 64, 7, 2, 5, 2, 0, 0, p, 8, null, null, null, null, null, null, 0, null, null, null)
+    assert st == 3                                                                                # too few sync words
+    assert lib.niti_head_i8_sync_words(1, 16, 10, 64) > 16 and lib.niti_head_i8_sync_words(1, 16, 10, 96) == 0
+    assert lib.niti_head_i8_sync_words(0, 16, 10, 64) == lib.niti_fc_i8_sync_words(0, 16, 10, 64) > 0
+    assert lib.niti_rng_words_u32(null, 1, p, 4, null) == 1 and lib.niti_rng_words_u32(p, 1, null, 0, null) == 0
+    assert lib.niti_loss_grad_i8_rng(p, p, p, null, p, 4, 10, 0, null) == 1 and lib.niti_loss_grad_i8(p, p, p, null, p, 4, 10, 0, null) == 1
+    # the first layer's one-launch weight gradient wants its accumulation buffer behind the finishing kernel's slots
+    assert lib.niti_conv2d_i8_wgrad_update_sync_words(8, 32, 32, 16, 128, 3, 3, 1, 1) >= 16 + 128 * 32
+    assert lib.niti_conv2d_i8_wgrad_update_sync_words(8, 16, 16, 16, 128, 3, 3, 1, 1) < 128 * 32
     # empty inputs are fine
     assert lib.niti_absmax_i32(null, 0, null, null) == 0
     assert lib.niti_fill_u32(null, 0, 0, null) == 0
