@@ -452,22 +452,19 @@ def main():
 
     wl = ConvTriple(dev)
     run, mode = make_runner(wl.step, args.warmup, not args.eager)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
-    tops = wl.ops_per_step / (ms_per_step * 1e-3) / 1e12
     from niti_amd import ops as _ops
-    if _ops.sync_timeouts(dev):
-        print("bench.py: a grid-wide wait timed out during the timed steps (the GPU was shared with other work); "
-              "no result", file=sys.stderr)
-        return 4
-    # the same step replayed back to back for a second or more: clocks and temperature settle, unlike in the K-step burst
+    # The same step replayed back to back for a second or more.  It runs BEFORE the K timed steps: a process that has
+    # just initialised the device finds it in its idle power state, and the first tens of milliseconds of work run at
+    # lower clocks (K = 20 steps timed first read 5-6 % slower than the same 20 steps a second later).
     sustained = None
     if args.sustained_seconds > 0:
-        n_rep = max(int(args.sustained_seconds * 1e3 / ms_per_step * 1.15), args.steps)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            run()
+        torch.cuda.synchronize()
+        est_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+        n_rep = max(int(args.sustained_seconds * 1e3 / est_ms * 1.15), args.steps)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         for _ in range(n_rep):
@@ -475,9 +472,23 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         sustained = {"steps": n_rep, "seconds": round(dt, 3), "ms_per_step": round(dt * 1e3 / n_rep, 4),
-                     "tops": round(wl.ops_per_step * n_rep / dt / 1e12, 2)}
+                     "tops": round(wl.ops_per_step * n_rep / dt / 1e12, 2),
+                     "first_steps_after_idle_ms_per_step": round(est_ms, 4)}
         if _ops.sync_timeouts(dev):
             sustained["error"] = "a grid-wide wait timed out"
+        for _ in range(args.warmup):     # the W untimed steps in front of the timed ones
+            run()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    tops = wl.ops_per_step / (ms_per_step * 1e-3) / 1e12
+    if _ops.sync_timeouts(dev):
+        print("bench.py: a grid-wide wait timed out during the timed steps (the GPU was shared with other work); "
+              "no result", file=sys.stderr)
+        return 4
 
     # Dominant kernel: the MFMA implicit-GEMM convolution (forward + data-gradient launches), timed
     # per launch with HIP events on the launch stream over the same K steps run eagerly.  A device
