@@ -243,7 +243,8 @@ int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int 
  * Two kinds of layer run as a single launch instead of the kernel pair: the first layer (side 32, C == 16 with
  * w_channels <= 3, K 32 / 64 / 128 / 256: a workgroup per image adds its sums with integer atomics into extra zeroed
  * sync words, the last workgroup to arrive rounds and updates - no workgroup waits for another) and layers on maps of
- * side 2 and 4 with C % 32 == 0, K % 32 == 0 (a workgroup owns 32 x 32 channels x 9 taps over all pixels).
+ * side 2 and 4 with C % 32 == 0, K % 32 == 0 and at most 8192 pixels (a workgroup owns 32 x 32 channels x 9 taps over
+ * all pixels; for these any N is covered, not only N*H*W % 256 == 0).
  *
  * act: [N,H,W,C] int8 (C may include zero channel padding); err: [N,H,W,K] int8; w: [K,3,3,w_channels] int8,
  * updated in place, w_channels <= C (gradient columns beyond w_channels are padding and are dropped).

@@ -514,7 +514,7 @@ extern "C" int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_
 
 extern "C" size_t niti_conv2d_i8_wgrad_update_sync_words(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
   if (N <= 0 || H <= 0 || W <= 0 || C <= 0 || K <= 0 || R <= 0 || S <= 0 || stride <= 0 || pad < 0) return 0;
-  if (!wgrad3x3_supported(N, H, W, C, K, R, S, stride, pad)) return 0;
+  if (!wgrad3x3_supported(N, H, W, C, K, R, S, stride, pad) && !wgrad_small_shape(N, H, W, C, K, R, S, stride, pad)) return 0;
   const int nb = wgrad3x3_finish_blocks(C, K);
   return nb > 0 ? wgrad3x3_sync_words(nb) + wgrad_first_extra_words(H, C, K) : 0;
 }

@@ -236,6 +236,7 @@ int launch_wgrad_first_update(const int8_t* act, const int8_t* err, int8_t* w, i
                               uint32_t* sync, int32_t* accum, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
                               hipStream_t stream);
 // one-launch weight gradient + update for 4 x 4 and 2 x 2 maps (wgrad_small.hip); sync words as for the finishing kernel
+bool wgrad_small_shape(int N, int H, int W, int C, int K, int R, int S, int stride, int pad);
 bool wgrad_small_supported(int N, int H, int C, int K, int w_channels);
 int launch_wgrad_small_update(const int8_t* act, const int8_t* err, int8_t* w, int N, int H, int C, int K, bool roundtrip,
                               uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep, hipStream_t stream);

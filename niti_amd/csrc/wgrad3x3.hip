@@ -892,6 +892,8 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
     if ((e == nullptr || e[0] != '0') && wgrad_small_supported(N, H, C, K, w_channels))
       return launch_wgrad_small_update(act, err, w, N, H, C, K, roundtrip, sync, rq, g8, dw, wprep, stream);
   }
+  if (!wgrad3x3_supported(N, H, H, C, K, 3, 3, 1, 1))
+    return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: %d pixels on %d x %d maps run only as the one-launch kernel, which this call cannot use", N * H * H, H, H);
   static int resident_of[kDeviceSlots][2] = {};   // workgroups of 4 / 16 wavefronts the device holds at once
   int* const resident = resident_of[device_slot()];
   if (resident[0] == 0) {

@@ -224,18 +224,23 @@ int ws_resident() {
 
 }  // namespace
 
-// Whether the one-launch form covers the layer; sync words are those of the finishing kernel (never fewer slots).
-bool wgrad_small_supported(int N, int H, int C, int K, int w_channels) {
-  if (H != 2 && H != 4) return false;
-  if (C % 32 != 0 || K % 32 != 0 || w_channels != C) return false;
+// Shapes of the one-launch form (a host-side test, no device query): any batch size - a last stage that reaches past
+// the tensor reads zeros.  Sync words are those of the finishing kernel (never fewer slots).
+bool wgrad_small_shape(int N, int H, int W, int C, int K, int R, int S, int stride, int pad) {
+  if (R != 3 || S != 3 || stride != 1 || pad != 1 || H != W || (H != 2 && H != 4)) return false;
+  if (N <= 0 || C % 32 != 0 || K % 32 != 0) return false;
   const long long pix = static_cast<long long>(N) * H * H;
   if (pix * C >= 0x7fffffffLL || pix * K >= 0x7fffffffLL || static_cast<long long>(K) * 9 * C >= 0x7fffffffLL) return false;
   const long long nb = static_cast<long long>(C / 32) * (K / 32);
   if (nb > wgrad3x3_finish_blocks(C, K)) return false;   // the caller's sync words are sized for the finishing kernel
-  // long pixel ranges belong to the kernels that split them
-  if (pix > 8192) return false;
+  return pix <= 8192;                                     // long pixel ranges belong to the kernels that split them
+}
+
+// ... and whether this device holds all its workgroups at once
+bool wgrad_small_supported(int N, int H, int C, int K, int w_channels) {
+  if (w_channels != C || !wgrad_small_shape(N, H, H, C, K, 3, 3, 1, 1)) return false;
   const int resident = H == 2 ? ws_resident<2>() : ws_resident<4>();
-  return nb <= resident;
+  return static_cast<long long>(C / 32) * (K / 32) <= resident;
 }
 
 int launch_wgrad_small_update(const int8_t* act, const int8_t* err, int8_t* w, int N, int H, int C, int K, bool roundtrip,

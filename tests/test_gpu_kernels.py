@@ -455,7 +455,8 @@ def test_conv_wgrad_arrangements(dev, case, wgrad_arrangement):
 
 @pytest.mark.parametrize("case", [(4, 32, 16, 32), (8, 16, 128, 64), (6, 8, 80, 144), (64, 8, 64, 256), (16, 16, 256, 128),
                                   (2, 8, 16, 16), (4, 8, 3, 16), (8, 32, 3, 128), (32, 8, 512, 512), (16, 4, 64, 128), (64, 4, 512, 256), (64, 2, 128, 64), (256, 2, 512, 512),
-                                  (3, 32, 3, 64), (2, 32, 3, 32), (2, 32, 3, 256), (5, 32, 2, 64), (1, 32, 1, 128)])
+                                  (3, 32, 3, 64), (2, 32, 3, 32), (2, 32, 3, 256), (5, 32, 2, 64), (1, 32, 1, 128),
+                                  (8, 4, 64, 128), (3, 2, 32, 32), (37, 4, 96, 160), (300, 2, 64, 32)])   # any batch size on 4 x 4 / 2 x 2 maps
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 def test_conv_wgrad_update(dev, case, div_mode):
     """wgrad + grad_calc + weight update in one call against the oracle's three steps."""
