@@ -93,7 +93,7 @@ def test_rng_words_and_step(dev):
         assert [int(v) for v in _u32(rng)] == [key[0], key[1], step + 1, 0]
 
 
-HEAD_CASES = [(128, 10, 8192), (256, 10, 512), (20, 10, 512), (16, 7, 64), (33, 16, 1088), (1, 1, 64)]
+HEAD_CASES = [(128, 10, 8192), (256, 10, 512), (20, 10, 512), (16, 7, 64), (33, 16, 1088), (1, 1, 64), (24, 10, 32768)]
 
 
 @pytest.mark.gpu
@@ -171,7 +171,7 @@ def test_head_forward_loss_branches(dev):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("case", [(128, 10, 8192), (256, 10, 512), (20, 10, 512), (16, 7, 64), (33, 16, 1088), (1, 1, 64), (200, 3, 128)])
+@pytest.mark.parametrize("case", [(128, 10, 8192), (256, 10, 512), (20, 10, 512), (16, 7, 64), (33, 16, 1088), (1, 1, 64), (200, 3, 128), (24, 10, 32768)])
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 def test_head_backward(dev, case, div_mode):
     """niti_head_i8_backward against TiLinear.backward + TiDropout.backward of the oracle."""
