@@ -127,15 +127,18 @@ struct HGeom {
   // 512 pixels x 64 channels: both halves of the workgroup's wavefronts work on the same 64 channels, each on 256 of
   // the pixels (for launches of the 64-channel tile with more workgroups than the device holds at once)
   static constexpr bool TWO = PX == 512;
-  static constexpr int NWF = TWO ? 2 : KT / 64;            // 32-channel tiles per wavefront
-  static constexpr int RPS = (KT == 64 && !TWO) ? 3 : 1;   // filter rows per stage: the narrow tile takes a whole slice
+  // KT == 32 (launches that would otherwise leave compute units idle): 8 wavefronts of 32 pixels x 32 channels
+  static constexpr int PT = KT == 32 ? 1 : 2;              // 32-pixel tiles per wavefront
+  static constexpr int NWF = TWO ? 2 : (KT == 32 ? 1 : KT / 64);   // 32-channel tiles per wavefront
+  static constexpr int RPS = (KT <= 64 && !TWO) ? 3 : 1;   // filter rows per stage: the narrow tiles take a whole slice
   static constexpr int W_BYTES = RPS * 3 * KT * 32;        // one filter stage: RPS filter rows of three taps
   static constexpr int W_INSTR = W_BYTES / 1024;
   static constexpr int WSTAGES = 3;
   static constexpr int TILE_BYTES = 2 * ACT_BYTES + WSTAGES * W_BYTES;
   static constexpr int LDS_BYTES = TILE_BYTES + 1024;      // + dump slot / reduction words
   static_assert(PX == 256 || (PX == 512 && KT == 64), "a workgroup owns 256 output pixels, or 512 with the 64-channel tile");
-  static_assert(KT == 64 || KT == 128, "channel tile");
+  static_assert(KT == 32 || KT == 64 || KT == 128, "channel tile");
+  static_assert(KT != 32 || Q <= 16, "the 32-channel tile's wavefronts own 32 pixels: whole 2 x 2 windows only up to 16-pixel rows");
   static_assert(NI == 1 || BR == Q, "several images per workgroup only as whole images");
 };
 
@@ -247,6 +250,8 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       const int cs = min(kt * (KT / 32) + q % (KT / 32), a.src_cslices - 1);
       return (cs * 9 + 8 - q / (KT / 32)) * 2048 + lane * 16 - wback;
     }
+    if (KT == 32)   // instruction q = tap q: the tile's half (32 rows) of the 64-row group
+      return min(kt >> 1, ngroups - 1) * a.cslices * (9 * 2048) + q * 2048 + (kt & 1) * 1024 + lane * 16;
     const int g = min(KT == 128 ? kt * 2 + q / 6 : kt, ngroups - 1);
     return g * a.cslices * (9 * 2048) + (KT == 128 ? q % 6 : q) * 1024 + lane * 16;
   };
@@ -266,10 +271,11 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   };
 
   // ---- fragment addressing
-  const int wp_ = wave & 3;   // 64-pixel group
-  const int wc = wave >> 2;   // channel group of KT/2 (TWO: pixel half, all wavefronts share the 64 channels)
+  constexpr int PT = G::PT;
+  const int wp_ = KT == 32 ? wave : (wave & 3);   // group of 32 PT pixels
+  const int wc = KT == 32 ? 0 : (wave >> 2);      // channel group of KT/2 (TWO: pixel half, all wavefronts share the 64 channels)
   const int lr = lane & 31, lk = lane >> 5;
-  constexpr int TAPB = kWT ? (KT / 32) * 1024 : 2048;   // bytes between consecutive taps inside a stage
+  constexpr int TAPB = (kWT || KT == 32) ? (KT / 32) * 1024 : 2048;   // bytes between consecutive taps inside a stage
   int w_addr[NWF][kWT ? 2 : 1];   // this lane's filter row(s) inside a stage, tap 0
 #pragma unroll
   for (int i = 0; i < NWF; ++i) {
@@ -288,10 +294,10 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       w_addr[i][0] = (KT == 128 ? wc * 6144 : 0) + grow * 32 + ((lk ^ ((grow >> 3) & 1)) << 4);
     }
   }
-  int p_addr[2];              // [pixel tile]: halo slot of this lane's pixel, filter row 0
+  int p_addr[PT];             // [pixel tile]: halo slot of this lane's pixel, filter row 0
 #pragma unroll
-  for (int j = 0; j < 2; ++j) {
-    const int pix = (G::TWO ? wc * 256 : 0) + wp_ * 64 + j * 32 + lr;   // output pixel inside the workgroup's share
+  for (int j = 0; j < PT; ++j) {
+    const int pix = (G::TWO ? wc * 256 : 0) + wp_ * (32 * PT) + j * 32 + lr;   // output pixel inside the workgroup's share
     const int prow = pix / Q, pw = pix % Q;        // row inside the workgroup's rows, column
     const int hrow = (prow / BR) * G::HR + (prow % BR);
     p_addr[j] = (hrow * G::RP + pw) * 32 + ((lk ^ (((pw >> 3) ^ hrow) & 1)) << 4);
@@ -300,11 +306,11 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const int keep_l = (lr % Q) != 0 ? -1 : 0;
   const int keep_r = (lr % Q) != Q - 1 ? -1 : 0;
 
-  v16i acc[NWF][2];  // [channel tile][pixel tile]
+  v16i acc[NWF][PT];  // [channel tile][pixel tile]
 #pragma unroll
   for (int i = 0; i < NWF; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < PT; ++j)
 #pragma unroll
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
@@ -313,9 +319,9 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const int roff = r * G::RP * 32;
     // pixels under the centre column of this filter row; the fragment layout is lane -> (pixel lane % 32,
     // 16 channels lane / 32), so the pixel to the left is one lane down and the one to the right one lane up
-    v4i pc[2];
+    v4i pc[PT];
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < PT; ++j) {
       const int at = (p_addr[j] + roff) ^ ((r & 1) << 4);
       if constexpr (kWT) pc[j] = lds_read_b128(lds_addr(sa) + at);   // counted by hand like the filter reads behind it
       else pc[j] = *reinterpret_cast<const v4i*>(sa + at);
@@ -349,7 +355,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         lds_settle<(2 - s) * 2 * NWF>();
         if (s == 0) {
 #pragma unroll
-          for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(pc[j]));
+          for (int j = 0; j < PT; ++j) asm volatile("" : "+v"(pc[j]));
         }
 #pragma unroll
         for (int i = 0; i < NWF; ++i) wf[s][i] = lds_landed(tlo[s][i], thi[s][i]);
@@ -359,26 +365,26 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
-    v4i ps[2];
+      for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
+    v4i ps[PT];
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < PT; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
     tap_ready(std::integral_constant<int, 1>{});
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < PT; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
     tap_ready(std::integral_constant<int, 2>{});
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
 #pragma unroll
-      for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
+      for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
   };
 
   // A whole slice (three filter rows) from one stage, for the pipeline with one slice per stage.  All fragment reads
@@ -387,16 +393,16 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   // to itself the compiler keeps the fragments in few registers and alternates read, wait, product.)
   auto stage_rows = [&](unsigned saa, unsigned swa) {
     constexpr int PER_TAP = NWF * (kWT ? 2 : 1);
-    constexpr int ROW_READS = 2 + 3 * PER_TAP;
+    constexpr int ROW_READS = PT + 3 * PER_TAP;
     static_assert(ROW_READS <= 15, "the wait counter holds 15");
-    v4i pcb[2][2];
+    v4i pcb[2][PT];
     v4i wfb[2][3][NWF];
     v2i tlo[2][3][NWF], thi[2][3][NWF];
     auto request = [&](auto rc) {
       constexpr int r = decltype(rc)::value;
       constexpr int b = r & 1;
 #pragma unroll
-      for (int j = 0; j < 2; ++j) pcb[b][j] = lds_read_b128_at<r * G::RP * 32>(saa + (p_addr[j] ^ ((r & 1) << 4)));
+      for (int j = 0; j < PT; ++j) pcb[b][j] = lds_read_b128_at<r * G::RP * 32>(saa + (p_addr[j] ^ ((r & 1) << 4)));
       static_for<3>([&](auto sc) {
         constexpr int s = decltype(sc)::value;
         constexpr int off = ((s + 1) % 3 + 3 * r) * TAPB;
@@ -417,9 +423,9 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       constexpr int b = r & 1;
       if constexpr (r < 2) request(std::integral_constant<int, r + 1>{});
       lds_settle<(r < 2) ? ROW_READS : 0>();
-      v4i pc[2], wf[3][NWF];
+      v4i pc[PT], wf[3][NWF];
 #pragma unroll
-      for (int j = 0; j < 2; ++j) {
+      for (int j = 0; j < PT; ++j) {
         pc[j] = pcb[b][j];
         asm volatile("" : "+v"(pc[j]));
       }
@@ -437,24 +443,24 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
-      v4i ps[2];
+        for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
+      v4i ps[PT];
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < PT; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < PT; ++j)
 #pragma unroll
         for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
+        for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);   // the next row's requests and wait stay behind these products
     });
   };
@@ -521,7 +527,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
   for (int i = 0; i < NWF; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < PT; ++j)
 #pragma unroll
       for (int e = 0; e < 16; e += 2) {
         vmax = max(vmax, max(acc[i][j][e], acc[i][j][e + 1]));
@@ -539,7 +545,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const uint32_t lmax = max(static_cast<uint32_t>(vmax), 0u - static_cast<uint32_t>(vmin));
   const long long total_pix = static_cast<long long>(a.N) * Q * Q;
   const int chbase = G::TWO ? kt * KT : kt * KT + wc * (KT / 2);
-  const int pixwave = pixbase + (G::TWO ? wc * 256 : 0) + wp_ * 64;   // first pixel of this wavefront
+  const int pixwave = pixbase + (G::TWO ? wc * 256 : 0) + wp_ * (32 * PT);   // first pixel of this wavefront
   uint32_t* const red = reinterpret_cast<uint32_t*>(dump);  // behind the tiles, clear of the patches below
   if constexpr (!kFused) {
     hc_sync();  // all wavefronts are done with the tiles: reuse LDS as per-wavefront transposition patches
@@ -548,7 +554,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const int rrow = lane >> 3, rcol = lane & 7;  // 8 lanes x 16 bytes = one 32-channel row
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.y_bytes, 0x00020000);
 #pragma unroll
-    for (int j = 0; j < 2; ++j) {
+    for (int j = 0; j < PT; ++j) {
       const int mrow = pixwave + j * 32 + rrow;
 #pragma unroll
       for (int i = 0; i < NWF; ++i) {
@@ -635,7 +641,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
     const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
     constexpr int PROW = NWF * 32 + 16;  // the wavefront's channels of one pixel, padded
-    int8_t* patch = smem + wave * (64 * PROW);
+    int8_t* patch = smem + wave * (32 * PT * PROW);
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y8, 0, a.y8_bytes, 0x00020000);
     constexpr int LPP = NWF * 2;       // lanes (16-byte pieces) per pixel
     constexpr int PPI = 64 / LPP;      // pixels per store instruction
@@ -645,7 +651,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j)
+        for (int j = 0; j < PT; ++j)
 #pragma unroll
           for (int e = 0; e < 16; ++e) acc[i][j][e] = f32_roundtrip(acc[i][j][e]);
     }
@@ -656,13 +662,13 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) asm volatile("" : "+v"(acc[i][j]));
+        for (int j = 0; j < PT; ++j) asm volatile("" : "+v"(acc[i][j]));
       // round, pack four channels per dword, transpose through a per-wavefront patch, store 16-byte pieces; the
       // common rounding mode gets a short form
       const bool fast = shift >= 1 && !trunc && !psto;
       const int sm1 = shift - 1, lo = relu ? 0 : -127;
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < PT; ++j)
 #pragma unroll
         for (int i = 0; i < NWF; ++i)
 #pragma unroll
@@ -683,7 +689,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
           }
       // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
 #pragma unroll
-      for (int t = 0; t < 64 / PPI; ++t) {
+      for (int t = 0; t < 32 * PT / PPI; ++t) {
         const int pl = t * PPI + prow;
         v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
         const int m = pixwave + pl;
@@ -735,7 +741,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         // strip of whole image rows (or whole images), i.e. 16 whole 2 x 2 windows; a lane takes 16 channels of one.
         constexpr int PC = Q / 2;   // pooled pixels per row
         const int pq = lane / LPP;
-        if (pq < 16) {
+        if (pq < 8 * PT) {
           const int l0 = 2 * (pq / PC) * Q + 2 * (pq % PC);   // upper left pixel of the window inside the strip
           const int8_t* src = patch + l0 * PROW + piece * 16;
           const v4i p00 = *reinterpret_cast<const v4i*>(src), p01 = *reinterpret_cast<const v4i*>(src + PROW);
@@ -1050,6 +1056,9 @@ int halo_ktile(long long pix, int K, int H) {
   const char* e = getenv("NITI_HALO_KT");  // tests and tuning runs pin the tile
   const int forced = e != nullptr ? atoi(e) : 0;
   if (forced == 128 || forced == 64) return forced;
+  if (forced == 32 && H <= 16) return 32;
+  // fewer 64-channel tiles than compute units on the small maps: tiles of 32 channels, twice as many workgroups
+  if (forced == 0 && H <= 8 && K > 32 && (pix / 256) * ((K + 63) / 64) < cus) return 32;
   if (K <= 64) return 64;   // nothing to gain from computing 128 channels
   const long long b128 = (pix / 256) * ((K + 127) / 128);
   return (b128 < 2LL * cus && K > 64) ? 64 : 128;
@@ -1070,7 +1079,7 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
   using G = HGeom<Q, BR, NI, KT>;
   constexpr size_t lds = G::LDS_BYTES;
   static_assert(8 * 32 * (32 * 4 + 16) <= G::TILE_BYTES, "int32 patches must stay clear of the reduction words");
-  static_assert(8 * 64 * (G::NWF * 32 + 16) <= G::TILE_BYTES, "int8 patches must stay clear of the reduction words");
+  static_assert(8 * 32 * G::PT * (G::NWF * 32 + 16) <= G::TILE_BYTES, "int8 patches must stay clear of the reduction words");
   static_assert(2 * lds <= 160 * 1024, "two workgroups per compute unit");
   auto k = conv3x3_halo_kernel<Q, BR, NI, KT, kFused, kWT>;
   static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
@@ -1148,6 +1157,11 @@ int launch_halo_tiles(const HaloArgs& a, int H, hipStream_t stream) {
     if (H == 16) return launch_halo<16, 16, 1, 128, kFused, kWT>(a, stream);
     if (H == 8) return launch_halo<8, 8, 4, 128, kFused, kWT>(a, stream);
     return launch_halo<4, 4, 16, 128, kFused, kWT>(a, stream);
+  }
+  if (ktile == 32) {
+    if (H == 16) return launch_halo<16, 16, 1, 32, kFused, kWT>(a, stream);
+    if (H == 8) return launch_halo<8, 8, 4, 32, kFused, kWT>(a, stream);
+    return launch_halo<4, 4, 16, 32, kFused, kWT>(a, stream);
   }
   if constexpr (kFused) {
     if (halo_two_pixel_tiles(static_cast<long long>(a.N) * H * H, a.K, H, ktile)) {

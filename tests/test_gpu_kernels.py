@@ -114,7 +114,7 @@ FUSED_CASES = [(4, 8, 16, 16), (4, 8, 64, 128), (8, 8, 80, 144), (1, 16, 16, 48)
                (264, 16, 16, 272), (600, 32, 16, 48)]
 
 
-@pytest.fixture(params=["auto", "64", "128"])
+@pytest.fixture(params=["auto", "32", "64", "128"])
 def halo_tile(request):
     """Channel tile of the 3x3 halo kernel: the library's own choice, or pinned to either width."""
     import os
