@@ -796,13 +796,21 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 constexpr int kMap2Depth = 8;                               // reduction steps with their loads in flight, per wavefront
 constexpr int kMap2RedBytes = 4 * 64 * 16 * 4;              // sums of the second reduction half
 constexpr int kMap2StageBytes = 8 * kMap2Depth * 1024;      // kWT: filter blocks in flight, all wavefronts
-constexpr size_t map2_lds_bytes(bool wt) { return static_cast<size_t>(kMap2RedBytes) + 64 + (wt ? kMap2StageBytes : 0); }
+constexpr int kMap2ActMaxC = 512;                           // kLdsAct: input channels whose activations fit in LDS
+constexpr size_t map2_fixed_lds(bool wt) { return static_cast<size_t>(kMap2RedBytes) + 64 + (wt ? kMap2StageBytes : 0); }
+// kLdsAct: the workgroup's activations (32 images x 4 pixels x C) behind the rest, rows of 4 C + 16 bytes (the 16
+// spread the 32 images of a fragment read over the banks)
+constexpr size_t map2_lds_bytes(bool wt, int act_c) { return map2_fixed_lds(wt) + (act_c > 0 ? static_cast<size_t>(32) * (4 * act_c + 16) : 0); }
 
-template <bool kFused, bool kWT>
+// kLdsAct: the four wavefronts of a reduction half multiply the same activation fragments (with different taps), so
+// the workgroup stages its activations in LDS once and every wavefront reads its fragments there: 1.25 KB instead of
+// 2 KB per step come through the vector memory path, which is what bounds this kernel.
+template <bool kFused, bool kWT, bool kLdsAct>
 __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int itiles) {
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   int* const red = reinterpret_cast<int*>(smem);                                      // [p][4][64] x 16 bytes
   uint32_t* const words = reinterpret_cast<uint32_t*>(smem + kMap2RedBytes);          // 4 maxima, the range
+  int8_t* const act_s = smem + map2_fixed_lds(kWT);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -838,6 +846,19 @@ __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int
   }
   int8_t* const stage = smem + kMap2RedBytes + 64 + wave * (kMap2Depth * 1024);
 
+  const int act_pitch = 4 * a.C + 16;
+  if (kLdsAct) {
+    // rows = images, 4 C bytes each (the four pixels in a row); 16-byte pieces, coalesced
+    const int pieces = a.C >> 2;                          // 16-byte pieces of an image: 4 pixels x C / 16
+    for (int i = tid; i < 32 * pieces; i += 512) {
+      const int img = i / pieces, pc = i - img * pieces;
+      const int nn = it * 32 + img;
+      const v4i v = __builtin_amdgcn_raw_buffer_load_b128(rx, nn < a.N ? nn * 4 * a.C + pc * 16 : kOob, 0, 0);
+      *reinterpret_cast<v4i*>(act_s + img * act_pitch + pc * 16) = v;
+    }
+    __syncthreads();
+  }
+  const int8_t* const act_lane = act_s + lr * act_pitch + lk * 16;
   v4i fa[kMap2Depth], fw[kMap2Depth];
   // Loads of step s into slot u.  Steps past the wavefront's last one are issued all the same, with out-of-range
   // offsets (zeros, no memory traffic): the loop body is free of branches, so the number of loads in flight behind
@@ -848,7 +869,7 @@ __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int
     const bool live = s < nsteps;
     int aoff = kOob;
     if (live && a_base != kOob && cs * 32 + lk * 16 < a.C) aoff = a_base + q * a.C + cs * 32;
-    fa[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, aoff, 0, 0);
+    if (!kLdsAct) fa[u] = __builtin_amdgcn_raw_buffer_load_b128(rx, aoff, 0, 0);
     if (kWT) {
       // forward copy [reduction group of 64][this launch's output slice][flipped tap][64 rows][32 bytes]
       const int blk = (((cs >> 1) * a.src_cslices + kt) * 9 + 8 - tap) * 2048 + (cs & 1) * 1024;
@@ -869,14 +890,20 @@ __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int
 #pragma unroll
     for (int u = 0; u < kMap2Depth; ++u) {
       if (kWT) {
-        // two loads per step, completing in order: all but those of the seven younger steps have landed
-        __builtin_amdgcn_s_waitcnt(0x0F70 | (2 * (kMap2Depth - 1)));
+        // two loads per step (one with the activations in LDS), completing in order: all but those of the seven younger
+        // steps have landed
+        __builtin_amdgcn_s_waitcnt(0x0F70 | ((kLdsAct ? 1 : 2) * (kMap2Depth - 1)));
         asm volatile("" ::: "memory");
         const unsigned src = lds_addr(stage + u * 1024);
         const v2i lo = lds_read_tr8<0>(src + w_frag[0]);
         const v2i hi = lds_read_tr8<0>(src + w_frag[1]);
         lds_settle<0>();   // also: the slot is read out before the next block is sent to it
         fw[u] = lds_landed(lo, hi);
+      }
+      if (kLdsAct) {
+        const int st = base + u;                             // steps past the last one read slice 0 (their filter fragments are zero)
+        const int cs = st < nsteps ? cs0 + (st >> 2) : 0;
+        fa[u] = *reinterpret_cast<const v4i*>(act_lane + (st & 3) * a.C + cs * 32);
       }
       acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[u], fa[u], acc, 0, 0, 0);
       issue(base + u + kMap2Depth, u);
@@ -1119,10 +1146,10 @@ int launch_halo(const HaloArgs& a, hipStream_t stream) {
 
 inline int map2_blocks(int N, int K) { return ((N + 31) / 32) * ((K + 31) / 32); }
 
-template <bool kFused, bool kWT>
-int launch_map2(const HaloArgs& a, hipStream_t stream) {
-  constexpr size_t lds = map2_lds_bytes(kWT);
-  auto k = conv3x3_map2_kernel<kFused, kWT>;
+template <bool kFused, bool kWT, bool kLdsAct>
+int launch_map2_as(const HaloArgs& a, hipStream_t stream) {
+  constexpr size_t lds = map2_lds_bytes(kWT, kLdsAct ? kMap2ActMaxC : 0);
+  auto k = conv3x3_map2_kernel<kFused, kWT, kLdsAct>;
   static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
   static int resident_of[kDeviceSlots] = {};     // workgroups the device holds at once
   const int slot = device_slot();
@@ -1142,10 +1169,21 @@ int launch_map2(const HaloArgs& a, hipStream_t stream) {
   }
   const int itiles = (a.N + 31) / 32;
   const int nb = map2_blocks(a.N, a.K);
-  if (kFused && nb > resident)
+  if (kFused && nb > resident) {
+    // the variant with its activations in LDS holds fewer workgroups per compute unit: the direct loads may still fit
+    if constexpr (kLdsAct) return launch_map2_as<kFused, kWT, false>(a, stream);
     return fail(NITI_ERR_UNSUPPORTED, "conv3x3_map2: %d workgroups do not fit on the device at once (%d)", nb, resident);
+  }
   hipLaunchKernelGGL(k, dim3(nb), dim3(512), lds, stream, a, itiles);
   return check_launch("conv3x3_map2");
+}
+
+template <bool kFused, bool kWT>
+int launch_map2(const HaloArgs& a, hipStream_t stream) {
+  // activations through LDS where a workgroup's share fits (NITI_MAP2_LDS=0 pins the direct loads)
+  const char* e = getenv("NITI_MAP2_LDS");
+  if (a.C <= kMap2ActMaxC && a.C % 32 == 0 && (e == nullptr || e[0] != '0')) return launch_map2_as<kFused, kWT, true>(a, stream);
+  return launch_map2_as<kFused, kWT, false>(a, stream);
 }
 
 template <bool kFused, bool kWT>
