@@ -158,31 +158,50 @@ class ConvTriple:
                 self.wgrad_events.append((e0, e1, conv_ops(BATCH, hw, c, k), i, "wgrad"))
 
 
-def make_runner(step_fn, warmup, use_graph=True):
-    """Warm up eagerly, then capture one step into a HIP graph (launch-bound chains of small kernels
-    replay without per-launch host cost).  Returns (callable, "graph" | "eager")."""
-    import torch
-    side = torch.cuda.Stream()
-    side.wait_stream(torch.cuda.current_stream())
-    with torch.cuda.stream(side):
-        for _ in range(max(warmup, 3)):
-            step_fn()
-    torch.cuda.current_stream().wait_stream(side)
-    torch.cuda.synchronize()
-    if not use_graph:
-        return step_fn, "eager"
-    try:
-        g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
-            step_fn()
-        for _ in range(2):
-            g.replay()
+class Runner:
+    """Runs exactly n steps per call of run(n).  Warm up eagerly, then capture the step into HIP graphs (launch-bound
+    chains of small kernels replay without per-launch host cost): one graph of a single step and, with unroll > 1, one
+    of `unroll` consecutive steps - two consecutive graph launches leave the device idle for some microseconds, a
+    longer graph has fewer such seams.  n steps = n // unroll replays of the long graph + n % unroll of the short one."""
+
+    def __init__(self, step_fn, warmup, use_graph=True, unroll=1):
+        import torch
+        self.step_fn, self.mode, self.unroll, self.graphs = step_fn, "eager", 1, None
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(max(warmup, 3)):
+                step_fn()
+        torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
-        return g.replay, "graph"
-    except Exception as e:  # capture refused: keep measuring, say so
-        print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
-        torch.cuda.synchronize()
-        return step_fn, "eager"
+        if not use_graph:
+            return
+        try:
+            graphs = []
+            for u in ([1, unroll] if unroll > 1 else [1]):
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    for _ in range(u):
+                        step_fn()
+                g.replay()
+                torch.cuda.synchronize()
+                graphs.append(g)
+            self.graphs, self.mode, self.unroll = graphs, "graph", max(unroll, 1)
+        except Exception as e:  # capture refused: keep measuring, say so
+            print("bench.py: graph capture failed (%s); timing eager launches" % e, file=sys.stderr)
+            torch.cuda.synchronize()
+
+    def run(self, n=1):
+        if self.graphs is None:
+            for _ in range(n):
+                self.step_fn()
+            return
+        if self.unroll > 1:
+            for _ in range(n // self.unroll):
+                self.graphs[1].replay()
+            n %= self.unroll
+        for _ in range(n):
+            self.graphs[0].replay()
 
 
 def cpu_baseline(min_seconds=10.0):
@@ -214,7 +233,7 @@ def cpu_baseline(min_seconds=10.0):
             "sample": "%d pass(es) of the full six-layer conv triple at batch %d (plain-C oracle, OpenMP), %.1f s" % (passes, BATCH, t_total)}
 
 
-def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH, graph=True):
+def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH, graph=True, unroll=1):
     """images/s of a complete integer training step: VGG-small (six conv + FC), batch 128 (configs[3]), or the
     ten-convolution VGG-13 widths, batch 256 (configs[4])."""
     import torch
@@ -235,14 +254,14 @@ def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH, graph=True):
         net.forward_int8(x, 0, target)      # the targets are known: the classifier's forward launch evaluates the loss gradient
         net.backward(target)
 
-    run, mode = make_runner(one, warmup, graph)
+    runner = Runner(one, warmup, graph, unroll)
+    runner.run(max(steps, 2 * runner.unroll))      # the clocks settle, both graphs have run
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(steps):
-        run()
+    runner.run(steps)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / steps
-    return batch / dt, dt * 1e3, mode
+    return batch / dt, dt * 1e3, runner.mode
 
 
 def _avg_us(fn, reps=20, warm=3):
@@ -389,12 +408,13 @@ TRAIN_STEPS = (("train_step", 7, BATCH, "BASELINE configs[3]: VGG-small (6 conv 
                ("train_step_vgg13", 13, 256, "BASELINE configs[4]: VGG-13 widths (10 conv + FC) integer training step, batch 256"))
 
 
-def train_step_objects(dev, steps, warmup, graph=True):
+def train_step_objects(dev, steps, warmup, graph=True, unroll=1):
     out = {}
     for name, depth, batch, workload in TRAIN_STEPS:
         try:
-            ips, ms, mode = train_step_rate(dev, steps, warmup, depth, batch, graph)
-            out[name] = {"workload": workload, "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": mode}
+            ips, ms, mode = train_step_rate(dev, steps, warmup, depth, batch, graph, unroll)
+            out[name] = {"workload": workload, "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": mode,
+                         "steps_per_graph": unroll if mode == "graph" else None}
         except Exception as e:  # the headline line must still be printed
             out[name] = {"error": str(e)[:200]}
     return out
@@ -415,6 +435,8 @@ def main():
     ap.add_argument("--side-workloads-only", action="store_true",
                     help="run only config0 / config1 / max-pool and the MFMA probe and print their objects (for kernel traces)")
     ap.add_argument("--eager", action="store_true", help="time eager launches instead of a captured HIP graph")
+    ap.add_argument("--steps-per-graph", type=int, default=1,
+                    help="consecutive steps captured into one HIP graph (K steps = K // U replays of it + K %% U of a one-step graph)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run three plain 256 MiB device copies (a kernel of known traffic, to scale "
                          "rocprofv3 FETCH_SIZE / WRITE_SIZE readings)")
@@ -447,11 +469,12 @@ def main():
         return 0
 
     if args.train_steps_only:
-        print(json.dumps(train_step_objects(dev, args.steps, args.warmup, not args.eager)))
+        print(json.dumps(train_step_objects(dev, args.steps, args.warmup, not args.eager, args.steps_per_graph)))
         return 0
 
     wl = ConvTriple(dev)
-    run, mode = make_runner(wl.step, args.warmup, not args.eager)
+    runner = Runner(wl.step, args.warmup, not args.eager, args.steps_per_graph)
+    mode = runner.mode
     from niti_amd import ops as _ops
     # The same step replayed back to back for a second or more.  It runs BEFORE the K timed steps: a process that has
     # just initialised the device finds it in its idle power state, and the first tens of milliseconds of work run at
@@ -460,15 +483,13 @@ def main():
     if args.sustained_seconds > 0:
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(args.steps):
-            run()
+        runner.run(args.steps)
         torch.cuda.synchronize()
         est_ms = (time.perf_counter() - t0) * 1e3 / args.steps
         n_rep = max(int(args.sustained_seconds * 1e3 / est_ms * 1.15), args.steps)
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(n_rep):
-            run()
+        runner.run(n_rep)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         sustained = {"steps": n_rep, "seconds": round(dt, 3), "ms_per_step": round(dt * 1e3 / n_rep, 4),
@@ -476,12 +497,10 @@ def main():
                      "first_steps_after_idle_ms_per_step": round(est_ms, 4)}
         if _ops.sync_timeouts(dev):
             sustained["error"] = "a grid-wide wait timed out"
-        for _ in range(args.warmup):     # the W untimed steps in front of the timed ones
-            run()
+        runner.run(args.warmup)     # the W untimed steps in front of the timed ones
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    for _ in range(args.steps):
-        run()
+    runner.run(args.steps)
     torch.cuda.synchronize()
     ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
     tops = wl.ops_per_step / (ms_per_step * 1e-3) / 1e12
@@ -552,7 +571,7 @@ def main():
                                   "wgrad + grad rounding + weight update) over the six VGG-small conv shapes, batch 128, "
                                   "3x3 pad 1, uniform int8 inputs, Laplace int8 errors",
                       "ops_per_step": wl.ops_per_step, "batch": BATCH},
-           "launch_mode": mode,
+           "launch_mode": mode, "steps_per_graph": runner.unroll if mode == "graph" else None,
            "pct_int8_mfma_peak": round(100.0 * tops / INT8_MFMA_PEAK_TOPS, 2),
            "roofline": roofline, "per_layer": per_layer}
     try:
@@ -570,7 +589,7 @@ def main():
         except Exception as e:  # the headline line must still be printed
             out["side_workloads_error"] = str(e)[:300]
     if not args.no_train_step:
-        out.update(train_step_objects(dev, max(args.steps, 5), max(args.warmup, 2)))
+        out.update(train_step_objects(dev, max(args.steps, 5), max(args.warmup, 2), True, args.steps_per_graph))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
     print(json.dumps(out))
