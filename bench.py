@@ -389,8 +389,18 @@ def side_workloads(dev):
         fc[name + "_gbs"] = round(nbytes / t * 1e-3, 1)
         fc[name + "_frac_hbm"] = round(nbytes / t * 1e-3 / HBM_PEAK_GBS, 4)
         fc[name + "_tops"] = round(2.0 * M * Fin * O / t * 1e-6, 1)
+    # the drop-in int32 products of the extension boundary, operands as the reference hands them over
+    # (ti_torch.py:246,259,263: [m,k] and [k,n] row-major, the result the transposed view of an [n,m] buffer)
+    from niti_amd.shims import int8mm_cuda
+    Wt, Gt = W.t().contiguous(), G.t().contiguous()
+    for name, lhs, rhs in (("fwd", A, Wt), ("dgrad", G, W), ("wgrad", Gt, A)):
+        m_, k_, n_ = lhs.shape[0], lhs.shape[1], rhs.shape[1]
+        t = _avg_us(lambda: int8mm_cuda.int8_mm(lhs, rhs))
+        fc["dropin_int8_mm_" + name + "_us"] = round(t, 2)
+        fc["dropin_int8_mm_" + name + "_gbs"] = round((m_ * k_ + k_ * n_ + 4 * m_ * n_) / t * 1e-3, 1)
+    fc["dropin_note"] = "int8mm_cuda.int8_mm(lhs, rhs) -> int32, one launch, operands read as stored; bytes = m k + k n + 4 m n"
     out["config1"] = fc
-    del A, W, G, u_f, u_d, u_w, Wu
+    del A, W, G, u_f, u_d, u_w, Wu, Wt, Gt
     # ---- max-pool
     xp = torch.randint(-127, 128, (128, 32, 32, 128), generator=g, dtype=torch.int8).to(dev)
     yp = ops.maxpool_fwd(xp)

@@ -182,6 +182,12 @@ struct ConvProblem {
 };
 int launch_conv_igemm(const ConvProblem& p, hipStream_t stream);
 
+// int32 GEMM of operands with a slow reduction index (NN: b as [k][n]; TN: a as [k][m] too; TT: a as [k][m], b as
+// [n][k]), read as stored
+bool gemm_kmajor_shape(int trans_a, int trans_b, int m, int n, int k);
+int launch_gemm_kmajor(int trans_a, int trans_b, const int8_t* a, const int8_t* b, int32_t* c, int m, int n, int k, bool roundtrip,
+                       uint32_t* absmax, hipStream_t stream);
+
 int launch_fill_u32(uint32_t* dst, int64_t n, uint32_t value, hipStream_t stream);
 // dst[c][r][s][k] = w[k][R-1-r][S-1-s][c]
 int launch_filter_flip_transpose(const int8_t* w, int8_t* dst, int K, int R, int S, int C, hipStream_t stream);

@@ -394,8 +394,9 @@ def conv2d_wgrad_update(act, err, w, stride=1, padding=1, f32_epilogue=False, mu
     return g8, dw, shift_out, sync
 
 
-def gemm(a, b, trans_a=False, trans_b=False, absmax=None, out=None):
-    """c[m,n] = op(a) @ op(b), int8 x int8 -> int32.  trans_a: a stored [k,m]; trans_b: b stored [n,k]."""
+def gemm(a, b, trans_a=False, trans_b=False, absmax=None, out=None, f32_epilogue=False):
+    """c[m,n] = op(a) @ op(b), int8 x int8 -> int32.  trans_a: a stored [k,m]; trans_b: b stored [n,k].
+    f32_epilogue: every sum takes the int32 -> float32 -> int32 round trip of the reference's convolution epilogue."""
     _chk_dev(a, b, absmax, out)
     if a.dtype != torch.int8 or b.dtype != torch.int8:
         raise RuntimeError("gemm: int8 tensors expected")
@@ -406,7 +407,8 @@ def gemm(a, b, trans_a=False, trans_b=False, absmax=None, out=None):
     c = out if out is not None else torch.empty((m, n), dtype=torch.int32, device=a.device)
     nbytes = L.lib().niti_gemm_i8_workspace(int(trans_a), int(trans_b), m, n, k)
     ws = torch.empty(nbytes, dtype=torch.int8, device=a.device) if nbytes else None
-    st = L.lib().niti_gemm_i8(int(trans_a), int(trans_b), _ptr(a), _ptr(b), _ptr(c), m, n, k, 0, _ptr(absmax),
+    st = L.lib().niti_gemm_i8(int(trans_a), int(trans_b), _ptr(a), _ptr(b), _ptr(c), m, n, k,
+                              L.EPI_F32_ROUNDTRIP if f32_epilogue else 0, _ptr(absmax),
                               _ptr(ws), nbytes, _stream(a))
     L.check(st, "niti_gemm_i8")
     return c

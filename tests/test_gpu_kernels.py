@@ -617,7 +617,11 @@ def test_conv_wgrad(dev, case):
     assert int(am.cpu()) == po.absmax(ref)
 
 
-GEMM_CASES = [(128, 10, 8192), (16, 16, 16), (128, 128, 64), (100, 10, 512), (7, 5, 3), (130, 70, 100), (128, 1024, 1024), (33, 12, 8192)]
+# the last six take the kernel that reads operands with a slow reduction index as stored (n and k multiples of 32):
+# several staged chunks, a chunk tail, row counts that are not multiples of the 128-row tile, the three products of a
+# fully connected layer 8192 -> 1024 on a batch of 128
+GEMM_CASES = [(128, 10, 8192), (16, 16, 16), (128, 128, 64), (100, 10, 512), (7, 5, 3), (130, 70, 100), (128, 1024, 1024), (33, 12, 8192),
+              (48, 32, 32), (200, 64, 96), (160, 96, 2080), (64, 7, 1056), (128, 1024, 8192), (128, 8192, 1024), (1024, 8192, 128)]
 
 
 @pytest.mark.parametrize("mnk", GEMM_CASES)
@@ -636,6 +640,34 @@ def test_gemm(dev, mnk, ta, tb):
     c = ops.gemm(a, b, ta, tb, absmax=am)
     assert torch.equal(c.cpu(), ref)
     assert int(am.cpu()) == po.absmax(ref)
+
+
+@pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (True, True)])
+def test_gemm_f32_epilogue_above_2_24(dev, ta, tb):
+    """Sums beyond 2**24 through the kernel that reads both operands as stored: with the flag every sum takes the
+    reference epilogue's int32 -> float32 -> int32 round trip (linear_combination_clamp.h:371-389), without it none."""
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    _say("gemm f32 epilogue", ta, tb)
+    g = torch.Generator().manual_seed(411)
+    m, n, k = 160, 64, 2080
+    A, B = ri8(g, m, k), ri8(g, k, n)
+    A[:40] = 127
+    B[:, :20] = 127
+    B[:, 20:30] = -127
+    B[5, :30] = 126          # odd sums: not representable in float32 above 2**24
+    ref = po.int8mm(A, B)
+    assert int(ref.abs().max()) > 2 ** 24 + 2 ** 20
+    rt = ref.to(torch.float32).to(torch.int64).clamp(max=2 ** 31 - 1).to(torch.int32)
+    assert not torch.equal(rt, ref)
+    a = (A.t().contiguous() if ta else A).to(dev)
+    b = (B.t().contiguous() if tb else B).to(dev)
+    for f32 in (False, True):
+        am = ops.new_scalar_u32(dev)
+        c = ops.gemm(a, b, ta, tb, absmax=am, f32_epilogue=f32)
+        want = rt if f32 else ref
+        assert torch.equal(c.cpu(), want)
+        assert int(am.cpu()) == po.absmax(want)
 
 
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
