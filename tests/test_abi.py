@@ -131,8 +131,15 @@ def test_workspace_sizes(lib):
     # direct GEMM form needs nothing when k is a multiple of 16
     assert lib.niti_gemm_i8_workspace(0, 1, 128, 1024, 8192) == 0
     assert lib.niti_gemm_i8_workspace(0, 1, 128, 10, 100) > 0
-    assert lib.niti_gemm_i8_workspace(0, 0, 128, 1024, 8192) == 1024 * 8192
-    assert lib.niti_gemm_i8_workspace(1, 0, 128, 1024, 8192) == 128 * 8192 + 1024 * 8192
+    # operands with a slow reduction index are read as stored when n and k are multiples of 32 (the transposed
+    # first operand also needs m % 16 == 0, both transposed m % 32 == 0) ...
+    assert lib.niti_gemm_i8_workspace(0, 0, 128, 1024, 8192) == 0
+    assert lib.niti_gemm_i8_workspace(1, 0, 128, 1024, 8192) == 0
+    assert lib.niti_gemm_i8_workspace(1, 1, 1024, 10, 8192) == 0
+    # ... other shapes re-lay them: b [k,n] -> [n,k16]; a [k,m] -> [m,k16]
+    assert lib.niti_gemm_i8_workspace(0, 0, 128, 1000, 8192) == 1000 * 8192
+    assert lib.niti_gemm_i8_workspace(1, 1, 1000, 10, 8192) == 1000 * 8192
+    assert lib.niti_gemm_i8_workspace(1, 0, 120, 1024, 8192) == 120 * 8192 + 1024 * 8192
     # weight gradient: native 3x3 path = partial-sum slices, generic path = two transposed copies
     n = lib.niti_conv2d_i8_wgrad_workspace(128, 32, 32, 128, 128, 3, 3, 1)
     assert n >= 128 * 9 * 128 * 4 and n % 256 == 0
