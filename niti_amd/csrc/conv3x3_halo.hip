@@ -194,6 +194,16 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   const __amdgpu_buffer_rsrc_t rx = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.x), 0, a.x_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.wp), 0, a.wp_bytes, 0x00020000);
 
+  // NITI_RQ_SHIFT_HINT: *shift_out holds the caller's prediction (the previous training step's shift of this tensor).
+  // Read here, a whole main loop before it is needed; workgroup (0, 0) overwrites the word only after all slots are
+  // filled, i.e. after every workgroup has passed this line.
+  bool hinted = false;
+  int predicted = 0;
+  if constexpr (kFused) {
+    hinted = (a.rq_flags & NITI_RQ_SHIFT_HINT) != 0 && a.shift_out != nullptr && settle_shift < 0;
+    if (hinted) predicted = *a.shift_out;
+  }
+
   // ---- activation staging: an instruction fills 32 consecutive slots; lane -> (slot lane/2, half lane%2).
   // A lane's offset is split into a part fixed for the whole launch (vector register) and the slice's 32 * cs
   // (scalar offset of the load), so a stage spends no vector arithmetic on it.  A lane with nothing to fetch
@@ -595,17 +605,15 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const int nb = gridDim.x * gridDim.y;
     uint32_t* const slots = a.sync + kSyncSlot0;
     constexpr int kLook = 8;   // slots a lane reads with its loads in flight together
-    // NITI_RQ_SHIFT_HINT: *shift_out holds the caller's prediction (the previous training step's shift of this
-    // tensor).  Read before this workgroup fills its slot: workgroup (0, 0) overwrites the word only after all slots
-    // are filled.
     const bool nowait = (a.rq_flags & kRqNoWait) != 0;
     const bool settled = settle_shift >= 0;
-    const int predicted = ((a.rq_flags & NITI_RQ_SHIFT_HINT) != 0 && a.shift_out != nullptr && wave == 0 && !settled) ? *a.shift_out : 0;
-    uint32_t early[kLook];   // a hint: the first 64 * kLook slots as they are now
+    // Without a prediction, a hint: the first 64 * kLook slots as they are now.  With one the look would only put a
+    // trip to memory between the last product and the first store.
+    uint32_t early[kLook];
 #pragma unroll
     for (int u = 0; u < kLook; ++u) {
       const int i = u * 64 + lane;
-      early[u] = (wave == 0 && i < nb && !nowait && !settled) ? __hip_atomic_load(slot_word(slots, i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
+      early[u] = (wave == 0 && i < nb && !nowait && !settled && !hinted) ? __hip_atomic_load(slot_word(slots, i), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0u;
     }
     const uint32_t wmax = wave_max_u32(lmax);
     __syncthreads();  // the tiles are dead from here on
@@ -623,7 +631,6 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (lane == 0) {
         red[8] = g - 1u;
         red[9] = nb == 1 ? 1u : 0u;
-        red[10] = static_cast<uint32_t>(predicted);
       }
     }
     __syncthreads();
@@ -631,7 +638,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     // the slots seen so far already need more (or the range is final already)
     int shift = max(bitwidth_of(red[8], a.bw_mode) - a.target_bits, 0);
     bool final_range = red[9] != 0u;
-    if (!final_range) shift = max(shift, static_cast<int>(red[10]));
+    if (!final_range) shift = max(shift, predicted);
     if (settled) shift = settle_shift;
     if (nowait) {   // the shift this tile is stored with, for the settling launch
       if (tid == 0) slot_word(slots, blockIdx.y * gridDim.x + blockIdx.x)[1] = static_cast<uint32_t>(shift);
