@@ -723,6 +723,79 @@ def test_requant_special_cases(dev, kat):
     assert int(s_int.cpu()) == 23 - 7 and int(s_f32.cpu()) == 22 - 7 == po.bitwidth_f32(2 ** 22 + 2) - 7
 
 
+def _band_operands(g, N, Q, C, K):
+    """Activations and a filter whose largest convolution sum is exactly 2**22 + 2 (at one output pixel, channel 0):
+    260 products 127 * 127, one 127 * 6 and one 4 * 1 under the 3 x 3 x 32 window of pixel (0, 3, 3); everything else
+    is non-negative and smaller.  In (2**22, 2**22 (1 + 7e-7)] the reference's float evaluation of the bit width
+    (ti_torch.py:366-377) gives 22 where the exact integer form gives 23."""
+    x = torch.zeros((N, Q, Q, C), dtype=torch.int8)
+    w = torch.randint(0, 3, (K, 3, 3, C), generator=g, dtype=torch.int8)
+    xv = [127] * 260 + [127, 4] + [0] * (9 * 32 - 262)
+    wv = [127] * 260 + [6, 1] + [0] * (9 * 32 - 262)
+    x[0, 2:5, 2:5, :32] = torch.tensor(xv, dtype=torch.int8).view(3, 3, 32)
+    w[0, :, :, :] = 0
+    w[0, :, :, :32] = torch.tensor(wv, dtype=torch.int8).view(3, 3, 32)
+    x[1:] = torch.randint(0, 4, (N - 1, Q, Q, C), generator=g, dtype=torch.int8)
+    return x, w
+
+
+def test_fused_epilogues_in_both_bitwidth_modes(dev):
+    """The tensor-wide range lands in the thin band above 2**22 where the two bit-width rules differ: forward
+    convolution + act_calc, data gradient + err_calc and weight gradient + grad_calc + update, each as its one-launch
+    form, in the exact integer mode and in the reference's float mode."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    g = torch.Generator().manual_seed(977)
+    N, Q, C, K = 8, 8, 64, 64
+    T = 2 ** 22 + 2
+    assert po.bitwidth_int(T) == 23 and po.bitwidth_f32(T) == 22
+    x, w = _band_operands(g, N, Q, C, K)
+    acc = co.conv_fprop(x, w, 1, 1)
+    assert int(acc.abs().max()) == T
+    for mode, want in (("int", 16), ("f32", 15)):
+        _say("band fprop", mode)
+        ref, e = po.act_calc(acc, 0, "round", "floor", None, mode)
+        y, sh, _ = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), bw_mode=mode)
+        assert int(sh.cpu()) == want == e
+        assert torch.equal(y.cpu(), ref)
+    # data gradient: the error map plays the activations' part; flipping the filter's taps and swapping its channel
+    # roles turns the forward sums above into data-gradient sums (ti_torch.py:403-405)
+    wd = torch.flip(w, [1, 2]).permute(3, 1, 2, 0).contiguous()
+    accd = co.conv_dgrad(x, wd, Q, Q, 1, 1)
+    assert torch.equal(accd, acc)
+    for mode, want in (("int", 16), ("f32", 15)):
+        _say("band dgrad", mode)
+        ref, e = po.err_calc(accd, "round", "floor", None, mode)
+        dx, sh, _ = ops.conv2d_dgrad_requant(x.to(dev), wd.to(dev), bw_mode=mode)
+        assert int(sh.cpu()) == want == e
+        assert torch.equal(dx.cpu(), ref)
+    # weight gradient: 260 pixels with 127 in activation channel 0 and error channel 0, two isolated pixels carrying
+    # 127 * 6 and 4 * 1; the centre tap sums them all, every other tap loses at least one pair
+    Nw = 8
+    act = torch.zeros((Nw, Q, Q, C), dtype=torch.int8)
+    err = torch.zeros((Nw, Q, Q, K), dtype=torch.int8)
+    flat_a, flat_e = act.view(-1, C), err.view(-1, K)
+    flat_a[:260, 0] = 127
+    flat_e[:260, 0] = 127
+    flat_a[5 * 64 + 18, 0], flat_e[5 * 64 + 18, 0] = 127, 6
+    flat_a[6 * 64 + 45, 0], flat_e[6 * 64 + 45, 0] = 4, 1
+    act[7] = torch.randint(0, 3, (Q, Q, C), generator=g, dtype=torch.int8)
+    err[7] = torch.randint(0, 3, (Q, Q, K), generator=g, dtype=torch.int8)
+    act[7, :, :, 0] = 0     # nothing more for the element that carries the range
+    accw = co.conv_wgrad(act, err, 3, 3, 1, 1)
+    assert int(accw.abs().max()) == T == int(accw[0, 1, 1, 0])
+    w0 = torch.randint(-127, 128, (K, 3, 3, C), generator=g, dtype=torch.int8)
+    for mode, want in (("int", 18), ("f32", 17)):
+        _say("band wgrad", mode)
+        g8, e = po.grad_calc(accw, 5, "psto", "floor", None, mode)
+        wdev = w0.clone().to(dev)
+        got_g8, _, sh, _ = ops.conv2d_wgrad_update(act.to(dev), err.to(dev), wdev, mu=5, method="psto", bw_mode=mode, want_grad=True)
+        assert int(sh.cpu()) == want == e
+        assert torch.equal(got_g8.cpu(), g8)
+        assert torch.equal(wdev.cpu(), po.weight_update(w0, g8))
+
+
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 def test_grad_update_and_weight_update(dev, div_mode):
     from niti_amd import ops
