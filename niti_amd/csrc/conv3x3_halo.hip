@@ -3,8 +3,8 @@
 //
 // The plain implicit GEMM (conv_mfma.hip) fetches each activation nine times and each filter row
 // once per pixel tile through L2.  Here a workgroup owns 256 consecutive output pixels (whole rows of
-// an image, or whole small images) x KT output channels (128, or 64 when the launch would otherwise
-// leave compute units idle) and walks over the input channels in slices of 32 - one reduction step of
+// an image, or whole small images) x KT output channels (128; 64, or on small maps 32, when the launch would
+// otherwise leave compute units idle) and walks over the input channels in slices of 32 - one reduction step of
 // v_mfma_i32_32x32x32_i8.  Per slice it stages the activation rows with their one-pixel halo once
 // (10-20 KB, out-of-image positions read as zero through an out-of-range buffer offset) and serves all
 // nine taps from that tile; the filter streams one filter row (three taps) per stage from a
@@ -12,7 +12,7 @@
 // moves contiguous bytes.
 //
 // 8 wavefronts: 4 pixel groups of 64 x 2 channel groups of KT/2; a wavefront holds 2 x KT/64 tiles of
-// 32 x 32 sums.  Activation slices are double buffered and the filter stages run through a ring of
+// 32 x 32 sums (KT = 32: 8 pixel groups of 32, one tile each).  Activation slices are double buffered and the filter stages run through a ring of
 // three, so the only synchronisation is one s_barrier per filter row; all of it stays under 80 KB of
 // LDS and 128 VGPRs, so two workgroups share a compute unit and fill each other's stalls.  The same
 // kernel computes the data gradient when given the flipped / transposed filter arrangement (prepare
