@@ -280,6 +280,14 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst + 16 * 1024), 16, wsrc_c, rel, 0, 0);
   };
 
+  // The first loads leave before the fragment addresses below are worked out (about half a microsecond of integer
+  // arithmetic that the trip to memory can hide).  Per-wavefront load order, both pipelines: act(0), W(0), W(1).
+  issue_act(0, 0);
+  issue_w(0, 0, 0);
+  if constexpr (G::RPS == 1) issue_w(0, 1, 1);
+  else if (a.cslices > 1) issue_w(1, 0, 1);
+  __builtin_amdgcn_sched_barrier(0);
+
   // ---- fragment addressing
   constexpr int PT = G::PT;
   const int wp_ = KT == 32 ? wave : (wave & 3);   // group of 32 PT pixels
@@ -482,9 +490,6 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     // (issued three stages earlier, so older than W(t)).  Younger than W(t) are W(t+1) and the activation loads
     // issued in stage t-2 or t-1.
     const int nst = a.cslices * 3;
-    issue_act(0, 0);
-    issue_w(0, 0, 0);
-    issue_w(0, 1, 1);
     for (int ci = 0; ci < a.cslices; ++ci) {
       const int8_t* sa = act_buf + (ci & 1) * G::ACT_BYTES;
       const bool more = ci + 1 < a.cslices;
@@ -514,9 +519,6 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     // ---- pipeline, one slice per stage (a barrier every 18 MFMAs instead of every 6).  Per-wavefront load order:
     // act(0), W(0), W(1); inside stage ci after its barrier: act(ci+1), then W(ci+2).  Stage ci needs W(ci) and
     // act(ci); the only loads younger than both are those of W(ci+1).
-    issue_act(0, 0);
-    issue_w(0, 0, 0);
-    if (a.cslices > 1) issue_w(1, 0, 1);
     for (int ci = 0; ci < a.cslices; ++ci) {
       const int8_t* sa = act_buf + (ci & 1) * G::ACT_BYTES;
       if (ci + 1 < a.cslices)
