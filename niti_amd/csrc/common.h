@@ -84,6 +84,14 @@ __device__ inline int f32_roundtrip(int v) {
   return static_cast<int>(f);  // f is integral and >= -2^31 here
 }
 
+// Zero that the compiler cannot see through: added to a uniform address it keeps a load's result in a vector
+// register (a result known to be uniform is moved to a scalar register right behind the load, which waits for it).
+__device__ inline int opaque_zero() {
+  int z;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(z));
+  return z;
+}
+
 __device__ inline uint32_t uabs(int v) { return v < 0 ? 0u - static_cast<uint32_t>(v) : static_cast<uint32_t>(v); }
 
 // Largest value over the wavefront, in every lane.  A max-scan inside each row of 16 lanes (row_shr 1, 2, 4, 8: lanes

@@ -197,11 +197,16 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   // NITI_RQ_SHIFT_HINT: *shift_out holds the caller's prediction (the previous training step's shift of this tensor).
   // Read here, a whole main loop before it is needed; workgroup (0, 0) overwrites the word only after all slots are
   // filled, i.e. after every workgroup has passed this line.
+  // The load is unconditional (from the range word when there is no prediction), its address looks lane-dependent to
+  // the compiler and its result is not looked at before the epilogue: a load inside a branch, or one whose result the
+  // compiler knows to be the same in all lanes (and moves to a scalar register at once), would be waited for on the
+  // spot - a trip to memory in front of the first stage's loads.
   bool hinted = false;
-  int predicted = 0;
+  int predicted_raw = 0;
   if constexpr (kFused) {
     hinted = (a.rq_flags & NITI_RQ_SHIFT_HINT) != 0 && a.shift_out != nullptr && settle_shift < 0;
-    if (hinted) predicted = *a.shift_out;
+    const int32_t* const src = hinted ? a.shift_out : reinterpret_cast<const int32_t*>(a.sync);
+    predicted_raw = __hip_atomic_load(src + opaque_zero(), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
 
   // ---- activation staging: an instruction fills 32 consecutive slots; lane -> (slot lane/2, half lane%2).
@@ -640,7 +645,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     // the slots seen so far already need more (or the range is final already)
     int shift = max(bitwidth_of(red[8], a.bw_mode) - a.target_bits, 0);
     bool final_range = red[9] != 0u;
-    if (!final_range) shift = max(shift, predicted);
+    if (!final_range && hinted) shift = max(shift, predicted_raw);
     if (settled) shift = settle_shift;
     if (nowait) {   // the shift this tile is stored with, for the settling launch
       if (tid == 0) slot_word(slots, blockIdx.y * gridDim.x + blockIdx.x)[1] = static_cast<uint32_t>(shift);

@@ -554,8 +554,13 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
   __shared__ uint32_t gshare;
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  // read before this workgroup fills its slot: workgroup 0 overwrites the word only after all slots are filled
-  const int predicted = (a.predict != 0 && a.shift_out != nullptr) ? max(*a.shift_out, 0) : 0;
+  // Read before this workgroup fills its slot: workgroup 0 overwrites the word only after all slots are filled.
+  // An unconditional load (from the range word when there is no prediction) with an address that looks lane-dependent
+  // to the compiler, whose result is first looked at after the partial sums have been added: a load inside a branch, or
+  // one whose result is known to be uniform, would be waited for on the spot, in front of theirs.
+  const bool has_prediction = a.predict != 0 && a.shift_out != nullptr;
+  const int predicted_raw = __hip_atomic_load((has_prediction ? a.shift_out : reinterpret_cast<const int32_t*>(a.sync)) + opaque_zero(),
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   v4i fin[OWN];
   uint32_t lmax = 0;
   // Every wavefront has columns of its own at least in the first round (uniform over the grid): then each adds all
@@ -704,7 +709,7 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
   const bool speculate = a.predict != 0 && same_layout && gridDim.x > 1;
   int applied = -1;
   if (speculate) {
-    applied = max(max(bitwidth_of(bmax, a.bw_mode) - a.target_bits, 0), predicted);
+    applied = max(max(bitwidth_of(bmax, a.bw_mode) - a.target_bits, 0), has_prediction ? predicted_raw : 0);
     apply(applied, true);
   }
   if (wave == 0) {
