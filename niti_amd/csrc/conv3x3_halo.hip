@@ -669,6 +669,26 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
           for (int e = 0; e < 16; ++e) acc[i][j][e] = f32_roundtrip(acc[i][j][e]);
     }
+    // The mask bytes (ReLU backward of the layer below / the pooled map) do not depend on the rounding: the first two
+    // of the wavefront's pieces are requested here and each later one two pieces ahead of its use, so that they have
+    // arrived when the stores below need them - requested where it is used, every piece would be a trip to memory
+    // between two stores.
+    // (Only where registers allow: the wavefronts with four accumulator tiles are at the 128-register limit of two
+    // workgroups per CU and fetch each piece where it is used.)
+    constexpr int NPIECE = 32 * PT / PPI;
+    constexpr bool kMaskAhead = NWF * PT <= 2;
+    constexpr int MKD = !kMaskAhead ? 1 : (NPIECE < 2 ? NPIECE : 2);
+    v4i mkpre[MKD];
+    auto mask_request = [&](int t) {
+      const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
+      const int m = pixwave + t * PPI + prow;
+      const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
+      mkpre[t % MKD] = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
+    };
+    if (kMaskAhead && a.mask != nullptr) {
+#pragma unroll
+      for (int t = 0; t < MKD; ++t) mask_request(t);
+    }
 #pragma nounroll
     for (int pass = 0; pass < 2; ++pass) {
       // the sums look modified to the compiler in every pass: nothing derived from them (magnitudes, signs) is
@@ -708,9 +728,15 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         v4i v = *reinterpret_cast<const v4i*>(patch + pl * PROW + piece * 16);
         const int m = pixwave + pl;
         const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
+        v4i mk;
         if (a.mask != nullptr) {  // ReLU backward of the layer below, folded in: its output is this layer's input
-          const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
-          const auto mk = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
+          if constexpr (kMaskAhead) {
+            mk = mkpre[t % MKD];
+            if (t + MKD < NPIECE) mask_request(t + MKD);
+          } else {
+            const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
+            mk = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
+          }
 #pragma unroll
           for (int q = 0; q < 4; ++q) v[q] &= static_cast<int>(positive_bytes(static_cast<uint32_t>(mk[q])));
         }
@@ -718,8 +744,6 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
           // max-pool backward folded in (mk holds the pooled values): the window of pooled pixel m in the pooling's input
           const __amdgpu_buffer_rsrc_t rxp = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.pool_x), 0, a.unpool_bytes, 0x00020000);
           const __amdgpu_buffer_rsrc_t ru = __builtin_amdgcn_make_buffer_rsrc(a.unpool, 0, a.unpool_bytes, 0x00020000);
-          const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask), 0, a.y8_bytes, 0x00020000);
-          const auto mk = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
           const int n = m / (Q * Q), rem = m - n * (Q * Q);
           const int pp = rem / Q, pq = rem - pp * Q;
           const int rowb = 2 * Q * a.K;
@@ -786,6 +810,10 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (fshift == shift) break;
       shift = fshift;
       __builtin_amdgcn_s_waitcnt(0);   // the stores of the first pass leave before those that replace them
+      if (kMaskAhead && a.mask != nullptr) {
+#pragma unroll
+        for (int t = 0; t < MKD; ++t) mask_request(t);
+      }
     }
     if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0 && !nowait && !settled) {
       const int sh = shift > 0 ? shift : 0;
