@@ -685,9 +685,31 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       const int off = (m < total_pix && ch < a.K) ? m * a.K + ch : kOob;
       mkpre[t % MKD] = __builtin_amdgcn_raw_buffer_load_b128(rm, off, 0, 0);
     };
+    // the same for the pooling windows of the folded max-pool backward, one piece ahead
+    v4i xwpre[kMaskAhead ? 4 : 1];
+    auto window_offsets = [&](int t, int (&wo)[4]) {
+      const int m = pixwave + t * PPI + prow;
+      const bool in = m < total_pix && ch < a.K;
+      const int n = m / (Q * Q), rem = m - n * (Q * Q);
+      const int pp = rem / Q, pq = rem - pp * Q;
+      const int rowb = 2 * Q * a.K;
+      const int base = ((n * 2 * Q + 2 * pp) * 2 * Q + 2 * pq) * a.K + ch;
+#pragma unroll
+      for (int k = 0; k < 4; ++k) wo[k] = in ? base + (k >> 1) * rowb + (k & 1) * a.K : kOob;
+    };
+    auto window_request = [&](int t) {
+      if constexpr (kMaskAhead) {
+        const __amdgpu_buffer_rsrc_t rxp = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.pool_x), 0, a.unpool_bytes, 0x00020000);
+        int wo[4];
+        window_offsets(t, wo);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) xwpre[k] = __builtin_amdgcn_raw_buffer_load_b128(rxp, wo[k], 0, 0);
+      }
+    };
     if (kMaskAhead && a.mask != nullptr) {
 #pragma unroll
       for (int t = 0; t < MKD; ++t) mask_request(t);
+      if (a.unpool != nullptr) window_request(0);
     }
 #pragma nounroll
     for (int pass = 0; pass < 2; ++pass) {
@@ -744,16 +766,17 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
           // max-pool backward folded in (mk holds the pooled values): the window of pooled pixel m in the pooling's input
           const __amdgpu_buffer_rsrc_t rxp = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.pool_x), 0, a.unpool_bytes, 0x00020000);
           const __amdgpu_buffer_rsrc_t ru = __builtin_amdgcn_make_buffer_rsrc(a.unpool, 0, a.unpool_bytes, 0x00020000);
-          const int n = m / (Q * Q), rem = m - n * (Q * Q);
-          const int pp = rem / Q, pq = rem - pp * Q;
-          const int rowb = 2 * Q * a.K;
-          const int base = ((n * 2 * Q + 2 * pp) * 2 * Q + 2 * pq) * a.K + ch;
           int wo[4];
-#pragma unroll
-          for (int k = 0; k < 4; ++k) wo[k] = off == kOob ? kOob : base + (k >> 1) * rowb + (k & 1) * a.K;
+          window_offsets(t, wo);
           v4i xw[4], ow[4];
+          if constexpr (kMaskAhead) {
 #pragma unroll
-          for (int k = 0; k < 4; ++k) xw[k] = __builtin_amdgcn_raw_buffer_load_b128(rxp, wo[k], 0, 0);
+            for (int k = 0; k < 4; ++k) xw[k] = xwpre[k];
+            if (t + 1 < NPIECE) window_request(t + 1);
+          } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) xw[k] = __builtin_amdgcn_raw_buffer_load_b128(rxp, wo[k], 0, 0);
+          }
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
             uint32_t taken = 0;   // bytes whose gradient an earlier position of the window (scan order) already received
@@ -813,6 +836,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       if (kMaskAhead && a.mask != nullptr) {
 #pragma unroll
         for (int t = 0; t < MKD; ++t) mask_request(t);
+        if (a.unpool != nullptr) window_request(0);
       }
     }
     if (blockIdx.x == 0 && blockIdx.y == 0 && tid == 0 && !nowait && !settled) {
