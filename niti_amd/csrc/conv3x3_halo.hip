@@ -721,28 +721,37 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
         for (int j = 0; j < PT; ++j) asm volatile("" : "+v"(acc[i][j]));
       // round, pack four channels per dword, transpose through a per-wavefront patch, store 16-byte pieces; the
       // common rounding mode gets a short form
-      const bool fast = shift >= 1 && !trunc && !psto;
-      const int sm1 = shift - 1, lo = relu ? 0 : -127;
+      // The shift is the same in every lane but has come through LDS, which the compiler cannot know: made a scalar
+      // here, the choice between the two forms below is ONE scalar branch.  (Left inside the loops as a per-lane
+      // condition it cost every value both forms' set-up under execution masks and a taken branch.)
+      const int ushift = __builtin_amdgcn_readfirstlane(shift);
+      const bool fast = ushift >= 1 && !trunc && !psto;
+      const int sm1 = ushift - 1, lo = relu ? 0 : -127;
+      auto round_tiles = [&](auto fastc) {
+        constexpr bool kFast = decltype(fastc)::value;
 #pragma unroll
-      for (int j = 0; j < PT; ++j)
+        for (int j = 0; j < PT; ++j)
 #pragma unroll
-        for (int i = 0; i < NWF; ++i)
+          for (int i = 0; i < NWF; ++i)
 #pragma unroll
-          for (int g = 0; g < 4; ++g) {
-            int r[4];
+            for (int g = 0; g < 4; ++g) {
+              int r[4];
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-              const int x = acc[i][j][4 * g + e];
-              if (fast) {
-                r[e] = round_nearest_floor_fast(x, sm1, lo);
-              } else {
-                if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
-                else r[e] = wrap_to_i8(x);
-                if (relu && r[e] < 0) r[e] = 0;
+              for (int e = 0; e < 4; ++e) {
+                const int x = acc[i][j][4 * g + e];
+                if constexpr (kFast) {
+                  r[e] = round_nearest_floor_fast(x, sm1, lo);
+                } else {
+                  if (ushift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, ushift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, ushift, trunc);
+                  else r[e] = wrap_to_i8(x);
+                  if (relu && r[e] < 0) r[e] = 0;
+                }
               }
+              *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = pack4_i8(r[0], r[1], r[2], r[3]);
             }
-            *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = pack4_i8(r[0], r[1], r[2], r[3]);
-          }
+      };
+      if (fast) round_tiles(std::true_type{});
+      else round_tiles(std::false_type{});
       // same wavefront reads back what it wrote: LDS operations of one wavefront complete in order
 #pragma unroll
       for (int t = 0; t < 32 * PT / PPI; ++t) {
