@@ -655,7 +655,10 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
     const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
     wold[j] = (same_layout && v < kFinishV && col < a.nv) ? reinterpret_cast<const uint32_t*>(a.w)[col] : 0u;
   }
-  auto apply = [&](int shift, bool first) {
+  // shift: the same in every lane, but it has come through LDS or memory, which the compiler cannot know - as a scalar
+  // the choices below are scalar branches instead of both sides under execution masks
+  auto apply = [&](int shift_any, bool first) {
+    const int shift = __builtin_amdgcn_readfirstlane(shift_any);
 #pragma unroll
     for (int j = 0; j < OWN; ++j) {
       const int v = j * NW + wave;
