@@ -668,10 +668,15 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
       const v4i s = fin[j];
       if (first && a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
       int r[4];
+      if (shift < 1) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
-        else r[e] = wrap_to_i8(s[e]);
+        for (int e = 0; e < 4; ++e) r[e] = wrap_to_i8(s[e]);
+      } else if (psto) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
       }
       const uint32_t e0 = static_cast<uint32_t>(col) * 4u;
       const uint32_t rt = e0 / C;               // k * 9 + tap
