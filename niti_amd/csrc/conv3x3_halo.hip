@@ -62,6 +62,35 @@ __device__ inline void hc_sync() {
   asm volatile("" ::: "memory");
 }
 
+// The four dwords of a fragment, each lane taking its right-hand neighbour's (kLeft: wave_shl:1) or its left-hand
+// neighbour's (wave_shr:1) value - zero where there is none - and-ed with keep.  The shift rides on the AND as its DPP
+// modifier: one instruction per dword where a DPP move followed by the AND would be two.  The compiler does not see
+// inside the statement, so the wait states it would add are written out: two in front (a vector instruction that
+// wrote a source just before), two behind (an MFMA that reads the result right after).
+template <bool kLeft>
+__device__ inline v4i shifted_and4(v4i x, int keep) {
+  int r0, r1, r2, r3;
+  if constexpr (kLeft)
+    asm("s_nop 1\n\t"
+        "v_and_b32_dpp %0, %4, %8 wave_shl:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_and_b32_dpp %1, %5, %8 wave_shl:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_and_b32_dpp %2, %6, %8 wave_shl:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_and_b32_dpp %3, %7, %8 wave_shl:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "s_nop 1"
+        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(keep));
+  else
+    asm("s_nop 1\n\t"
+        "v_and_b32_dpp %0, %4, %8 wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_and_b32_dpp %1, %5, %8 wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_and_b32_dpp %2, %6, %8 wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "v_and_b32_dpp %3, %7, %8 wave_shr:1 row_mask:0xf bank_mask:0xf bound_ctrl:1\n\t"
+        "s_nop 1"
+        : "=&v"(r0), "=&v"(r1), "=&v"(r2), "=&v"(r3)
+        : "v"(x[0]), "v"(x[1]), "v"(x[2]), "v"(x[3]), "v"(keep));
+  return v4i{r0, r1, r2, r3};
+}
+
 struct HaloArgs {
   const int8_t* x;    // [N,Q,Q,C]
   const int8_t* wp;   // prepared filter: [ceil(K/64)][cslices][9][64][32], rows XOR-swizzled
@@ -392,8 +421,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     v4i ps[PT];
 #pragma unroll
     for (int j = 0; j < PT; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
+      ps[j] = shifted_and4<true>(pc[j], keep_r);
     tap_ready(std::integral_constant<int, 1>{});
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
@@ -401,8 +429,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
 #pragma unroll
     for (int j = 0; j < PT; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
+      ps[j] = shifted_and4<false>(pc[j], keep_l);
     tap_ready(std::integral_constant<int, 2>{});
 #pragma unroll
     for (int i = 0; i < NWF; ++i)
@@ -470,16 +497,14 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       v4i ps[PT];
 #pragma unroll
       for (int j = 0; j < PT; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x130, 0xf, 0xf, true) & keep_r;  // wave_shl:1
+        ps[j] = shifted_and4<true>(pc[j], keep_r);
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
         for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[1][i], ps[j], acc[i][j], 0, 0, 0);
 #pragma unroll
       for (int j = 0; j < PT; ++j)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) ps[j][q] = __builtin_amdgcn_update_dpp(0, pc[j][q], 0x138, 0xf, 0xf, true) & keep_l;  // wave_shr:1
+        ps[j] = shifted_and4<false>(pc[j], keep_l);
 #pragma unroll
       for (int i = 0; i < NWF; ++i)
 #pragma unroll
