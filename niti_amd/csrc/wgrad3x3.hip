@@ -76,7 +76,11 @@ __device__ inline WorkItem die_local_work_item() {
 // a_base: error-tile offsets of the lane's two 8-byte rows (reduction step 0); b_base: halo-tile offsets of its rows
 // (reduction step 0, filter row 0); ROWB: bytes of a halo row.  kShiftTaps: the second and third tap of a filter row
 // are byte shifts of the first one's pixel sequence (rows of at least 8 pixels), otherwise every tap is read.
-template <int Q, int BR, int HR, int ROWB, bool kShiftTaps, int NB>
+// kShiftErr (rows of 8 or 16 pixels, which lie whole inside a lane's 16 pixels): the ERROR fragment is shifted instead -
+// sum_q err[q] act[q+s-1] = sum_q' err[q'-s+1] act[q'] -, once per reduction step for all three filter rows (8 byte
+// shifts instead of 24 per nine MFMAs), and every filter row reads one aligned activation fragment (b_base then names
+// the pixels themselves, halo column + 1): 8 instead of 11 LDS reads.
+template <int Q, int BR, int HR, int ROWB, bool kShiftTaps, int NB, bool kShiftErr = false>
 __device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const int (&b_base)[NB], v16i (&acc)[9]) {
   v2i alo[2], ahi[2];   // [reduction step & 1]
   v2i rd[2][NB];        // [row step & 1]
@@ -104,7 +108,25 @@ __device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const
 #pragma unroll
     for (int q = 0; q < NB; ++q) asm volatile("" : "+v"(d[q]));
     const v4i a4 = af[ks & 1];
-    if constexpr (!kShiftTaps) {
+    if constexpr (kShiftErr) {
+      static_assert(NB == 2 && (Q == 8 || Q == 16));
+      const v4i bf = {d[0][0], d[0][1], d[1][0], d[1][1]};
+      // err[q'+1] (tap 0) and err[q'-1] (tap 2) of the lane's 16 pixels, zero where the row ends
+      const uint32_t l0 = static_cast<uint32_t>(a4[0]), l1 = static_cast<uint32_t>(a4[1]), h0 = static_cast<uint32_t>(a4[2]),
+                     h1 = static_cast<uint32_t>(a4[3]);
+      v4i aL, aR;
+      aL[0] = static_cast<int>(__builtin_amdgcn_alignbyte(l1, l0, 1));
+      aL[1] = static_cast<int>(Q == 16 ? __builtin_amdgcn_alignbyte(h0, l1, 1) : l1 >> 8);
+      aL[2] = static_cast<int>(__builtin_amdgcn_alignbyte(h1, h0, 1));
+      aL[3] = static_cast<int>(h1 >> 8);
+      aR[0] = static_cast<int>(l0 << 8);
+      aR[1] = static_cast<int>(__builtin_amdgcn_alignbyte(l1, l0, 3));
+      aR[2] = static_cast<int>(Q == 16 ? __builtin_amdgcn_alignbyte(h0, l1, 3) : h0 << 8);
+      aR[3] = static_cast<int>(__builtin_amdgcn_alignbyte(h1, h0, 3));
+      acc[r * 3 + 0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aL, bf, acc[r * 3 + 0], 0, 0, 0);
+      acc[r * 3 + 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, bf, acc[r * 3 + 1], 0, 0, 0);
+      acc[r * 3 + 2] = __builtin_amdgcn_mfma_i32_32x32x32_i8(aR, bf, acc[r * 3 + 2], 0, 0, 0);
+    } else if constexpr (!kShiftTaps) {
 #pragma unroll
       for (int s = 0; s < 3; ++s)
         acc[r * 3 + s] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a4, v4i{d[2 * s][0], d[2 * s][1], d[2 * s + 1][0], d[2 * s + 1][1]},
@@ -398,7 +420,8 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   // (3 or 4 reads per filter row).  Shorter rows (4 x 4 and 2 x 2 maps: eight pixels are two or four rows) read
   // every tap.
   constexpr bool kShiftTaps = Q >= 8;
-  constexpr int NB = kShiftTaps ? (Q >= 16 ? 3 : 4) : 6;
+  constexpr bool kShiftErr = Q == 8 || Q == 16;   // the error fragment is shifted instead, once for all three filter rows
+  constexpr int NB = kShiftErr ? 2 : (kShiftTaps ? (Q >= 16 ? 3 : 4) : 6);
   int b_base[NB];
 #pragma unroll
   for (int o = 0; o < 2; ++o) {
@@ -414,7 +437,10 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
       return G::ERR_BYTES + ((ph * G::HALF_ROWS + hrow) * G::RP + w) * 32 + cb;
     };
     const int p0 = 16 * lk + (j >> 1), p1 = p0 + 8;
-    if (!kShiftTaps) {
+    if constexpr (kShiftErr) {
+      b_base[0] = slot_addr(p0 / Q, p0 % Q + 1);
+      b_base[1] = slot_addr(p1 / Q, p1 % Q + 1);
+    } else if (!kShiftTaps) {
 #pragma unroll
       for (int t = 0; t < 3; ++t) {
         b_base[2 * t] = slot_addr(p0 / Q, p0 % Q + t);
@@ -447,7 +473,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
     else wg_wait_vmcnt<0>();
     wg_sync();
     if (it + G::STAGES - 1 < nb) issue(band_begin + it + G::STAGES - 1, (it + G::STAGES - 1) % G::STAGES);
-    wgrad_stage<Q, BR, G::HR, G::RP * 32, kShiftTaps, NB>(lds_addr(smem + (it % G::STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
+    wgrad_stage<Q, BR, G::HR, G::RP * 32, kShiftTaps, NB, kShiftErr>(lds_addr(smem + (it % G::STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
   }
 
   // ---- add the two pixel halves: half 1 -> LDS -> half 0 -> memory.  Slot layout [value][lane].
