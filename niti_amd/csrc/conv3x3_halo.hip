@@ -760,19 +760,21 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
           for (int i = 0; i < NWF; ++i)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-              int r[4];
+              uint32_t packed;
+              if constexpr (kFast) {
+                packed = round4_nearest_floor_fast(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], sm1, lo);
+              } else {
+                int r[4];
 #pragma unroll
-              for (int e = 0; e < 4; ++e) {
-                const int x = acc[i][j][4 * g + e];
-                if constexpr (kFast) {
-                  r[e] = round_nearest_floor_fast(x, sm1, lo);
-                } else {
+                for (int e = 0; e < 4; ++e) {
+                  const int x = acc[i][j][4 * g + e];
                   if (ushift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, ushift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, ushift, trunc);
                   else r[e] = wrap_to_i8(x);
                   if (relu && r[e] < 0) r[e] = 0;
                 }
+                packed = pack4_i8(r[0], r[1], r[2], r[3]);
               }
-              *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = pack4_i8(r[0], r[1], r[2], r[3]);
+              *reinterpret_cast<uint32_t*>(patch + (j * 32 + lr) * PROW + (i * 8 + 2 * g + lk) * 4) = packed;
             }
       };
       if (fast) round_tiles(std::true_type{});

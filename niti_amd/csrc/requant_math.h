@@ -88,6 +88,23 @@ __device__ inline int round_nearest_floor_fast(int x, int sm1, int lo) {
   return min(max(r, lo), 127);
 }
 
+// The same for four values at once, as the dword of their four int8 results: after the first shift the values fit
+// 16 bits (|x| < 2^(s + 7) gives |x >> (s-1)| <= 256; the conversion saturates beyond), so the increment, the second
+// shift and the clip run on packed 16-bit pairs - 15 instructions for four values instead of 23.  Exact whenever
+// |x >> (s-1)| < 32767, i.e. for every shift that is not far below the tensor's own.
+typedef short v2s __attribute__((ext_vector_type(2)));
+__device__ inline uint32_t round4_nearest_floor_fast(int x0, int x1, int x2, int x3, int sm1, int lo) {
+  v2s a = __builtin_amdgcn_cvt_pk_i16(x0 >> sm1, x1 >> sm1);
+  v2s b = __builtin_amdgcn_cvt_pk_i16(x2 >> sm1, x3 >> sm1);
+  const v2s one = {1, 1}, lo2 = {static_cast<short>(lo), static_cast<short>(lo)}, hi2 = {127, 127};
+  a = (a + one) >> 1;
+  b = (b + one) >> 1;
+  a = __builtin_elementwise_min(__builtin_elementwise_max(a, lo2), hi2);
+  b = __builtin_elementwise_min(__builtin_elementwise_max(b, lo2), hi2);
+  // bytes 0 and 2 of each pair
+  return __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, b), __builtin_bit_cast(uint32_t, a), 0x06040200u);
+}
+
 // 0xFF in every byte of m that is positive as an int8, 0x00 elsewhere (the ReLU-backward test on four activations)
 __host__ __device__ inline uint32_t positive_bytes(uint32_t m) {
   const uint32_t nz = (((m & 0x7F7F7F7Fu) + 0x7F7F7F7Fu) | m) & 0x80808080u;  // bit 7 where the byte is non-zero
