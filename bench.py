@@ -18,6 +18,7 @@ Usage: python bench.py [--gpus 1] [--steps K] [--warmup W]
 from __future__ import annotations
 
 import argparse
+import gc
 import json
 import os
 import sys
@@ -180,9 +181,16 @@ class Runner:
             graphs = []
             for u in ([1, unroll] if unroll > 1 else [1]):
                 g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    for _ in range(u):
-                        step_fn()
+                # no cyclic garbage collection while capturing (freeing tensors of the eager warm-up, allocated on
+                # another stream, makes the allocator record events, which a capturing process may not do)
+                gc.collect()
+                gc.disable()
+                try:
+                    with torch.cuda.graph(g):
+                        for _ in range(u):
+                            step_fn()
+                finally:
+                    gc.enable()
                 g.replay()
                 torch.cuda.synchronize()
                 graphs.append(g)

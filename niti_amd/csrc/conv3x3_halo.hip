@@ -1065,7 +1065,8 @@ __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int
     }
     __syncthreads();
     const uint32_t gmax = words[4];
-    const int shift = max(bitwidth_of(gmax, a.bw_mode) - a.target_bits, 0);
+    // a scalar, so that the choice of rounding form below is a scalar branch (see the kernel above)
+    const int shift = __builtin_amdgcn_readfirstlane(max(bitwidth_of(gmax, a.bw_mode) - a.target_bits, 0));
     if (rh == 0) {
       const bool trunc = a.trunc != 0;
       const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
@@ -1076,19 +1077,20 @@ __global__ __launch_bounds__(512) void conv3x3_map2_kernel(const HaloArgs a, int
       const __amdgpu_buffer_rsrc_t rm = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.mask != nullptr ? a.mask : a.y8), 0, a.y8_bytes, 0x00020000);
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        int r[4];
+        uint32_t v;
+        if (fast) {
+          v = round4_nearest_floor_fast(acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3], sm1, lo);
+        } else {
+          int r[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int x = acc[4 * g + e];
-          if (fast) {
-            r[e] = round_nearest_floor_fast(x, sm1, lo);
-          } else {
+          for (int e = 0; e < 4; ++e) {
+            const int x = acc[4 * g + e];
             if (shift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, shift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, shift, trunc);
             else r[e] = wrap_to_i8(x);
             if (relu && r[e] < 0) r[e] = 0;
           }
+          v = pack4_i8(r[0], r[1], r[2], r[3]);
         }
-        uint32_t v = pack4_i8(r[0], r[1], r[2], r[3]);
         const int c = ch + 8 * g;
         const int off = (n < a.N && c < a.K) ? static_cast<int>(row + c) : kOob;
         uint32_t mk = 0;

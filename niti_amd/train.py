@@ -11,6 +11,7 @@ without it, on a synthetic ten-class set of noisy class patterns (``synthetic_lo
 from __future__ import annotations
 
 import argparse
+import gc
 import logging
 import os
 import shutil
@@ -97,10 +98,21 @@ class StepGraph:
             cur.wait_stream(self.side)
         else:
             torch.cuda.synchronize()
+            # No cyclic garbage collection while the stream is capturing: a collection that frees device tensors of
+            # the eager steps (allocated on another stream) makes the allocator record events, which a capturing
+            # process may not do - the runtime aborts.  torch.cuda.graph collects once on entry, but a collection can
+            # still start at any allocation inside the captured step.
+            gc_was_on = gc.isenabled()
+            gc.collect()
+            gc.disable()
             try:
                 g = torch.cuda.CUDAGraph()
-                with torch.cuda.graph(g):
-                    self._step()
+                try:
+                    with torch.cuda.graph(g):
+                        self._step()
+                finally:
+                    if gc_was_on:
+                        gc.enable()
                 self.graph = g
                 self.out = (self.model.out, self.model.out_exp)     # where every replay leaves its logits
                 g.replay()
