@@ -91,7 +91,8 @@ __device__ inline int round_nearest_floor_fast(int x, int sm1, int lo) {
 // The same for four values at once, as the dword of their four int8 results: after the first shift the values fit
 // 16 bits (|x| < 2^(s + 7) gives |x >> (s-1)| <= 256; the conversion saturates beyond), so the increment, the second
 // shift and the clip run on packed 16-bit pairs - 15 instructions for four values instead of 23.  Exact whenever
-// |x >> (s-1)| < 32767, i.e. for every shift that is not far below the tensor's own.
+// |x >> (s-1)| < 32767; the callers' shift is never smaller than what their own largest magnitude needs (a predicted
+// shift only ever raises it), so |x >> (s-1)| <= 256 for every value they pass.
 typedef short v2s __attribute__((ext_vector_type(2)));
 __device__ inline uint32_t round4_nearest_floor_fast(int x0, int x1, int x2, int x3, int sm1, int lo) {
   v2s a = __builtin_amdgcn_cvt_pk_i16(x0 >> sm1, x1 >> sm1);
