@@ -513,6 +513,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     });
   };
 
+  __builtin_amdgcn_s_setprio(3);   // the main loop's instructions go ahead of a co-resident workgroup's epilogue
   if constexpr (G::RPS == 1) {
     // ---- pipeline, one filter row per stage.  Stage t = 3 * slice + filter row.  Per-wavefront load order: act(0),
     // W(0), W(1); inside stage t after its barrier: W(t+2), then - in the first stage of a slice - act(next slice).
@@ -564,6 +565,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   }
 
   // ---- epilogue: acc[i][j][4g+e] = channel kt*KT + wc*(KT/2) + i*32 + 8g + 4*lk + e of pixel pixbase+wp_*64+j*32+lr
+  __builtin_amdgcn_s_setprio(0);
   const bool roundtrip = (a.flags & NITI_EPI_F32_ROUNDTRIP) != 0;
   int vmax = 0, vmin = 0;
 #pragma unroll
