@@ -233,8 +233,11 @@ int niti_conv2d_i8_wgrad(const int8_t* act, const int8_t* err, int32_t* dw, int 
  *   (ti_torch.py:135-147) -> UpdateWeight.weight_update (ti_torch.py:11-21)
  * with the same result as niti_conv2d_i8_wgrad followed by niti_grad_update_i8, bit for bit; the int32 gradient
  * is only written when dw_out is given.  The partial sums of the weight-gradient kernel are added up, the
- * tensor-wide range is exchanged between the workgroups of the finishing kernel, and
+ * tensor-wide range is exchanged between the workgroups that add them, and
  *   g = round(dw >> max(bitwidth(max|dw|) - mu, 0)),  w = clip(w - g, +-127).
+ * Maps of side 8, 16 and 32 with N*H*W % 256 == 0 run all of it as one launch (its at most 256 workgroups add
+ * their partial sums once all of them have arrived, so they must all be resident: nothing else may run on the
+ * device beside it); other shapes, or a device that cannot hold the grid at once, run a main and a finishing launch.
  *
  * Covered: the shapes of the native 3x3 weight-gradient kernel (3x3, stride 1, pad 1, square maps of side 2, 4, 8,
  * 16 or 32, C % 16 == 0, K % 16 == 0, N*H*W % 128 == 0, even N for side 8, N*H*W % 256 == 0 for sides 2 and 4) with

@@ -314,6 +314,250 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
   }
 }
 
+// Partial sums -> rounded gradient -> updated weights in one launch (the int32 gradient is not stored unless
+// asked for).  A workgroup owns kFinishV x 64 int4 columns at a grid-wide stride; its NW wavefronts each add every
+// NW-th slice of every column (no barrier in between, so all those loads are in flight together), column v is
+// then completed through LDS by wavefront v % NW, which keeps the sums in registers.  The workgroup publishes its
+// largest magnitude in its slot and waits for the slots of all workgroups (all resident: the host sizes the grid
+// for that; the wait is bounded by a wall-clock limit), derives the shift from the maximum over the slots, and
+// every wavefront applies w = clip(w - round(sum >> shift)) to its columns.  NW = 16 serves the launches with
+// many slices and few columns, NW = 4 the others.
+constexpr int kFinishV = 16;
+constexpr int kFusedV = 48;         // columns per lane in the one-launch form (8 wavefronts: six each)
+constexpr int kArriveSlots = 256;   // workgroups of the one-launch form at most
+constexpr int kFinishSlot0 = 16;
+struct FinishArgs {
+  const int32_t* partial;
+  long long slice_stride;
+  int splits;
+  long long nv;        // int4 columns of the gradient: K*9*C / 4
+  int C, Cw;           // channels per gradient row / per weight row (Cw <= C; the rest is channel padding)
+  int8_t* w;           // [K][9][Cw], updated in place
+  int8_t* g8;          // optional rounded gradient, laid out like w
+  int32_t* dw;         // optional int32 gradient [K][9][C]
+  int8_t* wprep;       // optional: the halo convolution kernel's forward copy of the [K][9][C] filter, kept in step with w
+  uint32_t* sync;      // word 0: max |sum| (output); word 1: wait gave up; words kFinishSlot0..: slots, zero on entry
+  int roundtrip, target_bits, method, trunc, bw_mode;
+  int predict;         // *shift_out holds a predicted shift on entry
+  long long spin_limit;
+  uint32_t* sticky;    // device-wide word set when the wait gives up, may be null
+  int32_t* shift_out;
+  const int32_t* exp_a;
+  const int32_t* exp_b;
+  int32_t* exp_out;
+  uint32_t* arrive;    // one-launch form only: a slot per workgroup, zero on entry, filled when its partial sums are in memory
+};
+
+template <int NW>
+struct FinishShared {
+  v4i part[2][NW][64];
+  uint32_t wmax[NW];
+  uint32_t gshare;
+};
+
+// The finishing pass of workgroup `block` out of `nblocks` (V = int4 columns per lane it may own, NW its wavefronts).
+// predicted_raw: the word read from a.shift_out (or anything when there is no prediction) at kernel start.
+// kCoherent: the partial sums were written by this same launch (by other dies' workgroups, with write-through stores): they
+// are read with loads that do not hit a line another die may have changed (byte offsets then fit 31 bits: host check).
+template <int NW, int V, bool kCoherent = false>
+__device__ __forceinline__ void finish_columns(const FinishArgs& a, const int block, const int nblocks, FinishShared<NW>& sh,
+                                               const int predicted_raw) {
+  const __amdgpu_buffer_rsrc_t rpart =
+      __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(a.partial), 0, kCoherent ? static_cast<int>(a.slice_stride * a.splits * 4) : 0, 0x00020000);
+  auto slice_col = [&](int z, long long col) -> v4i {
+    if constexpr (kCoherent) {
+      constexpr int kSc1 = 16;   // cache policy bit: coherent across the dies' L2 caches
+      return __builtin_amdgcn_raw_buffer_load_b128(rpart, static_cast<int>((z * a.slice_stride + col * 4) * 4), 0, kSc1);
+    } else {
+      return reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
+    }
+  };
+  constexpr int OWN = V / NW > 0 ? V / NW : 1;   // columns a wavefront completes
+  constexpr int VS = V < NW ? V : NW;            // columns a workgroup has when the slices are shared (fewer rounds than wavefronts)
+  auto& part = sh.part;
+  auto& wmax = sh.wmax;
+  uint32_t& gshare = sh.gshare;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const bool has_prediction = a.predict != 0 && a.shift_out != nullptr;
+  v4i fin[OWN];
+  uint32_t lmax = 0;
+  // Every wavefront has columns of its own at least in the first round (uniform over the grid): then each adds all
+  // slices of its own columns and nothing goes through LDS.  With fewer columns than wavefronts the slices are
+  // shared instead (phases 1 and 2 below), so that no wavefront idles while another walks over all slices.
+  const bool direct = a.nv >= static_cast<long long>(NW) * nblocks * 64;
+  if (direct) {
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int v = j * NW + wave;
+      const long long col = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
+      v4i s = {0, 0, 0, 0};
+      if (v < V && col < a.nv) {
+        int z = 0;
+        for (; z + 3 < a.splits; z += 4) {
+          const v4i v0 = slice_col(z + 0, col);
+          const v4i v1 = slice_col(z + 1, col);
+          const v4i v2 = slice_col(z + 2, col);
+          const v4i v3 = slice_col(z + 3, col);
+          s += (v0 + v1) + (v2 + v3);
+        }
+        for (; z < a.splits; ++z) s += slice_col(z, col);
+      }
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
+        const uint32_t u = uabs(s[e]);
+        lmax = u > lmax ? u : lmax;
+      }
+      fin[j] = s;
+    }
+  } else {
+  v4i sum[VS];
+  // phase 1: every wavefront adds its share of the slices for all of the workgroup's columns
+#pragma unroll
+  for (int v = 0; v < VS; ++v) {
+    const long long col = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
+    v4i s = {0, 0, 0, 0};
+    if (col < a.nv) {
+      int z = wave;
+      for (; z + 3 * NW < a.splits; z += 4 * NW) {
+        const v4i v0 = slice_col(z + 0 * NW, col);
+        const v4i v1 = slice_col(z + 1 * NW, col);
+        const v4i v2 = slice_col(z + 2 * NW, col);
+        const v4i v3 = slice_col(z + 3 * NW, col);
+        s += (v0 + v1) + (v2 + v3);
+      }
+      for (; z < a.splits; z += NW) s += slice_col(z, col);
+    }
+    sum[v] = s;
+  }
+  // phase 2: column v is completed by wavefront v % NW (two LDS buffers in turn: one barrier per column)
+#pragma unroll
+  for (int v = 0; v < VS; ++v) {
+    if (static_cast<long long>(v) * nblocks * 64 >= a.nv) continue;  // uniform over the grid: nothing at this stride
+    part[v & 1][wave][lane] = sum[v];
+    __syncthreads();
+    if (wave == v % NW) {
+      v4i s = part[v & 1][0][lane];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) s += part[v & 1][w][lane];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
+        const uint32_t u = uabs(s[e]);
+        lmax = u > lmax ? u : lmax;
+      }
+      fin[v / NW] = s;
+    }
+  }
+  }
+  lmax = wave_max_u32(lmax);
+  if (lane == 0) wmax[wave] = lmax;
+  __syncthreads();
+  uint32_t bmax = 0;   // the workgroup's largest magnitude, in every wavefront
+#pragma unroll
+  for (int w = 0; w < NW; ++w) bmax = max(bmax, wmax[w]);
+  if (wave == 0 && lane == 0)
+    __hip_atomic_store(slot_word(a.sync + kFinishSlot0, block), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+
+  // phase 3: every wavefront rounds its columns and updates their weights (element counts fit 31 bits: host check).
+  // With a predicted shift (a.predict) the update is applied before the range is final, so that its stores overlap
+  // the wait for the other workgroups, and applied once more from the same old weights if the final shift differs.
+  const bool trunc = a.trunc != 0;
+  const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
+  const bool same_layout = a.Cw == a.C;
+  const uint32_t C = static_cast<uint32_t>(a.C), Cw = static_cast<uint32_t>(a.Cw);
+  uint32_t wold[OWN];
+#pragma unroll
+  for (int j = 0; j < OWN; ++j) {
+    const int v = j * NW + wave;
+    const long long col = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
+    wold[j] = (same_layout && v < V && col < a.nv) ? reinterpret_cast<const uint32_t*>(a.w)[col] : 0u;
+  }
+  // shift: the same in every lane, but it has come through LDS or memory, which the compiler cannot know - as a scalar
+  // the choices below are scalar branches instead of both sides under execution masks
+  auto apply = [&](int shift_any, bool first) {
+    const int shift = __builtin_amdgcn_readfirstlane(shift_any);
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      const int v = j * NW + wave;
+      if (v >= V) continue;
+      const long long col = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
+      if (col >= a.nv) continue;
+      const v4i s = fin[j];
+      if (first && a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
+      int r[4];
+      if (shift < 1) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = wrap_to_i8(s[e]);
+      } else if (psto) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc);
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
+      }
+      const uint32_t e0 = static_cast<uint32_t>(col) * 4u;
+      const uint32_t rt = e0 / C;               // k * 9 + tap
+      const uint32_t c0 = e0 - rt * C;
+      uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
+      if (same_layout) {
+        uint32_t gp = 0;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int wo = static_cast<int>(static_cast<int8_t>((wold[j] >> (8 * e)) & 0xFFu));
+          wnew |= (static_cast<uint32_t>(clip127(wo - r[e])) & 0xFFu) << (8 * e);
+          gp |= (static_cast<uint32_t>(r[e]) & 0xFFu) << (8 * e);
+        }
+        reinterpret_cast<uint32_t*>(a.w)[col] = wnew;
+        if (a.g8 != nullptr) reinterpret_cast<uint32_t*>(a.g8)[col] = gp;
+      } else {   // applied once only (the old weights are read here)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if (c0 + e < Cw) {
+            const uint32_t wi = rt * Cw + c0 + e;
+            const int wn = clip127(static_cast<int>(a.w[wi]) - r[e]);
+            a.w[wi] = static_cast<int8_t>(wn);
+            wnew |= (static_cast<uint32_t>(wn) & 0xFFu) << (8 * e);
+            if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
+          }
+        }
+      }
+      if (a.wprep != nullptr) {
+        // [64-channel group][32-channel slice][tap][64 rows][32 bytes], 16-byte halves swapped where (row >> 3) is odd
+        const uint32_t k = rt / 9u, tap = rt - k * 9u;
+        const uint32_t row = k & 63u, cs = c0 >> 5;
+        const uint32_t half = ((c0 >> 4) & 1u) ^ ((row >> 3) & 1u);
+        const uint32_t dst = (((((k >> 6) * ((C + 31u) >> 5) + cs) * 9u + tap) * 64u + row) << 5) + half * 16u + (c0 & 15u);
+        *reinterpret_cast<uint32_t*>(a.wprep + dst) = wnew;
+      }
+    }
+  };
+  const bool speculate = a.predict != 0 && same_layout && nblocks > 1;
+  int applied = -1;
+  if (speculate) {
+    applied = max(max(bitwidth_of(bmax, a.bw_mode) - a.target_bits, 0), has_prediction ? predicted_raw : 0);
+    apply(applied, true);
+  }
+  if (wave == 0) {
+    const uint32_t g = wait_slots(a.sync + kFinishSlot0, nblocks, a.spin_limit, &a.sync[1], a.sticky);
+    if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
+  }
+  __syncthreads();
+  const uint32_t gmax = gshare;
+  const int shift = max(bitwidth_of(gmax, a.bw_mode) - a.target_bits, 0);
+  if (block == 0 && threadIdx.x == 0) {
+    a.sync[0] = gmax;
+    if (a.shift_out != nullptr) *a.shift_out = shift;
+    if (a.exp_out != nullptr)
+      *a.exp_out = shift + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
+  }
+  if (shift != applied) {
+    if (applied >= 0) __builtin_amdgcn_s_waitcnt(0);   // the first update's stores leave before those that replace them
+    apply(shift, applied < 0);
+  }
+}
+
 // ---- the same computation with half the partial-sum traffic ------------------------------------------------
 // The kernel above leaves 128 x 64 x 9 partial sums (295 KB) per workgroup in memory; with about one workgroup
 // per compute unit that is almost 60 MB per launch, written and read again, whatever the layer - more time than
@@ -342,11 +586,18 @@ struct NGeom {
   static_assert(LDS_BYTES <= 160 * 1024, "stages must fit in LDS");
 };
 
-template <int Q, int BR, int NI>
-__global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs a) {
+template <int Q, int BR, int NI, bool kFinish>
+__global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs a, const FinishArgs f) {
   using G = NGeom<Q, BR, NI>;
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
   int8_t* const dump = smem + G::LDS_BYTES - 1024;
+  int predicted_raw = 0;
+  if constexpr (kFinish) {
+    // read at kernel start, looked at in the finishing part (see wgrad_finish_kernel)
+    const bool has_prediction = f.predict != 0 && f.shift_out != nullptr;
+    predicted_raw = __hip_atomic_load((has_prediction ? f.shift_out : reinterpret_cast<const int32_t*>(f.sync)) + opaque_zero(),
+                                      __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -498,9 +749,27 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
 #pragma unroll
         for (int t = 0; t < 9; ++t) {
           const int v = acc[t][4 * g + e] + park[(t * 16 + 4 * g + e) * 64];
-          if (c < a.Cp && k < a.K) out[(static_cast<long long>(k) * 9 + t) * a.Cp + c] = v;
+          if (c < a.Cp && k < a.K) {
+            int32_t* const dst = out + (static_cast<long long>(k) * 9 + t) * a.Cp + c;
+            if constexpr (kFinish) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // written through to memory
+            else *dst = v;
+          }
         }
       }
+  }
+  if constexpr (kFinish) {
+    // ---- the finishing pass in the same launch: all workgroups are resident (the host checks), every one takes a
+    // share of the gradient's columns once the partial sums of all of them are in memory.  The sums travel between
+    // the dies by write-through stores, completed before the arrival slot is filled, and by loads that bypass stale
+    // lines (fences would do the same by writing back and invalidating whole L2 caches, once per wavefront: 50 us).
+    const int nblocks = static_cast<int>(gridDim.x * gridDim.y * gridDim.z);
+    const int block = static_cast<int>(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's stores have been performed
+    __syncthreads();
+    if (tid == 0) __hip_atomic_store(slot_word(f.arrive, block), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (wave == 0) wait_slots(f.arrive, nblocks, f.spin_limit, &f.sync[1], f.sticky);
+    __syncthreads();
+    finish_columns<8, kFusedV, true>(f, block, nblocks, *reinterpret_cast<FinishShared<8>*>(smem), predicted_raw);
   }
 }
 
@@ -541,45 +810,9 @@ __global__ __launch_bounds__(256) void wgrad_reduce_kernel(const int32_t* __rest
   if (absmax != nullptr && wave == 0) fold_absmax(absmax, lmax);
 }
 
-// Partial sums -> rounded gradient -> updated weights in one launch (the int32 gradient is not stored unless
-// asked for).  A workgroup owns kFinishV x 64 int4 columns at a grid-wide stride; its NW wavefronts each add every
-// NW-th slice of every column (no barrier in between, so all those loads are in flight together), column v is
-// then completed through LDS by wavefront v % NW, which keeps the sums in registers.  The workgroup publishes its
-// largest magnitude in its slot and waits for the slots of all workgroups (all resident: the host sizes the grid
-// for that; the wait is bounded by a wall-clock limit), derives the shift from the maximum over the slots, and
-// every wavefront applies w = clip(w - round(sum >> shift)) to its columns.  NW = 16 serves the launches with
-// many slices and few columns, NW = 4 the others.
-constexpr int kFinishV = 16;
-constexpr int kFinishSlot0 = 16;
-struct FinishArgs {
-  const int32_t* partial;
-  long long slice_stride;
-  int splits;
-  long long nv;        // int4 columns of the gradient: K*9*C / 4
-  int C, Cw;           // channels per gradient row / per weight row (Cw <= C; the rest is channel padding)
-  int8_t* w;           // [K][9][Cw], updated in place
-  int8_t* g8;          // optional rounded gradient, laid out like w
-  int32_t* dw;         // optional int32 gradient [K][9][C]
-  int8_t* wprep;       // optional: the halo convolution kernel's forward copy of the [K][9][C] filter, kept in step with w
-  uint32_t* sync;      // word 0: max |sum| (output); word 1: wait gave up; words kFinishSlot0..: slots, zero on entry
-  int roundtrip, target_bits, method, trunc, bw_mode;
-  int predict;         // *shift_out holds a predicted shift on entry
-  long long spin_limit;
-  uint32_t* sticky;    // device-wide word set when the wait gives up, may be null
-  int32_t* shift_out;
-  const int32_t* exp_a;
-  const int32_t* exp_b;
-  int32_t* exp_out;
-};
-
 template <int NW>
 __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishArgs a) {
-  constexpr int OWN = kFinishV / NW > 0 ? kFinishV / NW : 1;   // columns a wavefront completes
-  __shared__ v4i part[2][NW][64];
-  __shared__ uint32_t wmax[NW];
-  __shared__ uint32_t gshare;
-  const int lane = threadIdx.x & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  __shared__ FinishShared<NW> sh;
   // Read before this workgroup fills its slot: workgroup 0 overwrites the word only after all slots are filled.
   // An unconditional load (from the range word when there is no prediction) with an address that looks lane-dependent
   // to the compiler, whose result is first looked at after the partial sums have been added: a load inside a branch, or
@@ -587,182 +820,7 @@ __global__ __launch_bounds__(NW * 64, 4) void wgrad_finish_kernel(const FinishAr
   const bool has_prediction = a.predict != 0 && a.shift_out != nullptr;
   const int predicted_raw = __hip_atomic_load((has_prediction ? a.shift_out : reinterpret_cast<const int32_t*>(a.sync)) + opaque_zero(),
                                               __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  v4i fin[OWN];
-  uint32_t lmax = 0;
-  // Every wavefront has columns of its own at least in the first round (uniform over the grid): then each adds all
-  // slices of its own columns and nothing goes through LDS.  With fewer columns than wavefronts the slices are
-  // shared instead (phases 1 and 2 below), so that no wavefront idles while another walks over all slices.
-  const bool direct = a.nv >= static_cast<long long>(NW) * gridDim.x * 64;
-  if (direct) {
-#pragma unroll
-    for (int j = 0; j < OWN; ++j) {
-      const int v = j * NW + wave;
-      const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
-      v4i s = {0, 0, 0, 0};
-      if (v < kFinishV && col < a.nv) {
-        int z = 0;
-        for (; z + 3 < a.splits; z += 4) {
-          const v4i v0 = reinterpret_cast<const v4i*>(a.partial + (z + 0) * a.slice_stride)[col];
-          const v4i v1 = reinterpret_cast<const v4i*>(a.partial + (z + 1) * a.slice_stride)[col];
-          const v4i v2 = reinterpret_cast<const v4i*>(a.partial + (z + 2) * a.slice_stride)[col];
-          const v4i v3 = reinterpret_cast<const v4i*>(a.partial + (z + 3) * a.slice_stride)[col];
-          s += (v0 + v1) + (v2 + v3);
-        }
-        for (; z < a.splits; ++z) s += reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
-      }
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
-        const uint32_t u = uabs(s[e]);
-        lmax = u > lmax ? u : lmax;
-      }
-      fin[j] = s;
-    }
-  } else {
-  v4i sum[kFinishV];
-  // phase 1: every wavefront adds its share of the slices for all of the workgroup's columns
-#pragma unroll
-  for (int v = 0; v < kFinishV; ++v) {
-    const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
-    v4i s = {0, 0, 0, 0};
-    if (col < a.nv) {
-      int z = wave;
-      for (; z + 3 * NW < a.splits; z += 4 * NW) {
-        const v4i v0 = reinterpret_cast<const v4i*>(a.partial + (z + 0 * NW) * a.slice_stride)[col];
-        const v4i v1 = reinterpret_cast<const v4i*>(a.partial + (z + 1 * NW) * a.slice_stride)[col];
-        const v4i v2 = reinterpret_cast<const v4i*>(a.partial + (z + 2 * NW) * a.slice_stride)[col];
-        const v4i v3 = reinterpret_cast<const v4i*>(a.partial + (z + 3 * NW) * a.slice_stride)[col];
-        s += (v0 + v1) + (v2 + v3);
-      }
-      for (; z < a.splits; z += NW) s += reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
-    }
-    sum[v] = s;
-  }
-  // phase 2: column v is completed by wavefront v % NW (two LDS buffers in turn: one barrier per column)
-#pragma unroll
-  for (int v = 0; v < kFinishV; ++v) {
-    if (static_cast<long long>(v) * gridDim.x * 64 >= a.nv) continue;  // uniform over the grid: nothing at this stride
-    part[v & 1][wave][lane] = sum[v];
-    __syncthreads();
-    if (wave == v % NW) {
-      v4i s = part[v & 1][0][lane];
-#pragma unroll
-      for (int w = 1; w < NW; ++w) s += part[v & 1][w][lane];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
-        const uint32_t u = uabs(s[e]);
-        lmax = u > lmax ? u : lmax;
-      }
-      fin[v / NW] = s;
-    }
-  }
-  }
-  lmax = wave_max_u32(lmax);
-  if (lane == 0) wmax[wave] = lmax;
-  __syncthreads();
-  uint32_t bmax = 0;   // the workgroup's largest magnitude, in every wavefront
-#pragma unroll
-  for (int w = 0; w < NW; ++w) bmax = max(bmax, wmax[w]);
-  if (wave == 0 && lane == 0)
-    __hip_atomic_store(slot_word(a.sync + kFinishSlot0, blockIdx.x), bmax + 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-
-  // phase 3: every wavefront rounds its columns and updates their weights (element counts fit 31 bits: host check).
-  // With a predicted shift (a.predict) the update is applied before the range is final, so that its stores overlap
-  // the wait for the other workgroups, and applied once more from the same old weights if the final shift differs.
-  const bool trunc = a.trunc != 0;
-  const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
-  const bool same_layout = a.Cw == a.C;
-  const uint32_t C = static_cast<uint32_t>(a.C), Cw = static_cast<uint32_t>(a.Cw);
-  uint32_t wold[OWN];
-#pragma unroll
-  for (int j = 0; j < OWN; ++j) {
-    const int v = j * NW + wave;
-    const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
-    wold[j] = (same_layout && v < kFinishV && col < a.nv) ? reinterpret_cast<const uint32_t*>(a.w)[col] : 0u;
-  }
-  // shift: the same in every lane, but it has come through LDS or memory, which the compiler cannot know - as a scalar
-  // the choices below are scalar branches instead of both sides under execution masks
-  auto apply = [&](int shift_any, bool first) {
-    const int shift = __builtin_amdgcn_readfirstlane(shift_any);
-#pragma unroll
-    for (int j = 0; j < OWN; ++j) {
-      const int v = j * NW + wave;
-      if (v >= kFinishV) continue;
-      const long long col = (static_cast<long long>(v) * gridDim.x + blockIdx.x) * 64 + lane;
-      if (col >= a.nv) continue;
-      const v4i s = fin[j];
-      if (first && a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
-      int r[4];
-      if (shift < 1) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) r[e] = wrap_to_i8(s[e]);
-      } else if (psto) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) r[e] = round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[e], shift, trunc);
-      } else {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) r[e] = round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
-      }
-      const uint32_t e0 = static_cast<uint32_t>(col) * 4u;
-      const uint32_t rt = e0 / C;               // k * 9 + tap
-      const uint32_t c0 = e0 - rt * C;
-      uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
-      if (same_layout) {
-        uint32_t gp = 0;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int wo = static_cast<int>(static_cast<int8_t>((wold[j] >> (8 * e)) & 0xFFu));
-          wnew |= (static_cast<uint32_t>(clip127(wo - r[e])) & 0xFFu) << (8 * e);
-          gp |= (static_cast<uint32_t>(r[e]) & 0xFFu) << (8 * e);
-        }
-        reinterpret_cast<uint32_t*>(a.w)[col] = wnew;
-        if (a.g8 != nullptr) reinterpret_cast<uint32_t*>(a.g8)[col] = gp;
-      } else {   // applied once only (the old weights are read here)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if (c0 + e < Cw) {
-            const uint32_t wi = rt * Cw + c0 + e;
-            const int wn = clip127(static_cast<int>(a.w[wi]) - r[e]);
-            a.w[wi] = static_cast<int8_t>(wn);
-            wnew |= (static_cast<uint32_t>(wn) & 0xFFu) << (8 * e);
-            if (a.g8 != nullptr) a.g8[wi] = static_cast<int8_t>(r[e]);
-          }
-        }
-      }
-      if (a.wprep != nullptr) {
-        // [64-channel group][32-channel slice][tap][64 rows][32 bytes], 16-byte halves swapped where (row >> 3) is odd
-        const uint32_t k = rt / 9u, tap = rt - k * 9u;
-        const uint32_t row = k & 63u, cs = c0 >> 5;
-        const uint32_t half = ((c0 >> 4) & 1u) ^ ((row >> 3) & 1u);
-        const uint32_t dst = (((((k >> 6) * ((C + 31u) >> 5) + cs) * 9u + tap) * 64u + row) << 5) + half * 16u + (c0 & 15u);
-        *reinterpret_cast<uint32_t*>(a.wprep + dst) = wnew;
-      }
-    }
-  };
-  const bool speculate = a.predict != 0 && same_layout && gridDim.x > 1;
-  int applied = -1;
-  if (speculate) {
-    applied = max(max(bitwidth_of(bmax, a.bw_mode) - a.target_bits, 0), has_prediction ? predicted_raw : 0);
-    apply(applied, true);
-  }
-  if (wave == 0) {
-    const uint32_t g = wait_slots(a.sync + kFinishSlot0, gridDim.x, a.spin_limit, &a.sync[1], a.sticky);
-    if (lane == 0) gshare = g != 0u ? g - 1u : 0u;
-  }
-  __syncthreads();
-  const uint32_t gmax = gshare;
-  const int shift = max(bitwidth_of(gmax, a.bw_mode) - a.target_bits, 0);
-  if (blockIdx.x == 0 && threadIdx.x == 0) {
-    a.sync[0] = gmax;
-    if (a.shift_out != nullptr) *a.shift_out = shift;
-    if (a.exp_out != nullptr)
-      *a.exp_out = shift + (a.exp_a != nullptr ? *a.exp_a : 0) + (a.exp_b != nullptr ? *a.exp_b : 0);
-  }
-  if (shift != applied) {
-    if (applied >= 0) __builtin_amdgcn_s_waitcnt(0);   // the first update's stores leave before those that replace them
-    apply(shift, applied < 0);
-  }
+  finish_columns<NW, kFinishV>(a, static_cast<int>(blockIdx.x), static_cast<int>(gridDim.x), sh, predicted_raw);
 }
 
 // Slices are spaced so that the same element of consecutive slices falls into different memory
@@ -801,21 +859,47 @@ int pick_splits(int N, int Q, int C, int K) {
   return (bands + per - 1) / per;
 }
 
-template <int Q, int BR, int NI>
-int launch_narrow_geom(const WgradArgs& a, int splits, hipStream_t stream) {
+// f != nullptr: the one-launch form (main loop + finishing pass); returns NITI_ERR_UNSUPPORTED without launching when its
+// grid would not be resident at once, and the caller then runs the pair of launches.
+template <int Q, int BR, int NI, bool kFinish>
+int launch_narrow_geom_as(const WgradArgs& a, int splits, hipStream_t stream, const FinishArgs& f) {
   using G = NGeom<Q, BR, NI>;
   constexpr size_t lds = G::LDS_BYTES;
-  auto k = wgrad3x3_narrow_kernel<Q, BR, NI>;
+  auto k = wgrad3x3_narrow_kernel<Q, BR, NI, kFinish>;
   static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
+  static int resident_of[kDeviceSlots] = {};    // workgroups of this kernel the device holds at once
   bool& attr_set = attr_set_of[device_slot()];
   if (!attr_set) {
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(k), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess)
       return fail(NITI_ERR_LAUNCH, "wgrad: cannot reserve %zu bytes of LDS", lds);
+    if (kFinish) {
+      int dev = 0, cus = 0, per = 0;
+      if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess ||
+          hipOccupancyMaxActiveBlocksPerMultiprocessor(&per, reinterpret_cast<const void*>(k), 512, lds) != hipSuccess)
+        return fail(NITI_ERR_LAUNCH, "wgrad: cannot query occupancy");
+      resident_of[device_slot()] = cus * per;
+    }
     attr_set = true;
   }
   dim3 grid((a.K + 127) / 128, (a.C + 31) / 32, splits);
-  hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, a);
+  if (kFinish) {
+    const long long nblocks = static_cast<long long>(grid.x) * grid.y * grid.z;
+    if (nblocks > resident_of[device_slot()] || nblocks > kArriveSlots || f.nv > nblocks * kFusedV * 64 ||
+        f.slice_stride * f.splits * 4 >= 0x7fffffffLL)
+      return NITI_ERR_UNSUPPORTED;
+  }
+  hipLaunchKernelGGL(k, grid, dim3(512), lds, stream, a, f);
   return check_launch("wgrad3x3_narrow");
+}
+
+template <int Q, int BR, int NI>
+int launch_narrow_geom(const WgradArgs& a, int splits, hipStream_t stream, const FinishArgs* f) {
+  if constexpr (Q >= 8) {
+    if (f != nullptr) return launch_narrow_geom_as<Q, BR, NI, true>(a, splits, stream, *f);
+  } else {
+    if (f != nullptr) return NITI_ERR_UNSUPPORTED;
+  }
+  return launch_narrow_geom_as<Q, BR, NI, false>(a, splits, stream, FinishArgs{});
 }
 
 template <int Q, int BR, int NI>
@@ -856,7 +940,7 @@ size_t wgrad3x3_workspace(int N, int H, int C, int K) {
 }
 
 static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N, int H, int C, int K, int Cp, void* workspace,
-                                    WgradArgs& a, int& splits, hipStream_t stream) {
+                                    WgradArgs& a, int& splits, hipStream_t stream, FinishArgs* finish = nullptr) {
   a.act = act;
   a.err = err;
   a.partial = static_cast<int32_t*>(workspace);
@@ -871,12 +955,18 @@ static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N,
   a.bands_per_split = (a.bands + splits - 1) / splits;
   a.act_bytes = static_cast<long long>(N) * H * H * C;
   a.err_bytes = static_cast<long long>(N) * H * H * K;
+  if (finish != nullptr) {
+    if (!narrow) return NITI_ERR_UNSUPPORTED;
+    finish->partial = a.partial;
+    finish->slice_stride = a.slice_stride;
+    finish->splits = splits;
+  }
   if (narrow) {
-    if (H == 32) return launch_narrow_geom<32, 8, 1>(a, splits, stream);
-    if (H == 16) return launch_narrow_geom<16, 16, 1>(a, splits, stream);
-    if (H == 8) return launch_narrow_geom<8, 8, 4>(a, splits, stream);
-    if (H == 4) return launch_narrow_geom<4, 4, 16>(a, splits, stream);
-    return launch_narrow_geom<2, 2, 64>(a, splits, stream);
+    if (H == 32) return launch_narrow_geom<32, 8, 1>(a, splits, stream, finish);
+    if (H == 16) return launch_narrow_geom<16, 16, 1>(a, splits, stream, finish);
+    if (H == 8) return launch_narrow_geom<8, 8, 4>(a, splits, stream, finish);
+    if (H == 4) return launch_narrow_geom<4, 4, 16>(a, splits, stream, finish);
+    return launch_narrow_geom<2, 2, 64>(a, splits, stream, finish);
   }
   if (H == 32) return launch_geom<32, 4, 1>(a, splits, stream);
   if (H == 16) return launch_geom<16, 8, 1>(a, splits, stream);
@@ -906,7 +996,10 @@ int wgrad3x3_finish_blocks(int C, int K) {
   return static_cast<int>(nb < 1 ? 1 : nb);
 }
 
-size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0) + slot_words(blocks); }
+// header, range slots (of the finishing launch or of the one-launch form, whichever has more workgroups), arrival slots
+static size_t range_slot_words(int blocks) { return slot_words(blocks > kArriveSlots ? blocks : kArriveSlots); }
+size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0) + range_slot_words(blocks) + slot_words(kArriveSlots); }
+static size_t wgrad3x3_arrive_offset(int C, int K) { return static_cast<size_t>(kFinishSlot0) + range_slot_words(wgrad3x3_finish_blocks(C, K)); }
 
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
                            bool roundtrip, uint32_t* sync, const RequantSpec& rq, int8_t* g8, int32_t* dw, int8_t* wprep,
@@ -947,12 +1040,7 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   if (nb > resident[0]) return fail(NITI_ERR_UNSUPPORTED, "wgrad_update: %d workgroups do not fit on the device at once (%d)", nb, resident[0]);
   WgradArgs a;
   int splits = 1;
-  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, Cp, workspace, a, splits, stream);
-  if (st != NITI_OK) return st;
   FinishArgs f{};
-  f.partial = a.partial;
-  f.slice_stride = a.slice_stride;
-  f.splits = splits;
   f.nv = static_cast<long long>(K) * 9 * Cp / 4;
   f.C = Cp;
   f.Cw = w_channels;
@@ -973,6 +1061,20 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   f.exp_a = rq.exp_a;
   f.exp_b = rq.exp_b;
   f.exp_out = rq.exp_out;
+  f.arrive = sync + wgrad3x3_arrive_offset(C, K);
+  {
+    // main loop and finishing pass as one launch where its grid is resident at once (NITI_WGRAD_ONE_LAUNCH=0 pins the pair)
+    const char* e = getenv("NITI_WGRAD_ONE_LAUNCH");
+    if (e == nullptr || e[0] != '0') {
+      const int st1 = launch_wgrad3x3_partials(act, err, N, H, C, K, Cp, workspace, a, splits, stream, &f);
+      if (st1 != NITI_ERR_UNSUPPORTED) return st1;
+    }
+  }
+  const int st = launch_wgrad3x3_partials(act, err, N, H, C, K, Cp, workspace, a, splits, stream);
+  if (st != NITI_OK) return st;
+  f.partial = a.partial;
+  f.slice_stride = a.slice_stride;
+  f.splits = splits;
   // many slices and few columns per workgroup: sixteen wavefronts share the slices
   if (splits >= 32 && nb <= resident[1]) hipLaunchKernelGGL(wgrad_finish_kernel<16>, dim3(nb), dim3(1024), 0, stream, f);
   else hipLaunchKernelGGL(wgrad_finish_kernel<4>, dim3(nb), dim3(256), 0, stream, f);

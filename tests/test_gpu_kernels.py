@@ -458,14 +458,20 @@ def test_conv_wgrad_arrangements(dev, case, wgrad_arrangement):
                                   (3, 32, 3, 64), (2, 32, 3, 32), (2, 32, 3, 256), (5, 32, 2, 64), (1, 32, 1, 128),
                                   (8, 4, 64, 128), (3, 2, 32, 32), (37, 4, 96, 160), (300, 2, 64, 32)])   # any batch size on 4 x 4 / 2 x 2 maps
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
-def test_conv_wgrad_update(dev, case, div_mode):
-    """wgrad + grad_calc + weight update in one call against the oracle's three steps."""
+@pytest.mark.parametrize("launches", ["one", "pair"])
+def test_conv_wgrad_update(dev, case, div_mode, launches, monkeypatch):
+    """wgrad + grad_calc + weight update in one call against the oracle's three steps.  `pair` pins the main + finishing
+    launches for the shapes that otherwise run both parts as one launch."""
     import torch.nn.functional as F
     from niti_amd import ops
     from oracle import c_oracle as co
     from oracle import niti_oracle as po
     N, Q, C, K = case
-    _say("conv_wgrad_update", case, div_mode)
+    if launches == "pair":
+        if Q < 8 or C < 16 or (N * Q * Q) % 256 != 0:
+            pytest.skip("this shape has no one-launch form of the general kernel to pin away from")
+        monkeypatch.setenv("NITI_WGRAD_ONE_LAUNCH", "0")
+    _say("conv_wgrad_update", case, div_mode, launches)
     g = torch.Generator().manual_seed(970 + C + K)
     act, err, w = ri8(g, N, Q, Q, C), ri8(g, N, Q, Q, K, lo=-40, hi=40), ri8(g, K, 3, 3, C)
     dw_ref = co.conv_wgrad(act, err, 3, 3, 1, 1)
