@@ -20,6 +20,8 @@
 // kernel adds the slices (integer addition: any split gives the same result).
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "lds_asm.h"
 #include "requant_math.h"
@@ -325,6 +327,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
 constexpr int kFinishV = 16;
 constexpr int kFusedV = 48;         // columns per lane in the one-launch form (8 wavefronts: six each)
 constexpr int kArriveSlots = 256;   // workgroups of the one-launch form at most
+constexpr uint32_t kPartialBias = 1u << 23;   // added to the partial sums of the one-launch form before they are cut to 24 bits
 constexpr int kFinishSlot0 = 16;
 struct FinishArgs {
   const int32_t* partial;
@@ -346,7 +349,15 @@ struct FinishArgs {
   const int32_t* exp_b;
   int32_t* exp_out;
   uint32_t* arrive;    // one-launch form only: a slot per workgroup, zero on entry, filled when its partial sums are in memory
+  // one-launch form only.  A slice then holds, per group of four consecutive output channels kg, tap t and input channel
+  // c (unit u = (kg * 9 + t) * C + c), three planes: bits 0..15 of the four sums (8 bytes at 8u), bits 16..23 (4 bytes at
+  // units * 8 + 4u) and bits 24..31 (4 bytes at units * 12 + 4u).  The third plane is written only by a workgroup whose
+  // sums do not fit 24 bits; it says so in wide[tile + tiles * slice] (zero on entry) and in the value of its arrival slot.
+  uint32_t* wide;
+  int tiles_k, tiles_c;
 };
+
+typedef unsigned int v2u __attribute__((ext_vector_type(2)));
 
 template <int NW>
 struct FinishShared {
@@ -357,17 +368,38 @@ struct FinishShared {
 
 // The finishing pass of workgroup `block` out of `nblocks` (V = int4 columns per lane it may own, NW its wavefronts).
 // predicted_raw: the word read from a.shift_out (or anything when there is no prediction) at kernel start.
+// any_wide (uniform): some workgroup wrote the third plane (top bytes) of its part of its slice.
 // kCoherent: the partial sums were written by this same launch (by other dies' workgroups, with write-through stores): they
 // are read with loads that do not hit a line another die may have changed (byte offsets then fit 31 bits: host check).
 template <int NW, int V, bool kCoherent = false>
 __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int block, const int nblocks, FinishShared<NW>& sh,
-                                               const int predicted_raw) {
+                                               const int predicted_raw, const bool any_wide = false) {
   const __amdgpu_buffer_rsrc_t rpart =
       __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(a.partial), 0, kCoherent ? static_cast<int>(a.slice_stride * a.splits * 4) : 0, 0x00020000);
-  auto slice_col = [&](int z, long long col) -> v4i {
+  constexpr int kSc1 = 16;   // cache policy bit: coherent across the dies' L2 caches
+  const int units = static_cast<int>(a.nv);   // kCoherent: a column is a unit (four output channels), not four input channels
+  // kMixed = false: no workgroup wrote a third plane, every sum is the sign-extended 24-bit value
+  auto slice_col = [&](auto mixed, int z, long long col) -> v4i {
     if constexpr (kCoherent) {
-      constexpr int kSc1 = 16;   // cache policy bit: coherent across the dies' L2 caches
-      return __builtin_amdgcn_raw_buffer_load_b128(rpart, static_cast<int>((z * a.slice_stride + col * 4) * 4), 0, kSc1);
+      const int zoff = __builtin_amdgcn_readfirstlane(static_cast<int>(z * a.slice_stride * 4));   // z is the same in all lanes
+      const v2u lo = __builtin_amdgcn_raw_buffer_load_b64(rpart, static_cast<int>(col) * 8, zoff, kSc1);
+      const uint32_t mid = __builtin_amdgcn_raw_buffer_load_b32(rpart, units * 8 + static_cast<int>(col) * 4, zoff, kSc1);
+      v4i r;   // biased sums, 24 bits each
+      r[0] = static_cast<int>(__builtin_amdgcn_perm(mid, lo[0], 0x0C040100u));   // 0, mid.b0, lo.b1, lo.b0
+      r[1] = static_cast<int>(__builtin_amdgcn_perm(mid, lo[0], 0x0C050302u));
+      r[2] = static_cast<int>(__builtin_amdgcn_perm(mid, lo[1], 0x0C060100u));
+      r[3] = static_cast<int>(__builtin_amdgcn_perm(mid, lo[1], 0x0C070302u));
+      if constexpr (decltype(mixed)::value) {   // rare: the writer of this column's tile in slice z tells whether it wrote top bytes
+        const uint32_t rt = static_cast<uint32_t>(col) / static_cast<uint32_t>(a.C);   // kg * 9 + t
+        const uint32_t tile = (rt / 9u >> 5) + static_cast<uint32_t>(a.tiles_k) * ((static_cast<uint32_t>(col) - rt * static_cast<uint32_t>(a.C)) >> 5);
+        const bool wide = __hip_atomic_load(a.wide + tile + static_cast<uint32_t>(a.tiles_k * a.tiles_c) * static_cast<uint32_t>(z), __ATOMIC_RELAXED,
+                                            __HIP_MEMORY_SCOPE_AGENT) != 0u;
+        uint32_t hi = 0;
+        if (wide) hi = __builtin_amdgcn_raw_buffer_load_b32(rpart, units * 12 + static_cast<int>(col) * 4, zoff, kSc1);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) r[e] = static_cast<int>(static_cast<uint32_t>(r[e]) | ((hi >> (8 * e)) << 24));
+      }
+      return r;
     } else {
       return reinterpret_cast<const v4i*>(a.partial + z * a.slice_stride)[col];
     }
@@ -380,12 +412,40 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const bool has_prediction = a.predict != 0 && a.shift_out != nullptr;
+  const bool trunc = a.trunc != 0;
+  const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
+  const bool same_layout = a.Cw == a.C;
+  const uint32_t C = static_cast<uint32_t>(a.C), Cw = static_cast<uint32_t>(a.Cw);
+  // division by the channel count: a shift for the usual powers of two (a 32-bit division is some forty instructions,
+  // and this part of the launch runs few wavefronts)
+  const int c_log2 = (C & (C - 1u)) == 0u ? 31 - __builtin_clz(C) : -1;
+  auto div_c = [&](uint32_t x) -> uint32_t { return c_log2 >= 0 ? x >> c_log2 : x / C; };
+  auto out_col = [&](long long col) -> long long {
+    if constexpr (kCoherent) {
+      const uint32_t rt = div_c(static_cast<uint32_t>(col)), c = static_cast<uint32_t>(col) - rt * C, kg = rt / 9u, tap = rt - kg * 9u;
+      return static_cast<long long>(((kg * 4u + (c & 3u)) * 9u + tap) * (C >> 2) + (c >> 2));
+    } else {
+      return col;
+    }
+  };
+  // the old weights are requested first: they depend on nothing and are wanted right after the sums
+  uint32_t wold[OWN];
+#pragma unroll
+  for (int j = 0; j < OWN; ++j) {
+    const int v = j * NW + wave;
+    const long long col = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
+    wold[j] = (same_layout && v < V && col < a.nv) ? reinterpret_cast<const uint32_t*>(a.w)[out_col(col)] : 0u;
+  }
   v4i fin[OWN];
   uint32_t lmax = 0;
   // Every wavefront has columns of its own at least in the first round (uniform over the grid): then each adds all
   // slices of its own columns and nothing goes through LDS.  With fewer columns than wavefronts the slices are
   // shared instead (phases 1 and 2 below), so that no wavefront idles while another walks over all slices.
   const bool direct = a.nv >= static_cast<long long>(NW) * nblocks * 64;
+  // the whole gathering phase exists twice, so that the usual case (no third plane anywhere) has no branch between
+  // its loads and keeps them all in flight
+  const int bias_total = kCoherent ? static_cast<int>(static_cast<uint32_t>(a.splits) * kPartialBias) : 0;   // modulo 2^32, as the sums
+  auto gather = [&](auto mixed) {
   if (direct) {
 #pragma unroll
     for (int j = 0; j < OWN; ++j) {
@@ -395,13 +455,14 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
       if (v < V && col < a.nv) {
         int z = 0;
         for (; z + 3 < a.splits; z += 4) {
-          const v4i v0 = slice_col(z + 0, col);
-          const v4i v1 = slice_col(z + 1, col);
-          const v4i v2 = slice_col(z + 2, col);
-          const v4i v3 = slice_col(z + 3, col);
+          const v4i v0 = slice_col(mixed, z + 0, col);
+          const v4i v1 = slice_col(mixed, z + 1, col);
+          const v4i v2 = slice_col(mixed, z + 2, col);
+          const v4i v3 = slice_col(mixed, z + 3, col);
           s += (v0 + v1) + (v2 + v3);
         }
-        for (; z < a.splits; ++z) s += slice_col(z, col);
+        for (; z < a.splits; ++z) s += slice_col(mixed, z, col);
+        s -= bias_total;
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
@@ -421,13 +482,13 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
     if (col < a.nv) {
       int z = wave;
       for (; z + 3 * NW < a.splits; z += 4 * NW) {
-        const v4i v0 = slice_col(z + 0 * NW, col);
-        const v4i v1 = slice_col(z + 1 * NW, col);
-        const v4i v2 = slice_col(z + 2 * NW, col);
-        const v4i v3 = slice_col(z + 3 * NW, col);
+        const v4i v0 = slice_col(mixed, z + 0 * NW, col);
+        const v4i v1 = slice_col(mixed, z + 1 * NW, col);
+        const v4i v2 = slice_col(mixed, z + 2 * NW, col);
+        const v4i v3 = slice_col(mixed, z + 3 * NW, col);
         s += (v0 + v1) + (v2 + v3);
       }
-      for (; z < a.splits; z += NW) s += slice_col(z, col);
+      for (; z < a.splits; z += NW) s += slice_col(mixed, z, col);
     }
     sum[v] = s;
   }
@@ -441,6 +502,7 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
       v4i s = part[v & 1][0][lane];
 #pragma unroll
       for (int w = 1; w < NW; ++w) s += part[v & 1][w][lane];
+      if ((static_cast<long long>(v) * nblocks + block) * 64 + lane < a.nv) s -= bias_total;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         if (a.roundtrip) s[e] = f32_roundtrip(s[e]);
@@ -450,6 +512,28 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
       fin[v / NW] = s;
     }
   }
+  }
+  };
+  if (kCoherent && any_wide) gather(std::true_type{});
+  else gather(std::false_type{});
+  // kCoherent: a lane holds four output channels of one input channel, its quad four consecutive input channels: a
+  // 4 x 4 transposition inside the quad (two rounds of swaps) gives every lane four input channels of one output
+  // channel, the form of the weights in memory, and out_col the column that is (quads lie inside one row: C % 4 == 0)
+  if constexpr (kCoherent) {
+    const bool odd1 = (lane & 1) != 0, odd2 = (lane & 2) != 0;
+#pragma unroll
+    for (int j = 0; j < OWN; ++j) {
+      v4i s = fin[j], x;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = __builtin_amdgcn_mov_dpp(s[e ^ 1], 0xB1, 0xf, 0xf, true);   // quad_perm:[1,0,3,2]
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] = (((e & 1) != 0) == odd1) ? s[e] : x[e];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) x[e] = __builtin_amdgcn_mov_dpp(s[e ^ 2], 0x4E, 0xf, 0xf, true);   // quad_perm:[2,3,0,1]
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] = (((e & 2) != 0) == odd2) ? s[e] : x[e];
+      fin[j] = s;
+    }
   }
   lmax = wave_max_u32(lmax);
   if (lane == 0) wmax[wave] = lmax;
@@ -463,17 +547,6 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
   // phase 3: every wavefront rounds its columns and updates their weights (element counts fit 31 bits: host check).
   // With a predicted shift (a.predict) the update is applied before the range is final, so that its stores overlap
   // the wait for the other workgroups, and applied once more from the same old weights if the final shift differs.
-  const bool trunc = a.trunc != 0;
-  const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
-  const bool same_layout = a.Cw == a.C;
-  const uint32_t C = static_cast<uint32_t>(a.C), Cw = static_cast<uint32_t>(a.Cw);
-  uint32_t wold[OWN];
-#pragma unroll
-  for (int j = 0; j < OWN; ++j) {
-    const int v = j * NW + wave;
-    const long long col = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
-    wold[j] = (same_layout && v < V && col < a.nv) ? reinterpret_cast<const uint32_t*>(a.w)[col] : 0u;
-  }
   // shift: the same in every lane, but it has come through LDS or memory, which the compiler cannot know - as a scalar
   // the choices below are scalar branches instead of both sides under execution masks
   auto apply = [&](int shift_any, bool first) {
@@ -482,8 +555,9 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
     for (int j = 0; j < OWN; ++j) {
       const int v = j * NW + wave;
       if (v >= V) continue;
-      const long long col = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
-      if (col >= a.nv) continue;
+      const long long gcol = (static_cast<long long>(v) * nblocks + block) * 64 + lane;
+      if (gcol >= a.nv) continue;
+      const long long col = out_col(gcol);
       const v4i s = fin[j];
       if (first && a.dw != nullptr) reinterpret_cast<v4i*>(a.dw)[col] = s;
       int r[4];
@@ -498,7 +572,7 @@ __device__ __forceinline__ void finish_columns(const FinishArgs& a, const int bl
         for (int e = 0; e < 4; ++e) r[e] = round_one32<NITI_ROUND_NEAREST>(s[e], shift, trunc);
       }
       const uint32_t e0 = static_cast<uint32_t>(col) * 4u;
-      const uint32_t rt = e0 / C;               // k * 9 + tap
+      const uint32_t rt = div_c(e0);            // k * 9 + tap
       const uint32_t c0 = e0 - rt * C;
       uint32_t wnew = 0;   // the four updated weights (zero where the gradient column is channel padding)
       if (same_layout) {
@@ -737,39 +811,107 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
       for (int e = 0; e < 16; ++e) park[(t * 16 + e) * 64] = acc[t][e];
   }
   __syncthreads();
-  if (ph == 0) {
-    // partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+(lane&31)]
-    int32_t* out = a.partial + static_cast<long long>(item.z) * a.slice_stride;
-    const int c = c0 + (lane & 31);
+  // partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+(lane&31)]
+  const int c = c0 + (lane & 31);
+  if constexpr (!kFinish) {
+    if (ph == 0) {
+      int32_t* out = a.partial + static_cast<long long>(item.z) * a.slice_stride;
 #pragma unroll
-    for (int g = 0; g < 4; ++g)
+      for (int g = 0; g < 4; ++g)
 #pragma unroll
-      for (int e = 0; e < 4; ++e) {
-        const int k = k0 + wk * 32 + g * 8 + lk * 4 + e;
+        for (int e = 0; e < 4; ++e) {
+          const int k = k0 + wk * 32 + g * 8 + lk * 4 + e;
 #pragma unroll
-        for (int t = 0; t < 9; ++t) {
-          const int v = acc[t][4 * g + e] + park[(t * 16 + 4 * g + e) * 64];
-          if (c < a.Cp && k < a.K) {
-            int32_t* const dst = out + (static_cast<long long>(k) * 9 + t) * a.Cp + c;
-            if constexpr (kFinish) __hip_atomic_store(dst, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);   // written through to memory
-            else *dst = v;
+          for (int t = 0; t < 9; ++t) {
+            const int v = acc[t][4 * g + e] + park[(t * 16 + 4 * g + e) * 64];
+            if (c < a.Cp && k < a.K) out[(static_cast<long long>(k) * 9 + t) * a.Cp + c] = v;
           }
         }
-      }
-  }
-  if constexpr (kFinish) {
+    }
+  } else {
     // ---- the finishing pass in the same launch: all workgroups are resident (the host checks), every one takes a
     // share of the gradient's columns once the partial sums of all of them are in memory.  The sums travel between
     // the dies by write-through stores, completed before the arrival slot is filled, and by loads that bypass stale
     // lines (fences would do the same by writing back and invalidating whole L2 caches, once per wavefront: 50 us).
+    // What bounds this part is the bytes, so the sums go as 24-bit values whenever all of the workgroup's fit (planes
+    // of 16 and 8 bits; a third plane with the top bytes only when they do not).
+    // a lane holds four consecutive output channels of one (tap, input channel): one unit of each plane, and 32 lanes
+    // (input channels) make every store instruction whole 128-byte lines.  The values go biased by 2^23, so that the
+    // reader adds zero-extended 24-bit numbers and takes the bias off once per column.
+    const __amdgpu_buffer_rsrc_t rout =
+        __builtin_amdgcn_make_buffer_rsrc(a.partial, 0, static_cast<int>(a.slice_stride * f.splits * 4), 0x00020000);
+    constexpr int kSc1 = 16;   // written through to memory
+    const int zoff = static_cast<int>(item.z * a.slice_stride * 4);
+    const int units = static_cast<int>(f.nv);
+    uint32_t over = 0;   // bits above the 24 of any biased value
+    if (ph == 0) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int k = k0 + wk * 32 + g * 8 + lk * 4;
+        const bool live = c < a.Cp && k < a.K;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+          uint32_t v[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            v[e] = static_cast<uint32_t>(acc[t][4 * g + e] + park[(t * 16 + 4 * g + e) * 64]) + kPartialBias;
+            acc[t][4 * g + e] = static_cast<int>(v[e]);
+            over |= v[e];
+          }
+          const int u = ((k >> 2) * 9 + t) * a.Cp + c;
+          v2u lo;
+          lo[0] = __builtin_amdgcn_perm(v[1], v[0], 0x05040100u);   // v1.b1 v1.b0 v0.b1 v0.b0
+          lo[1] = __builtin_amdgcn_perm(v[3], v[2], 0x05040100u);
+          const uint32_t m01 = __builtin_amdgcn_perm(v[1], v[0], 0x0C0C0602u);   // 0 0 v1.b2 v0.b2
+          const uint32_t m23 = __builtin_amdgcn_perm(v[3], v[2], 0x06020C0Cu);   // v3.b2 v2.b2 0 0
+          __builtin_amdgcn_raw_buffer_store_b64(lo, rout, live ? u * 8 : kOob, zoff, kSc1);
+          __builtin_amdgcn_raw_buffer_store_b32(m01 | m23, rout, live ? units * 8 + u * 4 : kOob, zoff, kSc1);
+        }
+      }
+    }
+    // does any value of the workgroup need the third plane
+    over = __builtin_amdgcn_readfirstlane(static_cast<int>(wave_max_u32(over >> 24)));
+    uint32_t* const wgm = reinterpret_cast<uint32_t*>(dump);   // no load is in flight any more
+    if (lane == 0) wgm[wave] = over;
+    __syncthreads();
+    uint32_t m = 0;
+#pragma unroll
+    for (int w = 0; w < 8; ++w) m |= wgm[w];
+    const bool wide = __builtin_amdgcn_readfirstlane(static_cast<int>(m)) != 0;
+    if (wide && ph == 0) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int k = k0 + wk * 32 + g * 8 + lk * 4;
+        const bool live = c < a.Cp && k < a.K;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+          const uint32_t v0 = acc[t][4 * g], v1 = acc[t][4 * g + 1], v2 = acc[t][4 * g + 2], v3 = acc[t][4 * g + 3];
+          const uint32_t h01 = __builtin_amdgcn_perm(v1, v0, 0x0C0C0703u), h23 = __builtin_amdgcn_perm(v3, v2, 0x07030C0Cu);
+          const int u = ((k >> 2) * 9 + t) * a.Cp + c;
+          __builtin_amdgcn_raw_buffer_store_b32(h01 | h23, rout, live ? units * 12 + u * 4 : kOob, zoff, kSc1);
+        }
+      }
+    }
     const int nblocks = static_cast<int>(gridDim.x * gridDim.y * gridDim.z);
     const int block = static_cast<int>(blockIdx.x + gridDim.x * (blockIdx.y + gridDim.y * blockIdx.z));
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): this wavefront's stores have been performed
     __syncthreads();
-    if (tid == 0) __hip_atomic_store(slot_word(f.arrive, block), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (wave == 0) wait_slots(f.arrive, nblocks, f.spin_limit, &f.sync[1], f.sticky);
+    if (tid == 0) {
+      if (wide) {
+        __hip_atomic_store(f.wide + item.x + f.tiles_k * (item.y + f.tiles_c * item.z), 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __builtin_amdgcn_s_waitcnt(0x0F70);
+      }
+      // the slot's value also says which form this workgroup used: the largest over all slots tells every workgroup
+      // whether it has to look at the per-workgroup words at all
+      __hip_atomic_store(slot_word(f.arrive, block), wide ? 2u : 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (wave == 0) {
+      const uint32_t seen = wait_slots(f.arrive, nblocks, f.spin_limit, &f.sync[1], f.sticky);
+      if (lane == 0) wgm[8] = seen;
+    }
     __syncthreads();
-    finish_columns<8, kFusedV, true>(f, block, nblocks, *reinterpret_cast<FinishShared<8>*>(smem), predicted_raw);
+    const bool any_wide = static_cast<uint32_t>(__builtin_amdgcn_readfirstlane(static_cast<int>(wgm[8]))) >= 2u;
+    finish_columns<8, kFusedV, true>(f, block, nblocks, *reinterpret_cast<FinishShared<8>*>(smem), predicted_raw, any_wide);
   }
 }
 
@@ -960,6 +1102,8 @@ static int launch_wgrad3x3_partials(const int8_t* act, const int8_t* err, int N,
     finish->partial = a.partial;
     finish->slice_stride = a.slice_stride;
     finish->splits = splits;
+    finish->tiles_k = (K + 127) / 128;
+    finish->tiles_c = (C + 31) / 32;
   }
   if (narrow) {
     if (H == 32) return launch_narrow_geom<32, 8, 1>(a, splits, stream, finish);
@@ -998,7 +1142,10 @@ int wgrad3x3_finish_blocks(int C, int K) {
 
 // header, range slots (of the finishing launch or of the one-launch form, whichever has more workgroups), arrival slots
 static size_t range_slot_words(int blocks) { return slot_words(blocks > kArriveSlots ? blocks : kArriveSlots); }
-size_t wgrad3x3_sync_words(int blocks) { return static_cast<size_t>(kFinishSlot0) + range_slot_words(blocks) + slot_words(kArriveSlots); }
+// ... and the words that say which workgroups wrote int32 sums (one-launch form)
+size_t wgrad3x3_sync_words(int blocks) {
+  return static_cast<size_t>(kFinishSlot0) + range_slot_words(blocks) + slot_words(kArriveSlots) + 16 + kArriveSlots;
+}
 static size_t wgrad3x3_arrive_offset(int C, int K) { return static_cast<size_t>(kFinishSlot0) + range_slot_words(wgrad3x3_finish_blocks(C, K)); }
 
 int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int w_channels, int N, int H, int C, int K,
@@ -1062,6 +1209,7 @@ int launch_wgrad3x3_update(const int8_t* act, const int8_t* err, int8_t* w, int 
   f.exp_b = rq.exp_b;
   f.exp_out = rq.exp_out;
   f.arrive = sync + wgrad3x3_arrive_offset(C, K);
+  f.wide = f.arrive + slot_words(kArriveSlots);
   {
     // main loop and finishing pass as one launch where its grid is resident at once (NITI_WGRAD_ONE_LAUNCH=0 pins the pair)
     const char* e = getenv("NITI_WGRAD_ONE_LAUNCH");

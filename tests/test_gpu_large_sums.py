@@ -122,6 +122,37 @@ def test_wgrad_sums_beyond_2_24(dev, case):
             assert torch.equal(g8.cpu(), g8_ref) and torch.equal(wd.cpu(), w_ref), (f32, method)
 
 
+@pytest.mark.parametrize("case", [(12, 16, 128, 128), (48, 8, 64, 256)])   # N, Q, C, K
+def test_wgrad_one_launch_partial_sums_beyond_2_23(dev, case, monkeypatch):
+    """The one-launch weight gradient hands its partial sums over as 24-bit values unless a workgroup's own sums need
+    more: few, long workgroups (NITI_WGRAD_BLOCKS) and constant +-127 operands in the first input-channel tile of the
+    first pixel range make exactly one kind of workgroup write 32-bit sums, next to others of the same slice and of the
+    same tile that do not."""
+    from niti_amd import ops
+    from oracle import c_oracle as co
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("wgrad one launch, partial sums > 2^23", case)
+    monkeypatch.setenv("NITI_WGRAD_BLOCKS", "16")
+    g = torch.Generator().manual_seed(4400 + Q)
+    act, err, w = ri8(g, N, Q, Q, C, lo=-20, hi=20), ri8(g, N, Q, Q, K, lo=-20, hi=20), ri8(g, K, 3, 3, C)
+    n_hot = N // 4                      # the first of at least four pixel ranges
+    act[:n_hot, :, :, :32] = 127
+    err[:n_hot] = 127
+    err[:n_hot, :, :, 1::2] = -127
+    dw = co.conv_wgrad(act, err, 3, 3, 1, 1)
+    assert int(dw.abs().max()) > 2 ** 23 and int(dw[:, :, :, 32:].abs().max()) < 2 ** 22
+    for method, mu in (("psto", 5), ("round", 4)):
+        g8_ref, sh_ref = po.grad_calc(dw, mu, method)
+        w_ref = po.weight_update(w, g8_ref)
+        wd = w.to(dev).clone()
+        g8, dwo, sh, sync = ops.conv2d_wgrad_update(act.to(dev), err.to(dev), wd, mu=mu, method=method, want_grad=True, want_dw=True)
+        sync = sync.cpu()
+        assert int(sync[1]) == 0 and int(sync[0]) == po.absmax(dw), method
+        assert torch.equal(dwo.cpu(), dw) and int(sh.cpu()) == sh_ref, method
+        assert torch.equal(g8.cpu(), g8_ref) and torch.equal(wd.cpu(), w_ref), method
+
+
 PLANT = 2 ** 22 + 2     # bit width 23 as an integer, 22 under the reference's float32 log2 (ti_torch.py:366-377)
 
 
