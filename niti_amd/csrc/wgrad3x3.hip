@@ -71,7 +71,7 @@ __device__ inline WorkItem die_local_work_item() {
   return w;
 }
 
-// One stage of the main loop: four reduction steps of 32 pixels x three filter rows x three taps, all fragments by
+// One stage of the main loop: KS reduction steps of 32 pixels x three filter rows x three taps, all fragments by
 // transposing LDS reads.  The reads are inline assembly (see lds_asm.h: the builtin form would wait for the loads
 // of the following stages, just issued, before every read) and run one filter row ahead of the MFMAs: row i + 1 is
 // requested, then the wait leaves exactly those requests in flight, then row i multiplies.
@@ -82,7 +82,7 @@ __device__ inline WorkItem die_local_work_item() {
 // sum_q err[q] act[q+s-1] = sum_q' err[q'-s+1] act[q'] -, once per reduction step for all three filter rows (8 byte
 // shifts instead of 24 per nine MFMAs), and every filter row reads one aligned activation fragment (b_base then names
 // the pixels themselves, halo column + 1): 8 instead of 11 LDS reads.
-template <int Q, int BR, int HR, int ROWB, bool kShiftTaps, int NB, bool kShiftErr = false>
+template <int Q, int BR, int HR, int ROWB, bool kShiftTaps, int NB, bool kShiftErr = false, int KS = 4>
 __device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const int (&b_base)[NB], v16i (&acc)[9]) {
   v2i alo[2], ahi[2];   // [reduction step & 1]
   v2i rd[2][NB];        // [row step & 1]
@@ -100,11 +100,11 @@ __device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const
     for (int q = 0; q < NB; ++q) rd[step & 1][q] = lds_read_tr8<(hrow0 + r) * ROWB>(sbase + b_base[q]);
   };
   request(std::integral_constant<int, 0>{});
-  static_for<12>([&](auto stepc) {
+  static_for<3 * KS>([&](auto stepc) {
     constexpr int step = decltype(stepc)::value;
     constexpr int ks = step / 3, r = step % 3;
-    if constexpr (step + 1 < 12) request(std::integral_constant<int, step + 1>{});
-    lds_settle<(step + 1 < 12) ? NB + ((step + 1) % 3 == 0 ? 2 : 0) : 0>();
+    if constexpr (step + 1 < 3 * KS) request(std::integral_constant<int, step + 1>{});
+    lds_settle<(step + 1 < 3 * KS) ? NB + ((step + 1) % 3 == 0 ? 2 : 0) : 0>();
     if constexpr (r == 0) af[ks & 1] = lds_landed(alo[ks & 1], ahi[ks & 1]);
     v2i (&d)[NB] = rd[step & 1];
 #pragma unroll
@@ -655,12 +655,15 @@ struct NGeom {
   static constexpr int REDUCE_BYTES = 4 * 9 * 16 * 64 * 4;  // four wavefronts park their accumulators
   static constexpr int LDS_BYTES = (STAGES * STAGE_BYTES > REDUCE_BYTES ? STAGES * STAGE_BYTES : REDUCE_BYTES) + 1024;
   static constexpr int HALF_ROWS = NI > 1 ? (NI / 2) * HR : 128 / Q;  // halo rows between the two pixel halves of a stage
+  static constexpr int QUARTER_ROWS = NI > 1 ? (NI / 4) * HR : 64 / Q;  // ... between its four pixel quarters (kHalfK)
   static_assert(BR * NI * Q == 256, "a stage is 256 output pixels");
   static_assert(NI == 1 || BR == Q, "several images per stage only as whole images");
   static_assert(LDS_BYTES <= 160 * 1024, "stages must fit in LDS");
 };
 
-template <int Q, int BR, int NI, bool kFinish>
+// kHalfK (at most 64 output channels): the wavefronts are 2 channel quarters x 4 pixel quarters instead of 4 x 2, so
+// that none multiplies channels that do not exist.
+template <int Q, int BR, int NI, bool kFinish, bool kHalfK>
 __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs a, const FinishArgs f) {
   using G = NGeom<Q, BR, NI>;
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -738,8 +741,11 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   const int j = lane & 15;
   const int gg = (lane >> 4) & 1;
   const int lk = lane >> 5;
-  const int wk = wave & 3;    // 32-output-channel quarter of the tile
-  const int ph = wave >> 2;   // 128-pixel half of a stage
+  const int wk = kHalfK ? wave & 1 : wave & 3;     // 32-output-channel quarter of the tile
+  const int ph = kHalfK ? wave >> 1 : wave >> 2;   // 128-pixel half (64-pixel quarter) of a stage
+  constexpr int kWavePixels = kHalfK ? 64 : 128;
+  constexpr int kPartRows = kHalfK ? G::QUARTER_ROWS : G::HALF_ROWS;
+  static_assert(!kHalfK || Q >= 8, "pixel quarters only for rows of at least 8 pixels");
   int a_base[2];
   // Rows of at least 8 pixels: the second and third tap of a filter row are byte shifts of the first one's pixels
   // (3 or 4 reads per filter row).  Shorter rows (4 x 4 and 2 x 2 maps: eight pixels are two or four rows) read
@@ -752,14 +758,14 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
   for (int o = 0; o < 2; ++o) {
     const int lpix = 16 * lk + 8 * o + (j >> 1);
     const int cb = wk * 32 + gg * 16 + 8 * (j & 1);
-    a_base[o] = (ph * 128 + lpix) * 128 + ((((cb >> 4) ^ ((lpix >> 1) & 7)) << 4) | (cb & 15));
+    a_base[o] = (ph * kWavePixels + lpix) * 128 + ((((cb >> 4) ^ ((lpix >> 1) & 7)) << 4) | (cb & 15));
   }
   {
     const int cb = gg * 16 + 8 * (j & 1);
     // lrow: output row inside the 32 pixels of a reduction step (which may span several whole images)
     auto slot_addr = [&](int lrow, int w) {
       const int hrow = (lrow / BR) * G::HR + lrow % BR;
-      return G::ERR_BYTES + ((ph * G::HALF_ROWS + hrow) * G::RP + w) * 32 + cb;
+      return G::ERR_BYTES + ((ph * kPartRows + hrow) * G::RP + w) * 32 + cb;
     };
     const int p0 = 16 * lk + (j >> 1), p1 = p0 + 8;
     if constexpr (kShiftErr) {
@@ -798,13 +804,31 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
     else wg_wait_vmcnt<0>();
     wg_sync();
     if (it + G::STAGES - 1 < nb) issue(band_begin + it + G::STAGES - 1, (it + G::STAGES - 1) % G::STAGES);
-    wgrad_stage<Q, BR, G::HR, G::RP * 32, kShiftTaps, NB, kShiftErr>(lds_addr(smem + (it % G::STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
+    wgrad_stage<Q, BR, G::HR, G::RP * 32, kShiftTaps, NB, kShiftErr, kHalfK ? 2 : 4>(lds_addr(smem + (it % G::STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
   }
 
   // ---- add the two pixel halves: half 1 -> LDS -> half 0 -> memory.  Slot layout [value][lane].
   __syncthreads();  // all tiles consumed, no load in flight (the last stage was waited for with vmcnt(0))
   int32_t* const park = reinterpret_cast<int32_t*>(smem) + wk * (9 * 16 * 64) + lane;
-  if (ph == 1) {
+  if constexpr (kHalfK) {
+    // four pixel quarters: 1 -> 0 and 3 -> 2 first (four parked wavefronts fill the area), then 2 -> 0 like the halves
+    int32_t* const park2 = park + (ph >> 1) * (2 * 9 * 16 * 64);
+    if ((ph & 1) != 0) {
+#pragma unroll
+      for (int t = 0; t < 9; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) park2[(t * 16 + e) * 64] = acc[t][e];
+    }
+    __syncthreads();
+    if ((ph & 1) == 0) {
+#pragma unroll
+      for (int t = 0; t < 9; ++t)
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[t][e] += park2[(t * 16 + e) * 64];
+    }
+    __syncthreads();
+  }
+  if (ph == (kHalfK ? 2 : 1)) {
 #pragma unroll
     for (int t = 0; t < 9; ++t)
 #pragma unroll
@@ -1003,11 +1027,11 @@ int pick_splits(int N, int Q, int C, int K) {
 
 // f != nullptr: the one-launch form (main loop + finishing pass); returns NITI_ERR_UNSUPPORTED without launching when its
 // grid would not be resident at once, and the caller then runs the pair of launches.
-template <int Q, int BR, int NI, bool kFinish>
+template <int Q, int BR, int NI, bool kFinish, bool kHalfK>
 int launch_narrow_geom_as(const WgradArgs& a, int splits, hipStream_t stream, const FinishArgs& f) {
   using G = NGeom<Q, BR, NI>;
   constexpr size_t lds = G::LDS_BYTES;
-  auto k = wgrad3x3_narrow_kernel<Q, BR, NI, kFinish>;
+  auto k = wgrad3x3_narrow_kernel<Q, BR, NI, kFinish, kHalfK>;
   static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
   static int resident_of[kDeviceSlots] = {};    // workgroups of this kernel the device holds at once
   bool& attr_set = attr_set_of[device_slot()];
@@ -1037,11 +1061,15 @@ int launch_narrow_geom_as(const WgradArgs& a, int splits, hipStream_t stream, co
 template <int Q, int BR, int NI>
 int launch_narrow_geom(const WgradArgs& a, int splits, hipStream_t stream, const FinishArgs* f) {
   if constexpr (Q >= 8) {
-    if (f != nullptr) return launch_narrow_geom_as<Q, BR, NI, true>(a, splits, stream, *f);
+    const bool half_k = a.K <= 64;   // two channel quarters x four pixel quarters
+    if (f != nullptr)
+      return half_k ? launch_narrow_geom_as<Q, BR, NI, true, true>(a, splits, stream, *f) : launch_narrow_geom_as<Q, BR, NI, true, false>(a, splits, stream, *f);
+    return half_k ? launch_narrow_geom_as<Q, BR, NI, false, true>(a, splits, stream, FinishArgs{})
+                  : launch_narrow_geom_as<Q, BR, NI, false, false>(a, splits, stream, FinishArgs{});
   } else {
     if (f != nullptr) return NITI_ERR_UNSUPPORTED;
+    return launch_narrow_geom_as<Q, BR, NI, false, false>(a, splits, stream, FinishArgs{});
   }
-  return launch_narrow_geom_as<Q, BR, NI, false>(a, splits, stream, FinishArgs{});
 }
 
 template <int Q, int BR, int NI>
