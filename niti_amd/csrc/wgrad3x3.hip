@@ -17,7 +17,9 @@
 // and the activation rows with their halo once, and serves all nine taps from that one halo
 // tile, so activations are read from L2 once instead of nine times.  The pixel range is split
 // over gridDim.z workgroups; each writes its partial sums to a workspace slice and a second
-// kernel adds the slices (integer addition: any split gives the same result).
+// kernel adds the slices (integer addition: any split gives the same result).  The arrangement with
+// 128 x 32 tiles (wgrad3x3_narrow_kernel) can also add the slices itself, at the end of the same
+// launch, once all of its workgroups - resident together - have written theirs.
 #include <stdlib.h>
 
 #include <type_traits>
