@@ -400,6 +400,16 @@ for i in range(4):
     torch.cuda.synchronize()
     flagged += int(sync.cpu()[1] != 0)
 print("FLAGGED", flagged, "ARENA", int(ops.sync_arena.timed_out(dev)))
+# the one-launch weight gradient waits twice (arrival of the partial sums, range): same limit, same flag
+act = torch.randint(-127, 128, (16, 16, 16, 64), generator=g, dtype=torch.int8).to(dev)
+err = torch.randint(-127, 128, (16, 16, 16, 128), generator=g, dtype=torch.int8).to(dev)
+wflag = 0
+for i in range(4):
+    wd = w.clone()
+    _, _, _, sync = ops.conv2d_wgrad_update(act, err, wd, mu=5, method="psto")
+    torch.cuda.synchronize()
+    wflag += int(sync.cpu()[1] != 0)
+print("WGRAD_FLAGGED", wflag)
 # the device-wide word survives the arena's reset, is cleared by a read, and the epoch driver's check raises on it
 ops.sync_arena.reset(dev)
 print("STICKY", int(ops.sync_arena.timed_out(dev)), int(ops.sync_timeouts(dev, clear=False)), int(ops.sync_timeouts(dev)),
@@ -419,6 +429,7 @@ except train.GridWaitTimeout:
     assert out.returncode == 0, out.stderr[-2000:]
     line = [l for l in out.stdout.splitlines() if l.startswith("FLAGGED")][0].split()
     assert int(line[1]) >= 1 and int(line[3]) == 1
+    assert int([l for l in out.stdout.splitlines() if l.startswith("WGRAD_FLAGGED")][0].split()[1]) >= 1
     sticky = [l for l in out.stdout.splitlines() if l.startswith("STICKY")][0].split()
     assert sticky[1:] == ["0", "1", "1", "0"], sticky
     assert "RAISED 1" in out.stdout
