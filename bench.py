@@ -49,11 +49,12 @@ def laplace_i8(g, shape, b=16.0):
 class ConvTriple:
     """Device state and one step of the conv-triple workload."""
 
-    def __init__(self, dev, seed=1236):
+    def __init__(self, dev, seed=1236, restore_weights=True):
         import torch
         import torch.nn.functional as F
         from niti_amd import ops
         self.torch, self.ops, self.dev = torch, ops, dev
+        self.restore_weights = restore_weights
         g = torch.Generator().manual_seed(seed)
         self.layers = []
         for (c, k, hw) in LAYERS:
@@ -84,6 +85,29 @@ class ConvTriple:
         self.sync = self.zeroed[:sync_words]
         self.absmax = self.zeroed[sync_words:]
         self.ws = ops.scratch(256 << 20, dev)    # shared by all weight-gradient launches
+        # Every step updates the weights (and their kernel-ready copies) in place.  So that each timed step multiplies
+        # the operands the configuration names - weights uniform in [-127, 127] from the seed, not the saturated values
+        # thousands of identical updates would leave - all weights and filter copies live in ONE buffer that the step
+        # restores from a pristine copy with a single device copy before anything else.
+        segs = []
+        for L in self.layers:
+            c, hw = L["c"], L["hw"]
+            L["w16"] = F.pad(L["w"], (0, 16 - c % 16)).contiguous() if c % 16 else L["w"]
+            L["wp"] = ops.conv_filter_prepare(L["w16"], BATCH, hw, hw)
+            segs += [(L, "w"), (L, "wp")] if L["wp"] is not None else [(L, "w")]
+        total = sum((L[key].numel() + 255) // 256 * 256 for L, key in segs)
+        self.wflat = torch.empty(total, dtype=torch.int8, device=dev)
+        o = 0
+        for L, key in segs:
+            t = L[key]
+            view = self.wflat[o:o + t.numel()].view(t.shape)
+            view.copy_(t)
+            if key == "w" and L["w16"] is t:
+                L["w16"] = view
+            L[key] = view
+            o += (t.numel() + 255) // 256 * 256
+        self.wpristine = self.wflat.clone()
+        self.restore_bytes = total
         self.exp0 = torch.zeros(1, dtype=torch.int32, device=dev)
         self.ops_per_step = sum(conv_ops(BATCH, hw, c, k) * (2 if i == 0 else 3) for i, (c, k, hw) in enumerate(LAYERS))
         self.main_kernel_ops = []     # algorithmic ops of every launch bracketed by events, in launch order
@@ -94,11 +118,13 @@ class ConvTriple:
         torch, ops = self.torch, self.ops
         import torch.nn.functional as F
         self.zeroed.zero_()
+        if self.restore_weights:
+            self.wflat.copy_(self.wpristine)
         for i, L in enumerate(self.layers):
             c, k, hw = L["c"], L["k"], L["hw"]
             am = self.absmax[3 * i: 3 * i + 3]
-            if L.get("wp") is None or not c % 16:
-                L["w16"] = F.pad(L["w"], (0, 16 - c % 16)).contiguous() if c % 16 else L["w"]
+            if L.get("wp") is None and c % 16:
+                L["w16"] = F.pad(L["w"], (0, 16 - c % 16)).contiguous()
             w16 = L["w16"]        # with a maintained filter copy only its shape is used
             # forward + activation requantisation; the kernel-ready forward filter copy is made once and from then
             # on maintained by the weight update below
@@ -212,7 +238,7 @@ class Runner:
             self.graphs[0].replay()
 
 
-def cpu_baseline(min_seconds=10.0):
+def cpu_baseline(min_seconds=5.0):
     """The plain-C oracle (OpenMP) over the same six layer triples, on synthetic inputs of the same
     shapes, repeated until at least `min_seconds` of CPU work."""
     import torch
@@ -239,6 +265,52 @@ def cpu_baseline(min_seconds=10.0):
         passes += 1
     return {"value": ops_total / t_total / 1e12, "unit": "TOPS", "cores": co.num_threads(), "kind": "port",
             "sample": "%d pass(es) of the full six-layer conv triple at batch %d (plain-C oracle, OpenMP), %.1f s" % (passes, BATCH, t_total)}
+
+
+def cpu_baseline_train_step(batch=BATCH):
+    """One complete integer training step of VGG-small (configs[3]) on the host cores: the reference's layer stack
+    and reverse-order backward (ti_net.py:17-32, ti_torch.py:235-455) restated on torch CPU int32 tensors - integer
+    convolutions through F.conv2d on int32 operands with the reference's own operand rewrites for the two gradients,
+    int32 matrix products, the literal requantisation sequences.  One warm-up pass on a batch of 8, one timed pass."""
+    import torch
+    from oracle import niti_model_oracle as mo
+    from niti_amd import ti_vgg
+    cfg_list = ti_vgg.cifar_cfg[7]
+    g = torch.Generator().manual_seed(1237 + 7)
+    weights, c = [], 3
+    for v in cfg_list:
+        if v != 'M':
+            weights.append(torch.randint(-127, 128, (v, 3, 3, c), generator=g, dtype=torch.int8))
+            c = v
+    weights.append(torch.randint(-127, 128, (10, 512 * 4 * 4), generator=g, dtype=torch.int8))
+    mask = torch.randint(0, 2, (512 * 4 * 4,), generator=g, dtype=torch.int8)
+
+    def one(n):
+        net = mo.build_vgg(cfg_list, weights, [-8] * len(weights), mo.Cfg(), mask)
+        x = torch.randint(-127, 128, (n, 32, 32, 3), generator=g, dtype=torch.int8)
+        target = torch.randint(0, 10, (n,), generator=g)
+        rand = torch.randint(0, 16, (n, 10), generator=g, dtype=torch.int32)
+        t0 = time.perf_counter()
+        net.forward_int8(x, 0)
+        net.backward(target, rand)
+        return time.perf_counter() - t0
+
+    one(8)
+    dt = one(batch)
+    model = ""
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("model name"):
+                    model = line.split(":", 1)[1].strip()
+                    break
+    except OSError:
+        pass
+    return {"value": batch / dt, "unit": "images/s", "seconds_per_step": round(dt, 3), "cores": torch.get_num_threads(),
+            "os_cpu_count": os.cpu_count(), "cpu_model": model, "kind": "port",
+            "sample": "1 warm-up pass at batch 8 + 1 timed pass of the full VGG-small (6 conv + FC) integer training step at "
+                      "batch %d: forward, TiLoss gradient, backward, weight updates (torch CPU int32 restatement of the "
+                      "reference's layers)" % batch}
 
 
 def train_step_rate(dev, steps, warmup, depth=7, batch=BATCH, graph=True, unroll=1):
@@ -299,10 +371,13 @@ def mfma_probe(dev):
     g = torch.Generator().manual_seed(4321)
     const = torch.ones(1 << 20, dtype=torch.int8, device=dev)
     rnd = torch.randint(-127, 128, (1 << 20,), generator=g, dtype=torch.int8).to(dev)
+    zero = torch.zeros(1 << 20, dtype=torch.int8, device=dev)
     ops.mfma_probe(const)                              # clocks up
+    zt, zg = ops.mfma_probe(zero)
     ct, cg = ops.mfma_probe(const)
     rt, rg = ops.mfma_probe(rnd)
-    return {"constant_operands_tops": round(ct, 1), "constant_operands_clock_ghz": round(cg, 2),
+    return {"zero_operands_tops": round(zt, 1), "zero_operands_clock_ghz": round(zg, 2),
+            "constant_operands_tops": round(ct, 1), "constant_operands_clock_ghz": round(cg, 2),
             "random_operands_tops": round(rt, 1), "random_operands_clock_ghz": round(rg, 2),
             "note": "512 workgroups x 8 wavefronts x 1200 x 12 v_mfma_i32_32x32x32_i8 on register operands; clock = shader "
                     "cycle counter against the 100 MHz wall clock inside the loop"}
@@ -426,6 +501,12 @@ TRAIN_STEPS = (("train_step", 7, BATCH, "BASELINE configs[3]: VGG-small (6 conv 
                ("train_step_vgg13", 13, 256, "BASELINE configs[4]: VGG-13 widths (10 conv + FC) integer training step, batch 256"))
 
 
+# the reference's default batch size (options.py:3) and the only speeds it publishes: seconds per iteration in its
+# committed training logs (results/int-vgg-small-{7,8,9}/results.log:12; data loading, display loss and host
+# synchronisations included, GPU model not recorded)
+TRAIN_STEPS_B256 = (("train_step_b256_vgg7", 7, 0.088), ("train_step_b256_vgg8", 8, 0.118), ("train_step_b256_vgg9", 9, 0.130))
+
+
 def train_step_objects(dev, steps, warmup, graph=True, unroll=1):
     out = {}
     for name, depth, batch, workload in TRAIN_STEPS:
@@ -434,6 +515,18 @@ def train_step_objects(dev, steps, warmup, graph=True, unroll=1):
             out[name] = {"workload": workload, "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": mode,
                          "steps_per_graph": unroll if mode == "graph" else None}
         except Exception as e:  # the headline line must still be printed
+            out[name] = {"error": str(e)[:200]}
+    for name, depth, ref_s in TRAIN_STEPS_B256:
+        try:
+            ips, ms, mode = train_step_rate(dev, steps, warmup, depth, 256, graph, unroll)
+            out[name] = {"workload": "cifar_cfg[%d] of the reference (ti_vgg.py:10-14), integer training step at its default batch "
+                                     "256 (options.py:3)" % depth,
+                         "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": mode,
+                         "reference_published_s_per_iter": ref_s,
+                         "reference_published_images_per_s": round(256 / ref_s, 1),
+                         "reference_note": "results/int-vgg-small-%d/results.log:12, whole iteration (data loading, display "
+                                           "loss, host synchronisations) on an unrecorded NVIDIA GPU: not the same quantity" % depth}
+        except Exception as e:
             out[name] = {"error": str(e)[:200]}
     return out
 
@@ -445,6 +538,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-train-step", action="store_true")
+    ap.add_argument("--no-drift-ab", action="store_true",
+                    help="skip timing the step without the per-step weight restore (weights drifting to +-127)")
     ap.add_argument("--no-side-workloads", action="store_true", help="skip config0 / config1 / max-pool figures")
     ap.add_argument("--sustained-seconds", type=float, default=1.0,
                     help="also replay the headline step back to back for at least this long (0: skip)")
@@ -564,7 +659,7 @@ def main():
         per_layer.append(row)
     # HBM bytes per launch of this kernel as the counters of an earlier rocprofv3 run gave them (the summary states
     # the figure on a line of its own); null when the summary is not there
-    traffic = None
+    traffic = wgrad_traffic = None
     tpath = os.path.join(ROOT, "profiles", "conv_triple_hbm_traffic.txt")
     traffic_source = None
     if os.path.exists(tpath):
@@ -574,6 +669,22 @@ def main():
             for line in f:
                 if line.startswith("traffic_bytes_per_launch:"):
                     traffic = int(line.split(":", 1)[1].split()[0])
+                if line.startswith("wgrad_traffic_bytes_per_launch:"):
+                    wgrad_traffic = int(line.split(":", 1)[1].split()[0])
+    # the weight-gradient family (layers 2-6: wgrad3x3_narrow_kernel with its finishing pass inside), same brackets
+    wsel = [ev for ev in wl.wgrad_events if ev[3] > 0]
+    w_ms = sum(max(ev[0].elapsed_time(ev[1]) - pair_ms, 0.0) for ev in wsel)
+    w_ops = sum(ev[2] for ev in wsel)
+    w_achieved = w_ops / (w_ms * 1e-3) / 1e12 if w_ms > 0 else 0.0
+    w_alg_bytes = sum(BATCH * hw * hw * (c + k) + 3 * k * 9 * c for (c, k, hw) in LAYERS[1:]) / (len(LAYERS) - 1)
+    roofline_wgrad = {"bound": "mfma", "achieved": round(w_achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
+                      "frac": round(w_achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": wgrad_traffic,
+                      "traffic_source": traffic_source,
+                      "kernel": "wgrad3x3_narrow_kernel<..., true> (weight gradient + gradient rounding + weight update + "
+                                "filter copy, one launch; layers 2-6)",
+                      "launches": len(wsel), "avg_launch_us": round(w_ms * 1e3 / max(len(wsel), 1), 2),
+                      "ops_per_launch_avg": w_ops / max(len(wsel), 1), "algorithmic_bytes_per_launch_avg": int(w_alg_bytes),
+                      "note": "algorithmic bytes = |x| + |err| + 3 |w| (weights read and written, kernel-ready filter copy written)"}
     roofline = {"bound": "mfma", "achieved": round(achieved, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TFLOP/s",
                 "frac": round(achieved / INT8_MFMA_PEAK_TOPS, 4), "traffic": traffic, "traffic_source": traffic_source,
                 "kernel": "conv3x3_halo_kernel<..., true, *> (convolution + requantisation)", "launches": n_launch,
@@ -591,7 +702,33 @@ def main():
                       "ops_per_step": wl.ops_per_step, "batch": BATCH},
            "launch_mode": mode, "steps_per_graph": runner.unroll if mode == "graph" else None,
            "pct_int8_mfma_peak": round(100.0 * tops / INT8_MFMA_PEAK_TOPS, 2),
-           "roofline": roofline, "per_layer": per_layer}
+           "roofline": roofline, "roofline_wgrad": roofline_wgrad, "per_layer": per_layer}
+    out["weights"] = {"state": "every step starts from the seeded uniform int8 weights: all weights and kernel-ready filter copies "
+                               "are restored from a pristine copy by one device copy inside the timed step",
+                      "restored_bytes_per_step": wl.restore_bytes}
+    if not args.no_drift_ab:
+        # the same step without the restore: the weights drift (the same gradient every step drives them to +-127)
+        try:
+            wl2 = ConvTriple(dev, restore_weights=False)
+            r2 = Runner(wl2.step, args.warmup, not args.eager, args.steps_per_graph)
+            r2.run(500)                    # saturates the weights, as a long run would
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            r2.run(args.steps)
+            torch.cuda.synchronize()
+            drift_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+            runner.run(args.steps)         # and the restored form again, right after it
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            runner.run(args.steps)
+            torch.cuda.synchronize()
+            fresh_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+            out["weights"].update({"fresh_ms_per_step": round(fresh_ms, 4), "drifted_ms_per_step": round(drift_ms, 4),
+                                   "drifted_note": "no restore, weights updated in place for 500+ steps with the same inputs "
+                                                   "(nearly all at +-127); timed back to back with the restored form"})
+            del wl2, r2
+        except Exception as e:
+            out["weights"]["drift_ab_error"] = str(e)[:200]
     try:
         probe = mfma_probe(dev)
         out["mfma_probe"] = probe
@@ -610,6 +747,13 @@ def main():
         out.update(train_step_objects(dev, max(args.steps, 5), max(args.warmup, 2), True, args.steps_per_graph))
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline()
+        try:
+            cb = cpu_baseline_train_step()
+            out["cpu_baseline_train_step"] = cb
+            if "images_per_s" in out.get("train_step", {}):
+                out["train_step"]["vs_cpu_baseline"] = round(out["train_step"]["images_per_s"] / cb["value"], 1)
+        except Exception as e:
+            out["cpu_baseline_train_step"] = {"error": str(e)[:200]}
     print(json.dumps(out))
     return 0
 

@@ -212,7 +212,9 @@ def test_f32_bitwidth_rule_inside_the_fused_weight_gradient(dev):
             assert torch.equal(g8.cpu(), g8_ref) and torch.equal(wd.cpu(), po.weight_update(w, g8_ref)), (bw_mode, method)
 
 
-@pytest.mark.parametrize("depth,N", [(7, 128), (13, 256)])
+# (7, 256): the reference's default batch (options.py:3); its two 128-channel layers on 32 x 32 maps have more tiles than the
+# device holds at once and run the two-launch form inside the step
+@pytest.mark.parametrize("depth,N", [(7, 128), (7, 256), (13, 256)])
 def test_full_batch_steps_fused_against_two_pass(dev, depth, N):
     """Two training steps at the batch size of the benchmark configurations: the network with every single-launch
     form switched on against the same network on the two-pass launches (int32 results + separate requantisation),

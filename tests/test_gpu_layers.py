@@ -191,6 +191,10 @@ def _build_pair(tt, cfg_list, widths_in, N, seed, dropout, image=32):
     ("vgg7-narrow", [16, 16, 'M', 32, 32, 'M', 512, 512, 'M'], 8),
     ("vgg7-full", [128, 128, 'M', 256, 256, 'M', 512, 512, 'M'], 16),
     ("vgg13", [64, 64, 'M', 128, 128, 'M', 256, 256, 'M', 512, 512, 'M', 512, 512, 'M'], 8),
+    # cifar_cfg[8] and cifar_cfg[9] of the reference (ti_vgg.py:12-13): stages of three convolutions, i.e. convolutions
+    # whose ReLU is followed by another convolution instead of a pooling
+    ("vgg8", [128, 128, 128, 'M', 256, 256, 'M', 512, 512, 'M'], 8),
+    ("vgg9", [128, 128, 128, 'M', 256, 256, 256, 'M', 512, 512, 'M'], 8),
 ])
 def test_training_step(tt, name, cfg_list, N):
     """One complete integer training step (forward, loss gradient, backward, weight update)."""
