@@ -195,6 +195,26 @@ int niti_conv2d_i8_dgrad_requant_unpool(const int8_t* err, const int8_t* w, int8
                                         size_t workspace_bytes, void* stream);
 
 /*
+ * The two single-launch entry points above with StoShift (ti_torch.py:33-46; selectable as ACT_ROUND_METHOD /
+ * ERROR_ROUND_METHOD, ti_torch.py:460-463) folded in: rand holds one int32 per OUTPUT element, laid out like the
+ * output ([N,H,W,K] forward, [N,H,W,C] data gradient), 16-byte aligned; it stands in for the reference's device
+ * torch.randint(0, 2^shift) and only its low `shift` bits are used, so values drawn from any wider range work.  The
+ * result equals niti_conv2d_i8_fprop / _dgrad followed by niti_requant_i32_i8(.., NITI_ROUND_STOCHASTIC, rand, ..).
+ * pool_out (forward, may be NULL) as in niti_conv2d_i8_fprop_requant_pool.  Same coverage as the entry points above
+ * except maps of side 2 (NITI_ERR_UNSUPPORTED: use the two-pass entry points there).
+ */
+int niti_conv2d_i8_fprop_requant_sto(const int8_t* x, const int8_t* w, int8_t* y8, int8_t* pool_out, const int32_t* rand, int N, int H,
+                                     int W, int C, int K, int R, int S, int stride, int pad, unsigned flags, int target_bits,
+                                     int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync, size_t sync_words,
+                                     int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+int niti_conv2d_i8_dgrad_requant_sto(const int8_t* err, const int8_t* w, int8_t* dx8, const int32_t* rand, int N, int H, int W, int C,
+                                     int K, int R, int S, int stride, int pad, unsigned flags, int target_bits, int div_mode,
+                                     int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync, size_t sync_words,
+                                     int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b, int32_t* exp_out,
+                                     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * niti_conv2d_i8_fprop_requant for callers that cannot allocate device memory or hand in scratch memory: code under HIP
  * graph capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
  * arithmetic and the same results as niti_conv2d_i8_fprop_requant; the sync words and the kernel-ready filter copy live

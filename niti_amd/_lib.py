@@ -41,6 +41,8 @@ SIGNATURES = {
     "niti_conv2d_i8_fprop_requant": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _i, _i, _i, _i, _u, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "niti_conv2d_i8_fprop_requant_pool": (_i, [_vp, _vp, _vp, _vp] + [_i] * 9 + [_u, _i, _i, _i, _i, _u, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "niti_static_scratch_bytes": (_sz, []),
+    "niti_conv2d_i8_fprop_requant_sto": (_i, [_vp, _vp, _vp, _vp, _vp] + [_i] * 9 + [_u, _i, _i, _i, _u, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "niti_conv2d_i8_dgrad_requant_sto": (_i, [_vp, _vp, _vp, _vp] + [_i] * 9 + [_u, _i, _i, _i, _u, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "niti_conv2d_i8_fprop_requant_static": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _i, _i, _i, _i, _u, _vp, _vp, _vp, _vp, _vp, _vp]),
     "niti_conv2d_i8_dgrad_requant": (_i, [_vp, _vp, _vp] + [_i] * 9 + [_u, _i, _i, _i, _i, _u, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
     "niti_conv2d_i8_dgrad_requant_unpool": (_i, [_vp, _vp, _vp, _vp, _vp, _i] + [_i] * 9 + [_u, _i, _i, _i, _i, _u, _vp, _sz, _vp, _vp, _vp, _vp,

@@ -232,6 +232,7 @@ struct RequantSpec {
   const int8_t* pool_x = nullptr;   // the pooling's input [N,2H,2W,C]
   int8_t* unpool = nullptr;         // result [N,2H,2W,C] (the [N,H,W,C] output is then not written)
   int ties_all = 0;
+  const int32_t* rand = nullptr;    // conv + requantisation with NITI_ROUND_STOCHASTIC: one integer per output element
 };
 // wall-clock ticks (100 MHz) a grid-wide wait may last (api.hip)
 long long sync_spin_limit();

@@ -117,6 +117,7 @@ struct HaloArgs {
   long long unpool_bytes;
   int ties_all;
   int target_bits, method, trunc, bw_mode;
+  const int32_t* rand;   // NITI_ROUND_STOCHASTIC: one random integer per output element [N,Q,Q,K], low `shift` bits used
   unsigned rq_flags;
   long long spin_limit;  // wall-clock ticks (100 MHz) the wait may last
   uint32_t* sticky;      // device-wide word set when the wait gives up, may be null
@@ -174,8 +175,11 @@ struct HGeom {
 // kWT: the filter operand is the FORWARD copy of the filter of the convolution whose data gradient this launch
 // computes (input channels of this launch = that filter's output channels and vice versa, taps flipped); its
 // 32 x 32 byte blocks are staged as they are and transposed by ds_read_b64_tr_b8 when the fragments are read.
-template <int Q, int BR, int NI, int KT, bool kFused, bool kWT>
+// kSto: the requantising variant with StoShift (random integers read in the epilogue); instances of their own so that the
+// others keep their register allocation.
+template <int Q, int BR, int NI, int KT, bool kFused, bool kWT, bool kSto = false>
 __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) {
+  static_assert(kFused || !kSto);
   using G = HGeom<Q, BR, NI, KT>;
   constexpr int NWF = G::NWF;
   extern __shared__ __attribute__((aligned(16))) int8_t smem[];
@@ -681,6 +685,10 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     const bool trunc = a.trunc != 0;
     const bool relu = (a.rq_flags & NITI_RQ_RELU) != 0;
     const bool psto = a.method == NITI_ROUND_PSEUDO_STOCHASTIC;
+    // StoShift: the caller's random integer of each output element decides its rounding step; a tile that is rounded
+    // twice (final shift unlike the first) takes the low bits of the same integers for the other shift
+    constexpr bool sto = kSto;
+    const __amdgpu_buffer_rsrc_t rrand = __builtin_amdgcn_make_buffer_rsrc(const_cast<int32_t*>(a.rand), 0, sto ? a.y8_bytes * 4 : 0, 0x00020000);
     constexpr int PROW = NWF * 32 + 16;  // the wavefront's channels of one pixel, padded
     int8_t* patch = smem + wave * (32 * PT * PROW);
     const __amdgpu_buffer_rsrc_t ry = __builtin_amdgcn_make_buffer_rsrc(a.y8, 0, a.y8_bytes, 0x00020000);
@@ -752,7 +760,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       // here, the choice between the two forms below is ONE scalar branch.  (Left inside the loops as a per-lane
       // condition it cost every value both forms' set-up under execution masks and a taken branch.)
       const int ushift = __builtin_amdgcn_readfirstlane(shift);
-      const bool fast = ushift >= 1 && !trunc && !psto;
+      const bool fast = ushift >= 1 && !trunc && !psto && !sto;
       const int sm1 = ushift - 1, lo = relu ? 0 : -127;
       auto round_tiles = [&](auto fastc) {
         constexpr bool kFast = decltype(fastc)::value;
@@ -767,10 +775,18 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
                 packed = round4_nearest_floor_fast(acc[i][j][4 * g], acc[i][j][4 * g + 1], acc[i][j][4 * g + 2], acc[i][j][4 * g + 3], sm1, lo);
               } else {
                 int r[4];
+                v4i u = {0, 0, 0, 0};
+                if (sto) {   // the four values are consecutive channels of one pixel
+                  const int m = pixwave + j * 32 + lr, c0 = chbase + i * 32 + 8 * g + 4 * lk;
+                  u = __builtin_amdgcn_raw_buffer_load_b128(rrand, (m < total_pix && c0 < a.K) ? (m * a.K + c0) * 4 : kOob, 0, 0);
+                }
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                   const int x = acc[i][j][4 * g + e];
-                  if (ushift >= 1) r[e] = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, ushift, trunc) : round_one32<NITI_ROUND_NEAREST>(x, ushift, trunc);
+                  if (ushift >= 1)
+                    r[e] = sto    ? round_sto32(x, ushift, trunc, u[e])
+                           : psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(x, ushift, trunc)
+                                  : round_one32<NITI_ROUND_NEAREST>(x, ushift, trunc);
                   else r[e] = wrap_to_i8(x);
                   if (relu && r[e] < 0) r[e] = 0;
                 }
@@ -1207,14 +1223,14 @@ bool halo_two_pixel_tiles(long long pix, int K, int H, int ktile) {
   return (pix / 256) * ((K + 63) / 64) > 2LL * cus;
 }
 
-template <int Q, int BR, int NI, int KT, bool kFused, bool kWT>
+template <int Q, int BR, int NI, int KT, bool kFused, bool kWT, bool kSto = false>
 int launch_halo(const HaloArgs& a, hipStream_t stream) {
   using G = HGeom<Q, BR, NI, KT>;
   constexpr size_t lds = G::LDS_BYTES;
   static_assert(8 * 32 * (32 * 4 + 16) <= G::TILE_BYTES, "int32 patches must stay clear of the reduction words");
   static_assert(8 * 32 * G::PT * (G::NWF * 32 + 16) <= G::TILE_BYTES, "int8 patches must stay clear of the reduction words");
   static_assert(2 * lds <= 160 * 1024, "two workgroups per compute unit");
-  auto k = conv3x3_halo_kernel<Q, BR, NI, KT, kFused, kWT>;
+  auto k = conv3x3_halo_kernel<Q, BR, NI, KT, kFused, kWT, kSto>;
   static bool attr_set_of[kDeviceSlots] = {};   // function attributes are per device
   static int resident_of[kDeviceSlots] = {};     // workgroups the device holds at once
   const int slot = device_slot();
@@ -1292,35 +1308,39 @@ int launch_map2(const HaloArgs& a, hipStream_t stream) {
   return launch_map2_as<kFused, kWT, false>(a, stream);
 }
 
-template <bool kFused, bool kWT>
+template <bool kFused, bool kWT, bool kSto = false>
 int launch_halo_tiles(const HaloArgs& a, int H, hipStream_t stream) {
   if (H == 2) return launch_map2<kFused, kWT>(a, stream);
   const int ktile = halo_ktile(static_cast<long long>(a.N) * H * H, a.K, H);
   if (ktile == 128) {
-    if (H == 32) return launch_halo<32, 8, 1, 128, kFused, kWT>(a, stream);
-    if (H == 16) return launch_halo<16, 16, 1, 128, kFused, kWT>(a, stream);
-    if (H == 8) return launch_halo<8, 8, 4, 128, kFused, kWT>(a, stream);
-    return launch_halo<4, 4, 16, 128, kFused, kWT>(a, stream);
+    if (H == 32) return launch_halo<32, 8, 1, 128, kFused, kWT, kSto>(a, stream);
+    if (H == 16) return launch_halo<16, 16, 1, 128, kFused, kWT, kSto>(a, stream);
+    if (H == 8) return launch_halo<8, 8, 4, 128, kFused, kWT, kSto>(a, stream);
+    return launch_halo<4, 4, 16, 128, kFused, kWT, kSto>(a, stream);
   }
   if (ktile == 32) {
-    if (H == 16) return launch_halo<16, 16, 1, 32, kFused, kWT>(a, stream);
-    if (H == 8) return launch_halo<8, 8, 4, 32, kFused, kWT>(a, stream);
-    return launch_halo<4, 4, 16, 32, kFused, kWT>(a, stream);
+    if (H == 16) return launch_halo<16, 16, 1, 32, kFused, kWT, kSto>(a, stream);
+    if (H == 8) return launch_halo<8, 8, 4, 32, kFused, kWT, kSto>(a, stream);
+    return launch_halo<4, 4, 16, 32, kFused, kWT, kSto>(a, stream);
   }
   if constexpr (kFused) {
     if (halo_two_pixel_tiles(static_cast<long long>(a.N) * H * H, a.K, H, ktile)) {
-      if (H == 32) return launch_halo<32, 16, 1, 64, kFused, kWT>(a, stream);
-      return launch_halo<16, 16, 2, 64, kFused, kWT>(a, stream);
+      if (H == 32) return launch_halo<32, 16, 1, 64, kFused, kWT, kSto>(a, stream);
+      return launch_halo<16, 16, 2, 64, kFused, kWT, kSto>(a, stream);
     }
   }
-  if (H == 32) return launch_halo<32, 8, 1, 64, kFused, kWT>(a, stream);
-  if (H == 16) return launch_halo<16, 16, 1, 64, kFused, kWT>(a, stream);
-  if (H == 8) return launch_halo<8, 8, 4, 64, kFused, kWT>(a, stream);
-  return launch_halo<4, 4, 16, 64, kFused, kWT>(a, stream);
+  if (H == 32) return launch_halo<32, 8, 1, 64, kFused, kWT, kSto>(a, stream);
+  if (H == 16) return launch_halo<16, 16, 1, 64, kFused, kWT, kSto>(a, stream);
+  if (H == 8) return launch_halo<8, 8, 4, 64, kFused, kWT, kSto>(a, stream);
+  return launch_halo<4, 4, 16, 64, kFused, kWT, kSto>(a, stream);
 }
 
 template <bool kFused>
 int launch_halo_any(const HaloArgs& a, int H, hipStream_t stream) {
+  if constexpr (kFused) {
+    if (a.method == NITI_ROUND_STOCHASTIC)
+      return a.src_cslices > 0 ? launch_halo_tiles<true, true, true>(a, H, stream) : launch_halo_tiles<true, false, true>(a, H, stream);
+  }
   return a.src_cslices > 0 ? launch_halo_tiles<kFused, true>(a, H, stream) : launch_halo_tiles<kFused, false>(a, H, stream);
 }
 
@@ -1410,6 +1430,12 @@ int launch_conv3x3_halo_requant(const int8_t* x, const int8_t* wp, int8_t* y8, i
   a.method = rq.method;
   a.trunc = rq.trunc;
   a.bw_mode = rq.bw_mode;
+  a.rand = rq.rand;
+  if (rq.method == NITI_ROUND_STOCHASTIC) {
+    if (rq.rand == nullptr) return fail(NITI_ERR_INVALID_ARG, "conv_requant: stochastic rounding needs the random integers");
+    if (H == 2 || a.unpool != nullptr)
+      return fail(NITI_ERR_UNSUPPORTED, "conv_requant: stochastic rounding is not folded in on 2 x 2 maps or with the pooling's backward pass; use the two-pass path");
+  }
   a.rq_flags = rq.flags;
   a.spin_limit = rq.spin_limit;
   a.sticky = rq.sticky;

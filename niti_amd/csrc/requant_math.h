@@ -72,6 +72,26 @@ __host__ __device__ inline int round_one32(int x, int s, bool trunc) {
   return r > 127 ? 127 : (r < -127 ? -127 : r);
 }
 
+// StoShift in 32-bit arithmetic (1 <= s <= 31): one step away from zero when the magnitude of the remainder exceeds
+// the low s bits of the random integer u (ti_torch.py:33-46: prob <= rand_num -> 0, else sign(input)).
+__host__ __device__ inline int round_sto32(int x, int s, bool trunc, int u) {
+  const bool neg = x < 0;
+  const uint32_t m = neg ? 0u - static_cast<uint32_t>(x) : static_cast<uint32_t>(x);
+  const uint32_t mask = (1u << s) - 1u;
+  int q;
+  uint32_t rem;
+  if (trunc && neg) {
+    q = -static_cast<int>(m >> s);
+    rem = m & mask;
+  } else {
+    q = x >> s;
+    rem = static_cast<uint32_t>(x) & mask;
+  }
+  const int sg = (x > 0) - (x < 0);
+  const int r = q + (rem > (static_cast<uint32_t>(u) & mask) ? sg : 0);
+  return r > 127 ? 127 : (r < -127 ? -127 : r);
+}
+
 // Four rounded values -> four bytes (value e in byte e), two's complement low bytes.
 __device__ inline uint32_t pack4_i8(int r0, int r1, int r2, int r3) {
   // v_perm_b32: selector byte 0x00-0x03 picks a byte of the second operand, 0x04-0x07 of the first, 0x0c is zero

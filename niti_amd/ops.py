@@ -114,8 +114,16 @@ def conv_requant_sync_words(N, H, W, C, K, R=3, S=3, stride=1, padding=1, dgrad=
 
 def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epilogue, target_bits, method, div_mode,
                   bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask=None, forward_filter=None,
-                  shift_hint=False, pool_out=None, unpool=None):
-    _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask, forward_filter)
+                  shift_hint=False, pool_out=None, unpool=None, rand=None):
+    _chk_dev(x, w, sync, shift_out, exp_a, exp_b, exp_out, prepared_filter, relu_mask, forward_filter, rand)
+    if method == "sto":
+        # StoShift folded in: one random integer per output element (its low `shift` bits are used)
+        if rand is None or rand.dtype != torch.int32 or tuple(rand.shape) != tuple(out_shape) or not rand.is_contiguous():
+            raise RuntimeError("%s: stochastic rounding needs `rand`, a contiguous int32 tensor shaped like the output" % entry)
+        if unpool is not None:
+            raise L.NitiError("%s: stochastic rounding is not folded in together with the pooling's backward pass" % entry)
+    elif rand is not None:
+        raise RuntimeError("%s: `rand` is only used by method='sto'" % entry)
     if relu_mask is not None and (relu_mask.dtype != torch.int8 or tuple(relu_mask.shape) != tuple(out_shape)):
         raise RuntimeError("%s: relu_mask must be int8 and shaped like the output" % entry)
     if unpool is not None:      # (pooling input [N,2H,2W,C], tie rule): the result is written at that size
@@ -153,7 +161,10 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
     head = (_ptr(x), wptr, _ptr(y), N, H, W, C, K, R, S, stride, padding, flags, target_bits, L.ROUND[method],
             L.DIV[div_mode], L.BW[bw_mode], (L.RQ_RELU if relu else 0) | (L.RQ_SHIFT_HINT if shift_hint else 0))
     tail = (_ptr(sync), sync.numel(), _ptr(shift_out), _ptr(exp_a), _ptr(exp_b), _ptr(exp_out), _ptr(ws), nbytes, _stream(x))
-    if pool_out is not None:    # the entry with the pooled output takes it right after the output
+    if method == "sto":         # entries of their own: (pooled output,) random integers behind the output, no method argument
+        entry = "niti_conv2d_i8_dgrad_requant_sto" if dgrad else "niti_conv2d_i8_fprop_requant_sto"
+        head = head[:3] + ((_ptr(rand),) if dgrad else (_ptr(pool_out), _ptr(rand))) + head[3:14] + head[15:]
+    elif pool_out is not None:    # the entry with the pooled output takes it right after the output
         head = head[:3] + (_ptr(pool_out),) + head[3:]
     if unpool is not None:
         head = head[:3] + (_ptr(relu_mask), _ptr(unpool[0]), L.TIES[unpool[1]]) + head[3:]
@@ -166,9 +177,9 @@ def _conv_requant(entry, dgrad, x, w, out_shape, dims, stride, padding, f32_epil
 
 def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", relu=False, sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None, shift_hint=False, pool_out=None):
+                         prepared_filter=None, shift_hint=False, pool_out=None, rand=None):
     """conv2d_fprop + requant as one launch: x [N,H,W,C] int8, w [K,R,S,C] int8 -> ([N,P,Q,K] int8, device shift,
-    sync).  ``pool_out`` ([N,P/2,Q/2,K] int8): also receives the 2x2 / stride-2 maximum of the output.  sync[0] holds max|sum| afterwards, sync[1] != 0 flags a timed-out wait (invalid output).  ``sync``, if
+    sync).  method "sto" takes ``rand`` (int32, shaped like the output).  ``pool_out`` ([N,P/2,Q/2,K] int8): also receives the 2x2 / stride-2 maximum of the output.  sync[0] holds max|sum| afterwards, sync[1] != 0 flags a timed-out wait (invalid output).  ``sync``, if
     given, must hold conv_requant_sync_words(...) zeroed int32 words.  ``shift_hint``: ``shift_out`` holds a
     predicted shift on entry (e.g. this tensor's shift of the previous training step); a good prediction saves the
     kernel a second store pass, the results do not depend on it."""
@@ -185,7 +196,7 @@ def conv2d_fprop_requant(x, w, stride=1, padding=1, f32_epilogue=False, target_b
     entry = "niti_conv2d_i8_fprop_requant_pool" if pool_out is not None else "niti_conv2d_i8_fprop_requant"
     return _conv_requant(entry, False, x, w, (N, P, Q, K), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, relu, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter, shift_hint=shift_hint, pool_out=pool_out)
+                         prepared_filter, shift_hint=shift_hint, pool_out=pool_out, rand=rand)
 
 
 def conv2d_fprop_requant_static(x, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
@@ -223,8 +234,9 @@ def conv2d_fprop_requant_static(x, w, stride=1, padding=1, f32_epilogue=False, t
 
 def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target_bits=7, method="round", div_mode="floor",
                          bw_mode="int", sync=None, shift_out=None, exp_a=None, exp_b=None, exp_out=None,
-                         prepared_filter=None, relu_mask=None, forward_filter=None, shift_hint=False, unpool=None):
+                         prepared_filter=None, relu_mask=None, forward_filter=None, shift_hint=False, unpool=None, rand=None):
     """conv2d_dgrad + requant as one launch: err [N,P,Q,K] int8, w [K,R,S,C] int8 -> ([N,H,W,C] int8, shift, sync).
+    method "sto" takes ``rand`` (int32, shaped like the output; not together with ``unpool``).
     ``unpool`` = (pool_in [N,2H,2W,C] int8, "first" | "all") with ``relu_mask`` = the pooled map: the backward pass of
     the 2x2 / stride-2 max-pool in front of the layer is folded in and the result has pool_in's shape.
     ``relu_mask`` (int8 [N,H,W,C]): results whose mask element is not positive are stored as zero, after range
@@ -238,7 +250,7 @@ def conv2d_dgrad_requant(err, w, stride=1, padding=1, f32_epilogue=False, target
     W = Q - 2 * padding + S - 1
     return _conv_requant("niti_conv2d_i8_dgrad_requant", True, err, w, (N, H, W, C), (N, H, W, C, K, R, S), stride, padding,
                          f32_epilogue, target_bits, method, div_mode, bw_mode, False, sync, shift_out, exp_a, exp_b, exp_out,
-                         prepared_filter, relu_mask, forward_filter, shift_hint, unpool=unpool)
+                         prepared_filter, relu_mask, forward_filter, shift_hint, unpool=unpool, rand=rand)
 
 
 _scratch = {}

@@ -192,10 +192,12 @@ _fused_refused = set()       # (dgrad, input shape, filter shape, stride, paddin
 def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp_b, relu_mask=None, prepared_filter=None,
                         forward_filter=None, shift_state=None, pool_out=None, unpool=None):
     """conv (forward or data gradient) + act_calc / err_calc as one launch.  Returns (int8 tensor, shift,
-    exp_out) or None when the call needs the two-pass path: random rounding, a shape outside the
-    single-launch kernel, or more workgroups than the device holds at once."""
+    exp_out) or None when the call needs the two-pass path: a shape outside the single-launch kernel, more
+    workgroups than the device holds at once, or StoShift (ti_torch.py:33-46) on a 2 x 2 map or together with the
+    pooling's backward pass.  StoShift otherwise runs inside the launch on ``rand`` (int32, shaped like the output;
+    drawn here when the caller gives none)."""
     method = _method_name(fn)
-    if not FUSE_CONV_REQUANT or method == "sto" or rand is not None:
+    if not FUSE_CONV_REQUANT or (method != "sto" and rand is not None):
         return None
     key = (dgrad, tuple(x.shape), tuple(w.shape), stride, padding, unpool is not None)
     if key in _fused_refused:
@@ -206,6 +208,15 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
     if ops.conv_requant_sync_words(N, H, W, C, K, R, S, stride, padding, dgrad) == 0:
         _fused_refused.add(key)
         return None
+    if method == "sto":
+        if unpool is not None or H == 2:
+            return None
+        out_shape = (N, H, W, C) if dgrad else (N, (H + 2 * padding - R) // stride + 1, (W + 2 * padding - S) // stride + 1, K)
+        if rand is None:
+            rand = torch.randint(0, 2 ** 31 - 1, out_shape, dtype=torch.int32, device=x.device)
+        elif rand.dtype != torch.int32 or tuple(rand.shape) != out_shape:
+            return None
+        rand = rand.contiguous()
     from ._lib import NitiError
     exp_out = torch.empty(1, dtype=torch.int32, device=x.device)
     call = ops.conv2d_dgrad_requant if dgrad else ops.conv2d_fprop_requant
@@ -216,6 +227,8 @@ def _conv_requant_fused(dgrad, x, w, stride, padding, fn, rand, relu, exp_a, exp
         kw.update(unpool=unpool)
     if shift_state is not None:     # the tensor's shift of the previous step: the kernel's prediction for this one
         kw.update(shift_out=shift_state, shift_hint=True)
+    if method == "sto":
+        kw.update(rand=rand)
     try:
         y, shift, _ = call(x, w, stride, padding, f32_epilogue=F32_EPILOGUE, target_bits=BITWIDTH, method=method,
                            div_mode=DIV_MODE, bw_mode=BW_MODE, exp_a=exp_a, exp_b=exp_b, exp_out=exp_out, **kw)

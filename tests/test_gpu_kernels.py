@@ -204,6 +204,71 @@ def test_conv_fprop_requant(dev, case, method, div_mode):
             assert torch.equal(pooled.cpu(), po.maxpool_fwd(y.cpu()))
 
 
+STO_CASES = [(4, 8, 16, 16), (8, 8, 80, 144), (3, 16, 192, 272), (2, 32, 16, 64), (8, 32, 128, 128), (16, 4, 64, 128),
+             (256, 32, 16, 64),      # workgroups of 512 pixels
+             (264, 16, 16, 272)]     # two launches, the second one settling the shift
+
+
+@pytest.mark.parametrize("div_mode", ["floor", "trunc"])
+@pytest.mark.parametrize("case", STO_CASES)
+def test_conv_requant_sto(dev, case, div_mode):
+    """StoShift (ti_torch.py:33-46) inside the single-launch convolutions: same random integers, same bytes as the
+    oracle's act_calc / err_calc / grad_calc with method 'sto'; wide random integers count by their low `shift` bits;
+    a wrong prediction (second store pass with another shift) changes nothing."""
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    N, Q, C, K = case
+    _say("conv_requant_sto", case, div_mode)
+    g = torch.Generator().manual_seed(990 + N + C + K)
+    x, w = ri8(g, N, Q, Q, C), ri8(g, K, 3, 3, C)
+    acc = po.conv2d_fprop_i32(x, w, 1, 1)
+    for tgt, relu in ((7, False), (7, True), (4, False)):
+        s = max(po.RangeEstimate(acc) - tgt, 1)
+        u = torch.randint(0, 2 ** s, acc.shape, generator=g, dtype=torch.int32)
+        ref, sh_ref = po.act_calc(acc, 0, "sto", div_mode, u) if tgt == 7 else po.grad_calc(acc, tgt, "sto", div_mode, u)
+        wide = u + (torch.randint(0, 2 ** (30 - s), acc.shape, generator=g, dtype=torch.int32) << s)
+        for rand, hint in ((u, None), (wide, 0), (wide, sh_ref + 2), (u, max(sh_ref - 1, 0))):
+            kw = {}
+            if hint is not None:
+                kw = dict(shift_out=torch.tensor([hint], dtype=torch.int32, device=dev), shift_hint=True)
+            y, sh, sync = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), 1, 1, target_bits=tgt, method="sto", div_mode=div_mode,
+                                                   relu=relu, rand=rand.to(dev), **kw)
+            sync = sync.cpu()
+            assert int(sync[1]) == 0 and int(sync[0]) == po.absmax(acc) and int(sh.cpu()) == sh_ref
+            assert torch.equal(y.cpu(), ref.clamp(min=0) if relu else ref), (tgt, relu, hint)
+    # with the pooled output next to it
+    pooled = torch.empty((N, Q // 2, Q // 2, K), dtype=torch.int8, device=dev)
+    y2, _, _ = ops.conv2d_fprop_requant(x.to(dev), w.to(dev), 1, 1, target_bits=4, method="sto", div_mode=div_mode, rand=u.to(dev),
+                                        pool_out=pooled)
+    assert torch.equal(y2.cpu(), ref) and torch.equal(pooled.cpu(), po.maxpool_fwd(ref))
+    # data gradient (the error map has K channels, the result C), with the ReLU mask of the layer below
+    e = ri8(g, N, Q, Q, K)
+    dacc = po.conv2d_dgrad_i32(e, w, 1, 1, f32_epilogue=False)
+    s = max(po.RangeEstimate(dacc) - 7, 1)
+    u = torch.randint(0, 2 ** s, dacc.shape, generator=g, dtype=torch.int32)
+    dref, dsh = po.err_calc(dacc, "sto", div_mode, u)
+    mask = ri8(g, N, Q, Q, C)
+    fwd_copy = ops.conv_filter_prepare(w.to(dev), N, Q, Q)
+    for kw in (dict(), dict(forward_filter=fwd_copy), dict(relu_mask=mask.to(dev))):
+        d8, sh, sync = ops.conv2d_dgrad_requant(e.to(dev), w.to(dev), 1, 1, method="sto", div_mode=div_mode, rand=u.to(dev), **kw)
+        assert int(sync.cpu()[1]) == 0 and int(sh.cpu()) == dsh
+        assert torch.equal(d8.cpu(), torch.where(mask > 0, dref, torch.zeros_like(dref)) if "relu_mask" in kw else dref)
+
+
+def test_conv_requant_sto_refusals(dev):
+    from niti_amd import ops
+    from niti_amd._lib import NitiError
+    g = torch.Generator().manual_seed(991)
+    x, w = ri8(g, 32, 2, 2, 32).to(dev), ri8(g, 32, 3, 3, 32).to(dev)
+    u = torch.zeros((32, 2, 2, 32), dtype=torch.int32, device=dev)
+    with pytest.raises(NitiError):       # 2 x 2 maps keep the two-pass path for StoShift
+        ops.conv2d_fprop_requant(x, w, method="sto", rand=u)
+    with pytest.raises(RuntimeError):    # no random integers
+        ops.conv2d_fprop_requant(x, w, method="sto")
+    with pytest.raises(RuntimeError):    # random integers of the wrong shape
+        ops.conv2d_fprop_requant(x, w, method="sto", rand=u[:1])
+
+
 def test_conv_fprop_requant_wraps_when_no_shift(dev):
     """Sums that already fit 7 bits (+ the 128 -> -128 wrap of the reference's int32 -> int8 cast)."""
     from niti_amd import ops

@@ -68,6 +68,51 @@ def test_conv_layer_fwd_bwd(tt, div_mode, first):
         assert torch.equal(r[0].cpu(), ro[0]) and _ei(r[1]) == ro[1]
 
 
+def test_conv_layer_sto_runs_in_the_single_launch_kernels(tt):
+    """ACT / ERROR_ROUND_METHOD = StoShift (selectable in the reference, ti_torch.py:460-463): the layer hands the random
+    integers to the convolution launches instead of falling back to int32 results + a requantisation pass."""
+    from oracle import niti_model_oracle as mo
+    from oracle import niti_oracle as po
+    from niti_amd import ops
+    dev = torch.device("cuda:0")
+    g = torch.Generator().manual_seed(1050)
+    N, H, C, K = 8, 16, 32, 64
+    _say("conv layer, StoShift")
+    tt.ACT_ROUND_METHOD = tt.ERROR_ROUND_METHOD = tt.StoShift
+    w, x, err = ri8(g, K, 3, 3, C), ri8(g, N, H, H, C), laplace_i8(g, (N, H, H, K))
+    rf = torch.randint(0, 2 ** 20, (N, H, H, K), generator=g, dtype=torch.int32)
+    rb = torch.randint(0, 2 ** 20, (N, H, H, C), generator=g, dtype=torch.int32)
+    cfg = mo.Cfg(act="sto", err="sto")
+    o = mo.OConv2d(w, -9)
+    # the oracle's StoShift compares with the integer as it is: hand it the low `shift` bits the kernels use
+    sf = max(po.RangeEstimate(po.conv2d_int8(x, w)) - 7, 1)
+    sb = max(po.RangeEstimate(po.conv2d_dgrad_i32(err, w)) - 7, 1)
+    yo, eo = o.forward((x, -3), cfg, rf & (2 ** sf - 1))
+    ro = o.backward((err, -5), cfg, rb & (2 ** sb - 1))
+    layer = tt.TiConv2d(C, K)
+    layer.weight, layer.weight_exp = w.to(dev), torch.tensor(-9.0)
+    calls = []
+    real = ops.requant
+    ops.requant = lambda *a, **k: calls.append(1) or real(*a, **k)
+    try:
+        y, e = layer.forward((x.to(dev), -3), rf.to(dev))
+        r = layer.backward((err.to(dev), -5), rb.to(dev))
+    finally:
+        ops.requant = real
+    assert not calls
+    assert torch.equal(y.cpu(), yo) and _ei(e) == eo
+    assert torch.equal(r[0].cpu(), ro[0]) and _ei(r[1]) == ro[1]
+    assert torch.equal(layer.weight.cpu(), o.weight) and _ei(layer.grad_exp) == o.grad_exp
+    # random integers drawn by the layer itself: between the results of the two extreme draws
+    y2, _ = layer.forward((x.to(dev), -3))
+    acc2 = po.conv2d_int8(x, o.weight)
+    s2 = max(po.RangeEstimate(acc2) - 7, 1)
+    a, _ = po.act_calc(acc2, 0, "sto", "floor", torch.zeros_like(acc2))
+    b, _ = po.act_calc(acc2, 0, "sto", "floor", torch.full_like(acc2, 2 ** s2 - 1))
+    y2 = y2.cpu().to(torch.int16)
+    assert bool(((y2 >= torch.minimum(a, b).to(torch.int16)) & (y2 <= torch.maximum(a, b).to(torch.int16))).all())
+
+
 def test_conv_layer_on_a_grid_larger_than_the_device(tt):
     """A layer whose convolutions have more workgroups than the device holds at once (136 images of 32 x 32, 80 -> 144
     channels: 1088 and 544 tiles): forward and data gradient run as two launches that do not wait.  Two training
