@@ -214,19 +214,23 @@ def fit(model, train_loader, test_loader, epochs, save_path=None, save_all=False
 
 
 class TensorLoader:
-    """Minimal stand-in for a ``DataLoader`` over in-memory tensors: fixed-size batches (the last ragged one is
-    dropped: the convolution kernels own whole tiles of a batch), reshuffled every pass when ``shuffle``."""
+    """Minimal stand-in for a ``DataLoader`` over in-memory tensors, reshuffled every pass when ``shuffle``.  Like the
+    reference's loaders (data.py:42-46: no ``drop_last``) it ends a pass with the smaller batch that is left over -
+    CIFAR-10 at batch 256 ends with 80 images; the layers run such a batch through whichever kernels cover its
+    shape (the single-launch ones need whole tiles of 256 pixels) and the reference's own odd-batch case
+    (ti_torch.py:419-428) needs no special path here.  ``drop_last=True`` keeps only whole batches."""
 
-    def __init__(self, x, y, batch_size, shuffle=False, seed=0):
-        self.x, self.y, self.batch_size, self.shuffle = x, y, batch_size, shuffle
+    def __init__(self, x, y, batch_size, shuffle=False, seed=0, drop_last=False):
+        self.x, self.y, self.batch_size, self.shuffle, self.drop_last = x, y, batch_size, shuffle, drop_last
         self.gen = torch.Generator().manual_seed(seed)
 
     def __len__(self):
-        return self.x.shape[0] // self.batch_size
+        n = self.x.shape[0]
+        return n // self.batch_size if self.drop_last else (n + self.batch_size - 1) // self.batch_size
 
     def __iter__(self):
-        n = len(self) * self.batch_size
-        order = torch.randperm(self.x.shape[0], generator=self.gen)[:n] if self.shuffle else torch.arange(n)
+        n = self.x.shape[0]
+        order = torch.randperm(n, generator=self.gen) if self.shuffle else torch.arange(n)
         for b in range(len(self)):
             idx = order[b * self.batch_size:(b + 1) * self.batch_size]
             yield self.x[idx], self.y[idx]

@@ -238,6 +238,10 @@ def _build_pair(tt, cfg_list, widths_in, N, seed, dropout, image=32):
     ("vgg13", [64, 64, 'M', 128, 128, 'M', 256, 256, 'M', 512, 512, 'M', 512, 512, 'M'], 8),
     # cifar_cfg[8] and cifar_cfg[9] of the reference (ti_vgg.py:12-13): stages of three convolutions, i.e. convolutions
     # whose ReLU is followed by another convolution instead of a pooling
+    # batches that are not whole tiles of the single-launch kernels: the last batch of a pass over a data set (80 =
+    # 50000 mod 256, the reference trains on it: data.py:42-46) and an odd one (ti_torch.py:419-428)
+    ("vgg7-narrow-batch80", [16, 16, 'M', 32, 32, 'M', 512, 512, 'M'], 80),
+    ("vgg7-narrow-batch37", [16, 16, 'M', 32, 32, 'M', 512, 512, 'M'], 37),
     ("vgg8", [128, 128, 128, 'M', 256, 256, 'M', 512, 512, 'M'], 8),
     ("vgg9", [128, 128, 128, 'M', 256, 256, 256, 'M', 512, 512, 'M'], 8),
 ])
@@ -413,6 +417,52 @@ def test_epoch_driver_learns_and_checkpoints(tt, tmp_path, use_graph):
     out_a, exp_a = model(x.to("cuda:0"))
     out_b, exp_b = fresh(x.to("cuda:0"))
     assert torch.equal(out_a, out_b) and _ei(exp_a) == _ei(exp_b)
+
+
+@pytest.mark.parametrize("use_graph", [False, True])
+def test_epoch_driver_trains_on_the_trailing_batch(tt, use_graph):
+    """A pass over 128 + 80 images: the smaller last batch is a training step like any other (the reference's loaders
+    do not drop it, data.py:42-46).  The pass must see all 208 samples, and its weights must equal those of the same
+    two batches stepped by hand."""
+    from niti_amd import train
+    from niti_amd.ti_vgg import TiVGG_cifar
+    _say("epoch_driver trailing batch", use_graph)
+    g = torch.Generator().manual_seed(77)
+    x = torch.randn(208, 3, 32, 32, generator=g)
+    y = torch.randint(0, 10, (208,), generator=g)
+    torch.manual_seed(11)
+    model = TiVGG_cifar(depth=7)
+    start = {k: v.clone() for k, v in model.state_dict().items()}
+    loader = train.TensorLoader(x, y, 128)
+    assert len(loader) == 2
+    seen = []
+    orig = train._add_metrics
+    train._add_metrics = lambda out, e, t, sums: seen.append(int(t.numel())) or orig(out, e, t, sums)
+    try:
+        torch.manual_seed(12)      # the dropout masks and the loss gradient's random integers come from torch's device generator
+        torch.cuda.manual_seed(12)
+        train.run_epoch(loader, model, True, use_graph=use_graph)
+    finally:
+        train._add_metrics = orig
+    assert seen == [128, 80]
+    twin = TiVGG_cifar(depth=7)
+    twin.load_state_dict(start)
+    tt.TRAINING = True
+    torch.manual_seed(12)
+    torch.cuda.manual_seed(12)
+    dev = torch.device("cuda:0")
+    before = {k: v.clone() for k, v in start.items()}    # load_state_dict adopts the tensors it is given
+    for lo, hi in ((0, 128), (128, 208)):
+        tgt = y[lo:hi].to(dev)
+        twin(x[lo:hi].to(dev), tgt)
+        twin.backward(tgt)
+    changed = 0
+    for (k, a), b in zip(model.state_dict().items(), twin.state_dict().values()):
+        assert torch.equal(a, b), k
+        changed += int(not torch.equal(a.cpu(), before[k].cpu()))
+    assert changed > 0
+    from niti_amd import ops
+    assert not ops.sync_timeouts(dev)
 
 
 def test_epoch_driver_command_line(tt, tmp_path, monkeypatch):

@@ -64,6 +64,11 @@ def test_npz_loader(tmp_path):
     np.savez(path, x_train=rng.integers(0, 256, (10, 32, 32, 3), dtype=np.uint8), y_train=rng.integers(0, 10, 10),
              x_test=rng.integers(0, 256, (4, 32, 32, 3), dtype=np.uint8), y_test=rng.integers(0, 10, 4))
     tr, te = train.npz_loaders(path, 4)
-    assert len(tr) == 2 and len(te) == 1
+    # data.py:42-46 builds its loaders without drop_last: the two images left over are the last batch
+    assert len(tr) == 3 and len(te) == 1
+    assert [x.shape[0] for x, _ in tr] == [4, 4, 2]
+    assert sorted(int(v) for _, y in tr for v in y) == sorted(int(v) for v in np.load(path)['y_train'])
+    whole = train.TensorLoader(tr.x, tr.y, 4, drop_last=True)
+    assert len(whole) == 2 and [x.shape[0] for x, _ in whole] == [4, 4]
     x, y = next(iter(te))
     assert x.shape == (4, 3, 32, 32) and float(x.min()) >= -1.0 and float(x.max()) <= 1.0 and y.dtype == torch.int64
