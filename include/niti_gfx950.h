@@ -139,7 +139,7 @@ int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t* dx, int N,
  *
  * sync: niti_conv2d_i8_requant_sync_words(...) uint32 words that are ZERO on entry (niti_fill_u32).  On return
  * word 0 holds max |sum| over the tensor; word 1 is non-zero if the wait for the other workgroups ran into its
- * time limit (10 s, or NITI_SYNC_TIMEOUT_MS from the environment), in which case the output is invalid - this
+ * time limit (2 s, or NITI_SYNC_TIMEOUT_MS from the environment), in which case the output is invalid - this
  * can only happen when other work keeps part of the device busy that long.  Launches that share a sync buffer
  * must not overlap.
  * flags: NITI_EPI_F32_ROUNDTRIP, NITI_CONV_FILTER_PREPARED (w is a copy made by niti_conv2d_i8_filter_prepare;
@@ -484,6 +484,9 @@ int niti_head_i8_backward(const int8_t* err, const int8_t* act, const int8_t* dr
 int niti_group_conv_i8_f32(const int8_t* x, const int8_t* w, float* y, int N, int H, int W, int C, int K, int R,
                            int S, int Cg, int stride, int pad, int dilation, int groups, void* stream);
 
+/* ==================================================================================================================
+ * MEASUREMENT ONLY - not part of the boundary a reference checkout binds to; nothing in the layers calls it.
+ * ================================================================================================================== */
 /*
  * Measurement aid, no counterpart in the reference: a register-resident int8 MFMA loop (v_mfma_i32_32x32x32_i8, no LDS
  * and no memory traffic inside the loop) over operand fragments read once from `operands` (operand_bytes >= 128,

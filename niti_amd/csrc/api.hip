@@ -5,6 +5,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "common.h"
 
 namespace niti {
@@ -86,12 +88,11 @@ static int check_flags(const char* who, unsigned flags, unsigned allowed) {
 }
 
 static bool halo_off() {
-  static int v = -1;
-  if (v < 0) {
+  static const bool off = [] {   // read once (initialisation of a function-local static is thread-safe)
     const char* e = getenv("NITI_NO_HALO");
-    v = (e && e[0] == '1') ? 1 : 0;
-  }
-  return v == 1;
+    return e != nullptr && e[0] == '1';
+  }();
+  return off;
 }
 
 // which filter copy a convolution of this shape uses: 0 none (w as stored), 1 flipped/transposed
@@ -227,15 +228,18 @@ extern "C" int niti_conv2d_i8_dgrad(const int8_t* err, const int8_t* w, int32_t*
 }
 
 // ---- convolution + requantisation in one launch -------------------------------------------------------
-// wall-clock ticks (100 MHz) a grid-wide wait may last; NITI_SYNC_TIMEOUT_MS overrides the 10 s default
+// wall-clock ticks (100 MHz) a grid-wide wait may last; NITI_SYNC_TIMEOUT_MS overrides the 2 s default (a healthy
+// wait lasts microseconds; the limit only matters when other work holds part of the device).  Fractions are allowed
+// (0.00001 ms is one tick); 0 makes every wait give up after its first look, which tests of that path use.
 long long niti::sync_spin_limit() {
-  static long long spin_limit = -1;
-  if (spin_limit < 0) {
-    const char* e = getenv("NITI_SYNC_TIMEOUT_MS");   // fractions allowed: 0.00001 ms is one tick
-    const double ms = e != nullptr ? atof(e) : 10000.0;
+  static std::once_flag once;
+  static long long spin_limit = 0;
+  std::call_once(once, [] {
+    const char* e = getenv("NITI_SYNC_TIMEOUT_MS");
+    const double ms = e != nullptr ? atof(e) : 2000.0;
     const double ticks = ms * 100000.0;
-    spin_limit = ticks >= 1.0 ? static_cast<long long>(ticks) : 1LL;
-  }
+    spin_limit = ticks >= 1.0 ? static_cast<long long>(ticks) : (ms > 0.0 ? 1LL : 0LL);
+  });
   return spin_limit;
 }
 

@@ -125,9 +125,12 @@ inline size_t slot_words(int blocks) { return static_cast<size_t>((blocks + 15) 
 // Called by a whole wavefront: waits until all nb slots are filled and returns the largest value.  512 slots at a
 // time, eight per lane with the loads in flight together (one trip to memory per look); a lane reads a slot again
 // only while it is still empty, so the reads of the waiting workgroups die down as the slots fill.  Gives up after
-// spin_limit ticks of the 100 MHz clock: *timed_out (the launch's own flag) and *sticky (the device-wide word that
-// niti_sync_timeouts reads, may be null) are set to 1 and the largest value seen so far is returned.
-__device__ inline uint32_t wait_slots(uint32_t* slots, int nb, long long spin_limit, uint32_t* timed_out, uint32_t* sticky) {
+// spin_limit ticks of the 100 MHz clock: `code` is or-ed into *timed_out (the launch's own flag: 1 = a wait for the
+// tensor-wide range, 2 = the one-launch weight gradient's wait for the partial sums), *sticky (the device-wide word
+// that niti_sync_timeouts reads, may be null) is set to 1 and the largest value seen so far is returned.  A limit of
+// zero gives up after the first look whatever it saw (tests of this path: every waiting wavefront then takes it).
+__device__ inline uint32_t wait_slots(uint32_t* slots, int nb, long long spin_limit, uint32_t* timed_out, uint32_t* sticky,
+                                      uint32_t code = 1u) {
   constexpr int kLook = 8;
   const int lane = threadIdx.x & 63;
   const long long t0 = wall_clock64();
@@ -148,10 +151,10 @@ __device__ inline uint32_t wait_slots(uint32_t* slots, int nb, long long spin_li
         v[u] = t[u];
         ok = ok && v[u] != 0u;
       }
-      if (__all(ok)) break;
-      if (wall_clock64() - t0 > spin_limit) {
+      if (__all(ok) && spin_limit > 0) break;
+      if (spin_limit <= 0 || wall_clock64() - t0 > spin_limit) {
         if (lane == 0) {
-          __hip_atomic_store(timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_or(timed_out, code, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           if (sticky != nullptr) __hip_atomic_store(sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         gave_up = true;

@@ -198,13 +198,12 @@ __global__ __launch_bounds__(256, 2) void conv_igemm_i8_kernel(const ConvArgs a)
 }  // namespace
 
 static int tile_override_from_env() {
-  static int v = -1;
-  if (v < 0) {
+  static const int tile = [] {   // read once (initialisation of a function-local static is thread-safe)
     const char* e = getenv("NITI_CONV_TILE");
-    v = e ? atoi(e) : 0;
-    if (v < 0 || v > 6) v = 0;
-  }
-  return v;
+    const int v = e != nullptr ? atoi(e) : 0;
+    return (v < 0 || v > 6) ? 0 : v;
+  }();
+  return tile;
 }
 
 int launch_conv_igemm(const ConvProblem& p, hipStream_t stream) {

@@ -471,10 +471,10 @@ __device__ inline void wait_slot_pairs(uint32_t* slots, int nb, long long spin_l
     for (;;) {
       if (v == 0ULL)
         v = __hip_atomic_load(reinterpret_cast<unsigned long long*>(slot_word(slots, base + lane)), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (__all(v != 0ULL)) break;
-      if (wall_clock64() - t0 > spin_limit) {
+      if (__all(v != 0ULL) && spin_limit > 0) break;
+      if (spin_limit <= 0 || wall_clock64() - t0 > spin_limit) {   // a limit of zero: give up after the first look (tests)
         if (lane == 0) {
-          __hip_atomic_store(timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          __hip_atomic_fetch_or(timed_out, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           if (sticky != nullptr) __hip_atomic_store(sticky, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         gave_up = true;

@@ -39,9 +39,13 @@ __device__ inline long long wave_sum_i64(long long v) {
 __global__ __launch_bounds__(256) void loss_grad_kernel(const LossArgs a) {
   const int lane = threadIdx.x & 63;
   const int row = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (row >= a.n) return;
+  // Every wavefront reads the generator state, then the workgroup reports in: the last workgroup to do so starts the
+  // next step, so no wavefront of this launch may still have its read ahead of it at that point.
   RngDraw draw{};
   if (a.rand == nullptr) draw = rng_read(a.rng);
+  __syncthreads();
+  if (a.rand == nullptr && threadIdx.x == 0) rng_arrive(a.rng, gridDim.x, draw);
+  if (row >= a.n) return;
   const int8_t* v = a.out + static_cast<long long>(row) * a.classes;
   const int e = *a.out_exp;
   const bool big = e > -7;
@@ -83,7 +87,6 @@ __global__ __launch_bounds__(256) void loss_grad_kernel(const LossArgs a) {
     const int u = a.rand != nullptr ? a.rand[idx] & 15 : static_cast<int>(rng_word(draw, kRngStreamLoss, static_cast<uint32_t>(idx)) & 15u);
     a.grad[idx] = static_cast<int8_t>(round_one<NITI_ROUND_STOCHASTIC>(x, 4, trunc, u));
   }
-  if (a.rand == nullptr && threadIdx.x == 0) rng_arrive(a.rng, gridDim.x, draw);   // the first row of a workgroup always exists
 }
 
 }  // namespace

@@ -932,7 +932,7 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
       __hip_atomic_store(slot_word(f.arrive, block), wide ? 2u : 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     if (wave == 0) {
-      const uint32_t seen = wait_slots(f.arrive, nblocks, f.spin_limit, &f.sync[1], f.sticky);
+      const uint32_t seen = wait_slots(f.arrive, nblocks, f.spin_limit, &f.sync[1], f.sticky, 2u);
       if (lane == 0) wgm[8] = seen;
     }
     __syncthreads();

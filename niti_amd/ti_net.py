@@ -71,9 +71,10 @@ class TiNet(Module):
     def quantize_input(x):
         """TiFloatToInt8 + NCHW -> NHWC (ti_net.py:18-19): (int8 NHWC batch, exponent).  A contiguous float32 batch on
         the GPU takes the library's two launches (channels come zero-padded to 16, which the first convolution
-        would do next anyway); anything else the reference's tensor operations."""
+        would do next anyway); anything else - and BW_MODE "f32", whose range exponent is the reference's float32
+        ``ceil(log2(r))`` rather than the exact one - the reference's tensor operations."""
         x = x.to(ti_torch.GPU)
-        if x.dtype == torch.float32 and x.dim() == 4 and x.is_contiguous() and x.is_cuda:
+        if x.dtype == torch.float32 and x.dim() == 4 and x.is_contiguous() and x.is_cuda and ti_torch.BW_MODE == "int":
             return ops.quantize_input(x, ti_torch.BITWIDTH)
         x_data, x_exp = ti_torch.TiFloatToInt8(x)
         return x_data.permute(0, 2, 3, 1).contiguous(), x_exp

@@ -275,9 +275,13 @@ def conv2d_weight_int8(input, weight_size, grad_output, stride=1, padding=0, dil
 # quantisers / initialisers (ti_torch.py:77-99, 334-364)
 # ------------------------------------------------------------------------------------------
 def _ceil_log2(r):
-    """``torch.ceil(torch.log2(r))`` of ti_torch.py:336,348 as exact arithmetic on the float's exponent and mantissa
-    (r = m * 2^e, 0.5 <= m < 1: e - 1 for a power of two, e otherwise), so that every device gives the same integer;
-    a float32 log2 rounds k + log2(1 + d) back to k for the first values above 2^k, k >= 4.  0-d float tensor."""
+    """``torch.ceil(torch.log2(r))`` of ti_torch.py:336,348.  BW_MODE "int" (default): exact arithmetic on the float's
+    exponent and mantissa (r = m * 2^e, 0.5 <= m < 1: e - 1 for a power of two, e otherwise), so that every device
+    gives the same integer.  BW_MODE "f32": the reference's own float32 expression, whose log2 rounds
+    k + log2(1 + d) back to k for the first float32 values above 2^k, k >= 4 (nextafter(16) gives 4 where the exact
+    value is 5: the exponent is then one lower and the largest value saturates at 127).  0-d float tensor."""
+    if BW_MODE == "f32":
+        return torch.ceil(torch.log2(r.float()))
     m, e = torch.frexp(r.float())
     return torch.where(m == 0.5, e - 1, e).to(torch.float32)
 

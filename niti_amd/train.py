@@ -106,8 +106,8 @@ class StepGraph:
             gc.collect()
             gc.disable()
             try:
-                g = torch.cuda.CUDAGraph()
                 try:
+                    g = torch.cuda.CUDAGraph()
                     with torch.cuda.graph(g):
                         self._step()
                 finally:
@@ -151,6 +151,10 @@ def run_epoch(data_loader, model, training, log_interval=0, epoch=0, use_graph=F
         if training and log_interval and i % log_interval == 0:
             s = (sums / count).tolist()
             logging.info('[%d][%3d] loss %.3f @1 %.3f', epoch, i, s[0], s[1])
+        # A shared device makes every grid-wide wait run into its limit and every step round with wrong shifts: find out
+        # after the first steps and whenever the host reads the device anyway, not at the end of a pass that looked hung
+        if i in (0, 3) or (training and log_interval and i % log_interval == 0):
+            check_waits(dev)
     if count == 0:
         return 0.0, 0.0, 0.0
     loss_avg, top1, top5 = (sums / count).tolist()

@@ -72,3 +72,21 @@ def test_npz_loader(tmp_path):
     assert len(whole) == 2 and [x.shape[0] for x, _ in whole] == [4, 4]
     x, y = next(iter(te))
     assert x.shape == (4, 3, 32, 32) and float(x.min()) >= -1.0 and float(x.max()) <= 1.0 and y.dtype == torch.int64
+
+
+def test_quantisers_follow_bw_mode():
+    """BW_MODE "f32" makes TiFloatToInt8 / weight_quant take the range exponent from the reference's own float32
+    expression (ti_torch.py:336,348); "int" (default) from the float's exponent and mantissa.  They differ for the
+    first float32 values above 2^k, k >= 4, when log2 rounds to k: with torch's CPU log2, nextafter(16) gives 4."""
+    import numpy as np
+    r = torch.tensor(float(np.nextafter(np.float32(16.0), np.float32(32.0))))
+    old = ti_torch.BW_MODE
+    try:
+        ti_torch.BW_MODE = "int"
+        assert float(ti_torch._ceil_log2(r)) == 5.0
+        assert float(ti_torch._ceil_log2(torch.tensor(16.0))) == 4.0 and float(ti_torch._ceil_log2(torch.tensor(0.75))) == 0.0
+        ti_torch.BW_MODE = "f32"
+        assert float(ti_torch._ceil_log2(r)) == float(torch.ceil(torch.log2(r)))
+        assert float(ti_torch._ceil_log2(torch.tensor(16.0))) == 4.0 and float(ti_torch._ceil_log2(torch.tensor(17.0))) == 5.0
+    finally:
+        ti_torch.BW_MODE = old
