@@ -79,11 +79,7 @@ class ConvTriple:
             n = ops.wgrad_update_sync_words(BATCH, L["hw"], L["hw"], L["x16"].shape[3], L["k"])
             L["sync_w"] = (off, n)
             off += n
-        # one buffer, hence one fill per step: the sync words, then (256-byte aligned) the ranges of the two-pass paths
         sync_words = (max(off, 1) + 63) // 64 * 64
-        self.zeroed = torch.zeros(sync_words + 3 * len(LAYERS), dtype=torch.int32, device=dev)
-        self.sync = self.zeroed[:sync_words]
-        self.absmax = self.zeroed[sync_words:]
         self.ws = ops.scratch(256 << 20, dev)    # shared by all weight-gradient launches
         # Every step updates the weights (and their kernel-ready copies) in place.  So that each timed step multiplies
         # the operands the configuration names - weights uniform in [-127, 127] from the seed, not the saturated values
@@ -95,9 +91,15 @@ class ConvTriple:
             L["w16"] = F.pad(L["w"], (0, 16 - c % 16)).contiguous() if c % 16 else L["w"]
             L["wp"] = ops.conv_filter_prepare(L["w16"], BATCH, hw, hw)
             segs += [(L, "w"), (L, "wp")] if L["wp"] is not None else [(L, "w")]
-        total = sum((L[key].numel() + 255) // 256 * 256 for L, key in segs)
-        self.wflat = torch.empty(total, dtype=torch.int8, device=dev)
-        o = 0
+        # ... and in front of them the words that every step must find zeroed (the sync words of all launches, then the
+        # ranges of the two-pass paths): zeros in the pristine copy, so the one copy is also the step's only fill
+        zero_bytes = ((sync_words + 3 * len(LAYERS)) * 4 + 255) // 256 * 256
+        total = zero_bytes + sum((L[key].numel() + 255) // 256 * 256 for L, key in segs)
+        self.wflat = torch.zeros(total, dtype=torch.int8, device=dev)
+        self.zeroed = self.wflat[:zero_bytes].view(torch.int32)
+        self.sync = self.zeroed[:sync_words]
+        self.absmax = self.zeroed[sync_words:sync_words + 3 * len(LAYERS)]
+        o = zero_bytes
         for L, key in segs:
             t = L[key]
             view = self.wflat[o:o + t.numel()].view(t.shape)
@@ -117,9 +119,10 @@ class ConvTriple:
     def step(self, record=False):
         torch, ops = self.torch, self.ops
         import torch.nn.functional as F
-        self.zeroed.zero_()
         if self.restore_weights:
-            self.wflat.copy_(self.wpristine)
+            self.wflat.copy_(self.wpristine)      # weights, filter copies and the zeroed words in one device copy
+        else:
+            self.zeroed.zero_()
         for i, L in enumerate(self.layers):
             c, k, hw = L["c"], L["k"], L["hw"]
             am = self.absmax[3 * i: 3 * i + 3]
@@ -704,7 +707,8 @@ def main():
            "pct_int8_mfma_peak": round(100.0 * tops / INT8_MFMA_PEAK_TOPS, 2),
            "roofline": roofline, "roofline_wgrad": roofline_wgrad, "per_layer": per_layer}
     out["weights"] = {"state": "every step starts from the seeded uniform int8 weights: all weights and kernel-ready filter copies "
-                               "are restored from a pristine copy by one device copy inside the timed step",
+                               "are restored from a pristine copy by one device copy inside the timed step, which also zeroes the sync words (the "
+                               "step's only fill)",
                       "restored_bytes_per_step": wl.restore_bytes}
     if not args.no_drift_ab:
         # the same step without the restore: the weights drift (the same gradient every step drives them to +-127)
