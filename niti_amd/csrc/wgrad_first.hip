@@ -82,6 +82,20 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
 #pragma unroll
   for (int h = 0; h < 2; ++h) xv[h] = *reinterpret_cast<const uint32_t*>(a.act + (static_cast<long long>(n) * 1024 + tid + 512 * h) * 16);
 
+  // The weights this lane would update if its workgroup turns out to be the last one: requested now by every workgroup
+  // (3 456 bytes each), so that the finishing part does not start with a trip to memory for them.  Nobody writes them
+  // before all workgroups have reported in.
+  constexpr int PER = (K * 27 + 511) / 512;
+  int wold[PER];
+  {
+    const int total_w = K * 9 * a.Cw;
+#pragma unroll
+    for (int i = 0; i < PER; ++i) {
+      const int idx = i * 512 + tid;
+      wold[i] = idx < total_w ? static_cast<int>(a.w[idx]) : 0;
+    }
+  }
+
   // ---- error tile staging: an instruction fills PPI pixels x K bytes; pieces swizzled by the pixel (bank spread)
   const __amdgpu_buffer_rsrc_t rerr = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.err), 0, a.err_bytes, 0x00020000);
   auto issue = [&](int piece8, int buf) {
@@ -192,7 +206,6 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
   if (flag == 0u) return;
 
   // ---- the last workgroup holds the whole gradient: range, rounding, update
-  constexpr int PER = (K * 27 + 511) / 512;
   int s[PER];
   uint32_t lmax = 0;
   const int total = K * ncols;
@@ -231,7 +244,7 @@ __global__ __launch_bounds__(512) void wgrad_first_kernel(const WfArgs a) {
     int r;
     if (shift >= 1) r = psto ? round_one32<NITI_ROUND_PSEUDO_STOCHASTIC>(s[i], shift, trunc) : round_one32<NITI_ROUND_NEAREST>(s[i], shift, trunc);
     else r = wrap_to_i8(s[i]);
-    const int wn = clip127(static_cast<int>(a.w[idx]) - r);   // w is [K][9][Cw]: element idx
+    const int wn = clip127(wold[i] - r);   // w is [K][9][Cw]: element idx
     a.w[idx] = static_cast<int8_t>(wn);
     if (a.g8 != nullptr) a.g8[idx] = static_cast<int8_t>(r);
     if (a.wprep != nullptr) {
