@@ -516,7 +516,10 @@ def train_step_objects(dev, steps, warmup, graph=True, unroll=1):
         try:
             ips, ms, mode = train_step_rate(dev, steps, warmup, depth, batch, graph, unroll)
             out[name] = {"workload": workload, "images_per_s": round(ips, 1), "ms_per_step": round(ms, 3), "launch_mode": mode,
-                         "steps_per_graph": unroll if mode == "graph" else None}
+                         "steps_per_graph": unroll if mode == "graph" else None,
+                         "weights_state": "updated in place by every step, as in training; on the one repeated synthetic batch they "
+                                          "drift towards +-127, which the conv-triple A/B (`weights`) shows to run about 7 % slower "
+                                          "than seeded uniform weights"}
         except Exception as e:  # the headline line must still be printed
             out[name] = {"error": str(e)[:200]}
     for name, depth, ref_s in TRAIN_STEPS_B256:
