@@ -622,7 +622,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
           const v4i v = *reinterpret_cast<const v4i*>(patch + (t * 8 + rrow) * ROWB + rcol * 16);
           const int m = mrow + t * 8;
           const int off = (m < total_pix && ch < a.K) ? (m * a.K + ch) * 4 : kOob;
-          __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 0);
+          __builtin_amdgcn_raw_buffer_store_b128(v, ry, off, 0, 2);
         }
       }
     }
