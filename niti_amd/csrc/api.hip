@@ -306,7 +306,7 @@ static int conv_requant(const char* who, int dgrad, const int8_t* x, const int8_
   if (!aligned16(x) || !aligned16(w) || !aligned16(y8)) return fail(NITI_ERR_INVALID_ARG, "%s: pointers must be 16-byte aligned", who);
   if (target_bits < 1 || target_bits > 7) return fail(NITI_ERR_INVALID_ARG, "%s: target_bits=%d outside 1..7", who, target_bits);
   if (method != NITI_ROUND_NEAREST && method != NITI_ROUND_PSEUDO_STOCHASTIC && !(method == NITI_ROUND_STOCHASTIC && rand != nullptr))
-    return fail(NITI_ERR_UNSUPPORTED, "%s: rounding method %d needs random input; use the _sto entry point or the two-pass path", who, method);
+    return fail(NITI_ERR_UNSUPPORTED, "%s: rounding method %d needs random integers (the _sto entry points take them; or use the two-pass path)", who, method);
   if (rand != nullptr && !aligned16(rand)) return fail(NITI_ERR_INVALID_ARG, "%s: rand must be 16-byte aligned", who);
   if (div_mode != NITI_DIV_FLOOR && div_mode != NITI_DIV_TRUNC) return fail(NITI_ERR_INVALID_ARG, "%s: div_mode=%d", who, div_mode);
   if (bw_mode != NITI_BW_INT && bw_mode != NITI_BW_F32) return fail(NITI_ERR_INVALID_ARG, "%s: bw_mode=%d", who, bw_mode);
@@ -383,10 +383,6 @@ extern "C" int niti_conv2d_i8_fprop_requant_sto(const int8_t* x, const int8_t* w
                                                 int target_bits, int div_mode, int bw_mode, unsigned rq_flags, uint32_t* sync,
                                                 size_t sync_words, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b,
                                                 int32_t* exp_out, void* workspace, size_t workspace_bytes, void* stream) {
-  if (rand == nullptr) {
-    clear_error();
-    return fail(NITI_ERR_INVALID_ARG, "conv_fprop_requant_sto: null pointer");
-  }
   return conv_requant("conv_fprop_requant_sto", 0, x, w, y8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, NITI_ROUND_STOCHASTIC,
                       div_mode, bw_mode, rq_flags, nullptr, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes,
                       stream, pool_out, nullptr, -1, rand);
@@ -397,10 +393,6 @@ extern "C" int niti_conv2d_i8_dgrad_requant_sto(const int8_t* err, const int8_t*
                                                 int div_mode, int bw_mode, unsigned rq_flags, const int8_t* relu_mask, uint32_t* sync,
                                                 size_t sync_words, int32_t* shift_out, const int32_t* exp_a, const int32_t* exp_b,
                                                 int32_t* exp_out, void* workspace, size_t workspace_bytes, void* stream) {
-  if (rand == nullptr) {
-    clear_error();
-    return fail(NITI_ERR_INVALID_ARG, "conv_dgrad_requant_sto: null pointer");
-  }
   return conv_requant("conv_dgrad_requant_sto", 1, err, w, dx8, N, H, W, C, K, R, S, stride, pad, flags, target_bits, NITI_ROUND_STOCHASTIC,
                       div_mode, bw_mode, rq_flags, relu_mask, sync, sync_words, shift_out, exp_a, exp_b, exp_out, workspace, workspace_bytes,
                       stream, nullptr, nullptr, -1, rand);

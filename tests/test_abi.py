@@ -157,6 +157,9 @@ def test_unknown_flag_bits_are_refused(lib):
         "niti_conv2d_i8_dgrad": (None, None, None) + conv + (bad, None, None, 0, None),
         "niti_conv2d_i8_wgrad": (None, None, None) + conv + (bad, None, None, 0, None),
         "niti_conv2d_i8_fprop_requant": (None, None, None) + conv + (bad, 7, 0, 0, 0, 0, None, 0, None, None, None, None, None, 0, None),
+        # the StoShift forms: (pooled output,) random integers behind the output, no method argument
+        "niti_conv2d_i8_fprop_requant_sto": (None, None, None, None, None) + conv + (bad, 7, 0, 0, 0, None, 0, None, None, None, None, None, 0, None),
+        "niti_conv2d_i8_dgrad_requant_sto": (None, None, None, None) + conv + (bad, 7, 0, 0, 0, None, None, 0, None, None, None, None, None, 0, None),
         "niti_conv2d_i8_wgrad_update": (None, None, None, 16) + conv + (bad, 5, 0, 0, 0, None, 0, None, None, None, None, None, None, None,
                                                                       None, 0, None),
         "niti_gemm_i8": (0, 1, None, None, None, 4, 4, 16, bad, None, None, 0, None),
