@@ -182,6 +182,130 @@ __global__ __launch_bounds__(1024) void fcw_fwd_kernel(const FcwArgs a) {
   *reinterpret_cast<uint32_t*>(a.out8 + at) = pack4_i8(r[0], r[1], r[2], r[3]);
 }
 
+// ---- forward, operands through LDS --------------------------------------------------------------------------
+// The kernel above fetches its fragments as 64-byte pieces of the rows, which the path from L2 into a compute unit
+// moves at well under half the rate of whole 128-byte lines - and that path is what bounds this pass (a workgroup
+// pulls (16 + MT * 16) rows of F bytes).  Here (F a multiple of 128) every wavefront stages its share of the reduction
+// one line per row at a time (buffer_load ... lds: an instruction moves eight rows' lines, lane -> (row lane / 8,
+// 16-byte piece lane % 8), pieces XOR-swizzled by the row so that the fragment reads below spread over the banks; every
+// instruction's kilobyte starts 16 bytes further on for the same reason) and reads the MFMA fragments from there.
+// Eight wavefronts split the reduction; a wavefront only ever reads what it loaded itself, so the loop needs no
+// barrier: two buffers per wavefront, the next line on its way while this one multiplies.
+constexpr int kFwdInstrBytes = 1024 + 16;
+template <int MT>
+constexpr int fwd_lds_stage_bytes() { return (2 + 2 * MT) * kFwdInstrBytes; }
+template <int MT>
+__global__ __launch_bounds__(512) void fcw_fwd_lds_kernel(const FcwArgs a) {
+  constexpr int NI = 2 + 2 * MT;                      // load instructions per line: 16 weight rows, MT x 16 sample rows
+  constexpr int STAGE = fwd_lds_stage_bytes<MT>();
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // 8 wavefronts x 2 stages; later the partial sums
+  int (*part)[MT * 256] = reinterpret_cast<int (*)[MT * 256]>(smem);
+  uint32_t* const words = reinterpret_cast<uint32_t*>(smem + 8 * 2 * STAGE);
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int o0 = blockIdx.x * 16;
+  const int m0 = blockIdx.y * (MT * 16);
+  const int k0 = wave * a.kchunk;
+  const int nlines = k0 < a.F ? (min(k0 + a.kchunk, a.F) - k0) >> 7 : 0;
+  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(a.w, 0, a.O * a.F, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.act), 0, a.M * a.F, 0x00020000);
+  // staging: instruction j moves rows 8 j .. 8 j + 7 of the (16 + MT * 16)-row panel
+  const int r8 = lane >> 3, piece = (lane & 7) ^ r8;
+  int src[NI];
+#pragma unroll
+  for (int j = 0; j < NI; ++j) {
+    const int row = 8 * j + r8;
+    const int g = row < 16 ? o0 + row : m0 + row - 16;            // weight row / sample
+    const bool in = row < 16 ? g < a.O : g < a.M;
+    src[j] = in ? g * a.F + piece * 16 : static_cast<int>(0x80000000u);   // out of range whatever scalar offset is added: zeros
+  }
+  const unsigned stage0 = lds_addr(smem) + wave * (2 * STAGE);
+  auto issue = [&](int line, int buf) {
+    const int kb = k0 + line * 128;
+#pragma unroll
+    for (int j = 0; j < NI; ++j) {
+      const unsigned dst = stage0 + buf * STAGE + j * kFwdInstrBytes;
+      const int off = src[j];
+      if (j < 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst), 16, off, kb, 0, 0);
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, NITI_LDS_AT(dst), 16, off, kb, 0, 0);
+    }
+  };
+  // fragments: lane (row i = lane % 16, 16-byte group kg = lane / 16) of 64-step s reads piece 4 s + kg of row i
+  const int fi = lane & 15, kg = lane >> 4;
+  const unsigned frow = (fi >> 3) * kFwdInstrBytes + (fi & 7) * 128;
+  unsigned fpiece[2];
+#pragma unroll
+  for (int sstep = 0; sstep < 2; ++sstep) fpiece[sstep] = static_cast<unsigned>(((4 * sstep + kg) ^ (fi & 7)) * 16);
+  v4i acc[MT];
+  const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+  for (int t = 0; t < MT; ++t) acc[t] = zero;
+  if (nlines > 0) issue(0, 0);
+  for (int line = 0; line < nlines; ++line) {
+    const int buf = line & 1;
+    if (line + 1 < nlines) {
+      issue(line + 1, buf ^ 1);
+      __builtin_amdgcn_s_waitcnt(0x0F70 | NI);                     // vmcnt(NI): this line has landed, the next one is on its way
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);                          // vmcnt(0)
+    }
+    const unsigned base = stage0 + buf * STAGE + frow;
+    v4i fw[2], fa[MT][2];
+#pragma unroll
+    for (int sstep = 0; sstep < 2; ++sstep) {
+      fw[sstep] = lds_read_b128(base + fpiece[sstep]);
+#pragma unroll
+      for (int t = 0; t < MT; ++t) fa[t][sstep] = lds_read_b128(base + (2 + 2 * t) * kFwdInstrBytes + fpiece[sstep]);
+    }
+    lds_settle<0>();
+#pragma unroll
+    for (int sstep = 0; sstep < 2; ++sstep) {
+      asm volatile("" : "+v"(fw[sstep]));
+#pragma unroll
+      for (int t = 0; t < MT; ++t) {
+        asm volatile("" : "+v"(fa[t][sstep]));
+        acc[t] = __builtin_amdgcn_mfma_i32_16x16x64_i8(fw[sstep], fa[t][sstep], acc[t], 0, 0, 0);
+      }
+    }
+  }
+  sync_mem();   // every wavefront is done with its stages: the area now takes the partial sums
+#pragma unroll
+  for (int t = 0; t < MT; ++t)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) part[wave][t * 256 + i * 64 + lane] = acc[t][i];
+  __syncthreads();
+  // wavefront t completes tile t (wavefronts beyond MT only take part in the barriers)
+  uint32_t lmax = 0;
+  v4i fin = zero;
+  if (wave < MT) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int sum = 0;
+#pragma unroll
+      for (int w = 0; w < 8; ++w) sum += part[w][wave * 256 + i * 64 + lane];
+      fin[i] = sum;
+      const uint32_t u = uabs(sum);                        // rows beyond M and columns beyond O are sums of zeros
+      lmax = u > lmax ? u : lmax;
+    }
+  }
+  const int shift = grid_shift<8>(a, lmax, words, words + 8);
+  if (wave >= MT) return;
+  const int m = m0 + wave * 16 + (lane & 15);
+  const int ob = o0 + 4 * (lane >> 4);
+  if (m >= a.M || ob >= a.O) return;                       // O is a multiple of 4: a dword is inside or outside
+  const bool trunc = a.trunc != 0, relu = (a.rq_flags & NITI_RQ_RELU) != 0;
+  const long long at = static_cast<long long>(m) * a.O + ob;
+  v4i u = zero;
+  if (a.method == NITI_ROUND_STOCHASTIC) u = *reinterpret_cast<const v4i*>(a.rand + at);
+  int r[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    r[i] = round_any(fin[i], shift, a.method, trunc, u[i]);
+    if (relu && r[i] < 0) r[i] = 0;
+  }
+  *reinterpret_cast<uint32_t*>(a.out8 + at) = pack4_i8(r[0], r[1], r[2], r[3]);
+}
+
 // ---- data gradient ------------------------------------------------------------------------------------------
 // grid.x = 32-feature tiles of the result, grid.y = groups of 128 samples.  MFMA A = 32 features x 32 reduction steps
 // (transposing reads of the staged weight columns), B = 32 samples x 32 steps (error rows): result element 4 g + e of
@@ -421,6 +545,13 @@ int resident_cached(int (&cache)[kDeviceSlots], K kernel, int threads, size_t ld
   return r;
 }
 
+size_t fwd_lds_bytes(int mt) { return static_cast<size_t>(16) * (2 + 2 * mt) * kFwdInstrBytes + 32 * 4; }
+// workgroups of the LDS-staged forward kernel the device holds at once (MT = 1, 2)
+int fwd_lds_resident(int mt) {
+  static int c1[kDeviceSlots] = {}, c2[kDeviceSlots] = {};
+  if (mt == 1) return resident_cached(c1, fcw_fwd_lds_kernel<1>, 512, fwd_lds_bytes(1));
+  return resident_cached(c2, fcw_fwd_lds_kernel<2>, 512, fwd_lds_bytes(2));
+}
 int fwd_resident(int mt) {
   static int c1[kDeviceSlots] = {}, c2[kDeviceSlots] = {}, c4[kDeviceSlots] = {};
   if (mt == 1) return resident_cached(c1, fcw_fwd_kernel<1>, 1024, fwd_lds(1));
@@ -545,6 +676,14 @@ extern "C" int niti_linear_i8_fwd_requant(const int8_t* act, const int8_t* w, in
   plan(NITI_FC_FORWARD, M, O, F, &mt);
   const dim3 grid((O + 15) / 16, (M + 16 * mt - 1) / (16 * mt));
   hipStream_t s = static_cast<hipStream_t>(stream);
+  // whole lines through LDS where the rows are whole lines (NITI_FC_LDS=0 pins the direct-fragment kernel)
+  const char* e = getenv("NITI_FC_LDS");
+  if (F % 128 == 0 && mt <= 2 && (e == nullptr || e[0] != '0') && static_cast<long long>(grid.x) * grid.y <= fwd_lds_resident(mt)) {
+    a.kchunk = ((F + 7) / 8 + 127) / 128 * 128;
+    if (mt == 1) hipLaunchKernelGGL(fcw_fwd_lds_kernel<1>, grid, dim3(512), fwd_lds_bytes(1), s, a);
+    else hipLaunchKernelGGL(fcw_fwd_lds_kernel<2>, grid, dim3(512), fwd_lds_bytes(2), s, a);
+    return check_launch(who);
+  }
   if (mt == 1) hipLaunchKernelGGL(fcw_fwd_kernel<1>, grid, dim3(1024), fwd_lds(1), s, a);
   else if (mt == 2) hipLaunchKernelGGL(fcw_fwd_kernel<2>, grid, dim3(1024), fwd_lds(2), s, a);
   else hipLaunchKernelGGL(fcw_fwd_kernel<4>, grid, dim3(1024), fwd_lds(4), s, a);
