@@ -387,6 +387,124 @@ __global__ __launch_bounds__(512) void fcw_dgrad_kernel(const FcwArgs a) {
   }
 }
 
+// ---- data gradient, operands through LDS as whole lines -----------------------------------------------------------
+// The kernel above stages 32-byte pieces of the weight rows (a quarter of every line it fetches), takes the error rows
+// in 32-byte pieces as well and stores 4-byte pieces.  Here (F and O multiples of 128) a workgroup owns 128 features x
+// 32 samples: per chunk of 128 reduction steps it stages w[o .. o+128)[f0 .. f0+128) and err[m0 .. m0+32)[o .. o+128) -
+// one whole line per row (buffer_load ... lds, pieces XOR-swizzled by the row) - through a ring of three stages with one
+// barrier per chunk; 8 wavefronts = 4 feature quarters x 2 halves of the chunk; the rounded bytes leave through an LDS
+// patch so that every sample's 128 features are one line.
+constexpr int kDgStage = 128 * 128 + 32 * 128;        // weight chunk + error chunk
+constexpr int kDgLdsBytes = 3 * kDgStage + 32 * 4;
+__global__ __launch_bounds__(512) void fcw_dgrad_lds_kernel(const FcwArgs a) {
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // 3 stages; later 16 KB of parked sums / the 4 KB patch
+  uint32_t* const words = reinterpret_cast<uint32_t*>(smem + 3 * kDgStage);
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int f0 = blockIdx.x * 128;
+  const int m0 = blockIdx.y * 32;
+  const int nchunks = a.O >> 7;
+  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(a.w, 0, a.O * a.F, 0x00020000);
+  const __amdgpu_buffer_rsrc_t re = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.err), 0, a.M * a.O, 0x00020000);
+  // staging: 20 instructions per chunk (16 of weight rows, 4 of error rows), wavefront w issues numbers w, w + 8, w + 16
+  const int r8 = lane >> 3, piece = (lane & 7) ^ r8;
+  constexpr int kFar = static_cast<int>(0x80000000u);   // out of range whatever scalar offset is added: zeros
+  const int src0 = (8 * wave + r8) * a.F + f0 + piece * 16;                 // weight rows 8 w ..
+  const int src1 = (8 * (wave + 8) + r8) * a.F + f0 + piece * 16;           // weight rows 64 + 8 w ..
+  // error rows (wavefronts 0 - 3): swizzled by row / 2, since their readers below take 16 bytes of 16 consecutive rows at once
+  const int epiece = (lane & 7) ^ ((4 * (wave & 1) + (r8 >> 1)) & 7);
+  const int src2 = m0 + 8 * wave + r8 < a.M ? (m0 + 8 * wave + r8) * a.O + epiece * 16 : kFar;
+  const unsigned lds0 = lds_addr(smem);
+  auto issue = [&](int c, int st) {
+    const unsigned dst = lds0 + st * kDgStage;
+    const int wo = c * 128 * a.F, eo = c * 128;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst + wave * 1024), 16, src0, wo, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst + (wave + 8) * 1024), 16, src1, wo, 0, 0);
+    if (wave < 4) __builtin_amdgcn_raw_ptr_buffer_load_lds(re, NITI_LDS_AT(dst + 16384 + wave * 1024), 16, src2, eo, 0, 0);
+  };
+  // fragments
+  const int ft = wave & 3, kh = wave >> 2;
+  const int lr = lane & 31, lk = lane >> 5;
+  const int j = lane & 15, gg = (lane >> 4) & 1;
+  // weight chunk row kh * 64 + s * 32 + lk * 16 + (j >> 1) (+ 8), bytes ft * 32 + gg * 16 + 8 (j & 1) .. + 8
+  const unsigned a_off = static_cast<unsigned>((kh * 64 + lk * 16 + (j >> 1)) * 128 + (((ft * 2 + gg) ^ (j >> 1)) << 4) + 8 * (j & 1));
+  // error chunk row lr, bytes kh * 64 + s * 32 + lk * 16 .. + 16
+  unsigned b_off[2];
+#pragma unroll
+  for (int sstep = 0; sstep < 2; ++sstep) b_off[sstep] = static_cast<unsigned>(16384 + lr * 128 + (((kh * 4 + sstep * 2 + lk) ^ ((lr >> 1) & 7)) << 4));
+  v16i acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+  issue(0, 0);
+  if (nchunks > 1) issue(1, 1);
+  for (int c = 0; c < nchunks; ++c) {
+    // younger than this chunk's loads: the next chunk's (3 per wavefront 0 - 3, 2 per wavefront 4 - 7)
+    if (c + 1 < nchunks) {
+      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
+      else __builtin_amdgcn_s_waitcnt(0x0F70 | 2);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    sync_mem();   // the chunk has landed for every wavefront, and the stage refilled below has been read by all
+    if (c + 2 < nchunks) issue(c + 2, (c + 2) % 3);
+    const unsigned base = lds0 + (c % 3) * kDgStage;
+    v2i lo[2], hi[2];
+    v4i fb[2];
+#pragma unroll
+    for (int sstep = 0; sstep < 2; ++sstep) {
+      lo[sstep] = lds_read_tr8<0>(base + a_off + sstep * 4096);
+      hi[sstep] = lds_read_tr8<1024>(base + a_off + sstep * 4096);
+      fb[sstep] = lds_read_b128(base + b_off[sstep]);
+    }
+    lds_settle<0>();
+#pragma unroll
+    for (int sstep = 0; sstep < 2; ++sstep) {
+      asm volatile("" : "+v"(fb[sstep]));
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lds_landed(lo[sstep], hi[sstep]), fb[sstep], acc, 0, 0, 0);
+    }
+  }
+  sync_mem();   // every wavefront is done with the stages
+  int* const park = reinterpret_cast<int*>(smem) + ft * (16 * 64) + lane;
+  if (kh == 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) park[e * 64] = acc[e];
+  }
+  __syncthreads();
+  uint32_t lmax = 0;
+  if (kh == 0) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      acc[e] += park[e * 64];
+      const uint32_t u = uabs(acc[e]);                 // samples beyond M are sums of zeros
+      lmax = u > lmax ? u : lmax;
+    }
+  }
+  const int shift = grid_shift<8>(a, lmax, words, words + 8);   // its barriers also retire the parked sums
+  const int m = m0 + lr;
+  const bool trunc = a.trunc != 0;
+  int8_t* const patch = smem + 16384;                            // [32 samples][128 features], clear of the parked sums
+  if (kh == 0) {
+    const v4i zero = {0, 0, 0, 0};
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+      const int fo = ft * 32 + 8 * g + 4 * lk;
+      v4i u = zero;
+      if (a.method == NITI_ROUND_STOCHASTIC && m < a.M) u = *reinterpret_cast<const v4i*>(a.rand + static_cast<long long>(m) * a.F + f0 + fo);
+      int r[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) r[e] = round_any(acc[4 * g + e], shift, a.method, trunc, u[e]);
+      *reinterpret_cast<uint32_t*>(patch + lr * 128 + fo) = pack4_i8(r[0], r[1], r[2], r[3]);
+    }
+  }
+  __syncthreads();
+  if (tid < 256) {
+    const int row = tid >> 3, p16 = tid & 7;
+    if (m0 + row < a.M)
+      *reinterpret_cast<v4i*>(a.out8 + static_cast<long long>(m0 + row) * a.F + f0 + p16 * 16) = *reinterpret_cast<const v4i*>(patch + row * 128 + p16 * 16);
+  }
+}
+
 // ---- weight gradient + update -------------------------------------------------------------------------------
 // grid.x = 256-feature tiles, grid.y = groups of T 32-row tiles of the weight matrix.  Samples are walked in chunks of
 // 128.  MFMA A = 32 features x 32 samples (activation columns), B = 32 output features x 32 samples (error columns):
@@ -565,6 +683,18 @@ int wgrad_resident(int t) {
   return resident_cached(c4, fcw_wgrad_kernel<4>, 512, wgrad_lds(4));
 }
 
+int dgrad_lds_resident() {
+  static int c[kDeviceSlots] = {};
+  return resident_cached(c, fcw_dgrad_lds_kernel, 512, static_cast<size_t>(kDgLdsBytes));
+}
+// workgroups of the whole-line data-gradient kernel for this shape, or 0 when the other kernel runs it
+long long dgrad_lds_blocks(int M, int O, int F) {
+  if (F % 128 != 0 || O % 128 != 0) return 0;
+  const char* e = getenv("NITI_FC_LDS");
+  if (e != nullptr && e[0] == '0') return 0;
+  const long long nb = static_cast<long long>(F / 128) * ((M + 31) / 32);
+  return (nb <= kMaxSlots && nb <= dgrad_lds_resident()) ? nb : 0;
+}
 int dgrad_resident(int O) {
   static int attr_of[kDeviceSlots] = {};
   int& attr = attr_of[device_slot()];
@@ -583,6 +713,10 @@ long long plan(int which, int M, int O, int F, int* tiles) {
   *tiles = 0;
   if (!shape_ok(which, M, O, F)) return 0;
   if (which == NITI_FC_DGRAD) {
+    if (const long long nl = dgrad_lds_blocks(M, O, F)) {
+      *tiles = 1;
+      return nl;
+    }
     const long long nb = static_cast<long long>(F / 32) * ((M + 127) / 128);
     *tiles = 1;
     return (nb <= kMaxSlots && nb <= dgrad_resident(O)) ? nb : 0;
@@ -704,6 +838,12 @@ extern "C" int niti_linear_i8_dgrad_requant(const int8_t* err, const int8_t* w, 
   a.err = err;
   a.w = const_cast<int8_t*>(w);
   a.out8 = dx8;
+  if (dgrad_lds_blocks(M, O, F) != 0) {
+    if (!aligned16(dx8)) return fail(NITI_ERR_INVALID_ARG, "%s: misaligned pointer", who);
+    hipLaunchKernelGGL(fcw_dgrad_lds_kernel, dim3(F / 128, (M + 31) / 32), dim3(512), static_cast<size_t>(kDgLdsBytes),
+                       static_cast<hipStream_t>(stream), a);
+    return check_launch(who);
+  }
   const size_t lds = dgrad_lds(O);
   hipLaunchKernelGGL(fcw_dgrad_kernel, dim3(F / 32, (M + 127) / 128), dim3(512), lds, static_cast<hipStream_t>(stream), a);
   return check_launch(who);
