@@ -484,7 +484,7 @@ def side_workloads(dev):
         t = _avg_us(lambda: int8mm_cuda.int8_mm(lhs, rhs))
         fc["dropin_int8_mm_" + name + "_us"] = round(t, 2)
         fc["dropin_int8_mm_" + name + "_gbs"] = round((m_ * k_ + k_ * n_ + 4 * m_ * n_) / t * 1e-3, 1)
-    fc["dropin_note"] = "int8mm_cuda.int8_mm(lhs, rhs) -> int32, one launch, operands read as stored; bytes = m k + k n + 4 m n"
+    fc["dropin_note"] = "int8mm_cuda.int8_mm(lhs, rhs) -> int32, operands read as stored (one launch; the forward product splits its reduction over workgroups and adds the parts in a second launch); bytes = m k + k n + 4 m n"
     out["config1"] = fc
     del A, W, G, u_f, u_d, u_w, Wu, Wt, Gt
     # ---- max-pool

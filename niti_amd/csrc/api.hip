@@ -583,7 +583,7 @@ extern "C" int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err,
 
 extern "C" size_t niti_gemm_i8_workspace(int trans_a, int trans_b, int m, int n, int k) {
   if (m <= 0 || n <= 0 || k <= 0) return 0;
-  if (gemm_kmajor_shape(trans_a, trans_b, m, n, k)) return 0;   // read as stored
+  if (gemm_kmajor_shape(trans_a, trans_b, m, n, k)) return gemm_kmajor_workspace(trans_a, trans_b, m, n, k);   // read as stored; partial sums of a split reduction
   const size_t kp = static_cast<size_t>(round16(k));
   size_t bytes = 0;
   if (trans_a || k % 16 != 0) bytes += round256(static_cast<size_t>(m) * kp);
@@ -605,7 +605,7 @@ extern "C" int niti_gemm_i8(int trans_a, int trans_b, const int8_t* a, const int
   // reduction index slow in b (and in a): one launch, both operands read as stored
   if (gemm_kmajor_shape(trans_a, trans_b, m, n, k)) {
     if (!aligned16(a) || !aligned16(b)) return fail(NITI_ERR_INVALID_ARG, "gemm: operands must be 16-byte aligned");
-    return launch_gemm_kmajor(trans_a, trans_b, a, b, c, m, n, k, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, absmax, s);
+    return launch_gemm_kmajor(trans_a, trans_b, a, b, c, m, n, k, (flags & NITI_EPI_F32_ROUNDTRIP) != 0, absmax, workspace, s);
   }
   const int kp = round16(k);
   int8_t* ws = static_cast<int8_t*>(workspace);

@@ -196,8 +196,9 @@ int launch_conv_igemm(const ConvProblem& p, hipStream_t stream);
 // int32 GEMM of operands with a slow reduction index (NN: b as [k][n]; TN: a as [k][m] too; TT: a as [k][m], b as
 // [n][k]), read as stored
 bool gemm_kmajor_shape(int trans_a, int trans_b, int m, int n, int k);
+size_t gemm_kmajor_workspace(int trans_a, int trans_b, int m, int n, int k);   // partial sums of a reduction split over workgroups
 int launch_gemm_kmajor(int trans_a, int trans_b, const int8_t* a, const int8_t* b, int32_t* c, int m, int n, int k, bool roundtrip,
-                       uint32_t* absmax, hipStream_t stream);
+                       uint32_t* absmax, void* workspace, hipStream_t stream);
 
 int launch_fill_u32(uint32_t* dst, int64_t n, uint32_t value, hipStream_t stream);
 // dst[c][r][s][k] = w[k][R-1-r][S-1-s][c]

@@ -165,6 +165,167 @@ __global__ __launch_bounds__(512) void gemm_kmajor_kernel(const KmArgs g) {
         v4i{acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
 }
 
+// ---- NN form, both operands through LDS as whole 128-byte lines ------------------------------------------------------
+// The kernel above stages b in 32-byte pieces of its rows and takes a in 32-byte pieces as well; the path from L2 into
+// a compute unit moves such pieces at a quarter of the rate of whole lines.  Here (n and k multiples of 128) a workgroup
+// owns 32 rows x 128 columns of c and a range of the reduction: per chunk of 128 steps it stages b[k .. k+128)[n0 ..
+// n0+128) and a[m0 .. m0+32)[k .. k+128), one whole line per row (buffer_load ... lds, 16-byte pieces XOR-swizzled by
+// the row), through a ring of three stages with one barrier per chunk.  8 wavefronts = 4 column quarters x 2 halves of
+// the chunk.  blockIdx.z splits the reduction when the tiles alone would leave most of the device idle: the parts then
+// write int32 partial results and km_reduce_parts_kernel adds them.
+constexpr int kLnStage = 128 * 128 + 32 * 128;        // b chunk + a chunk
+constexpr int kLnPatchPitch = 128 * 4 + 16;
+constexpr int kLnLdsBytes = 3 * kLnStage;
+
+struct LnArgs {
+  const int8_t* a;
+  const int8_t* b;
+  int32_t* out;           // c, or the partial results [part][m * n]
+  uint32_t* absmax;
+  int m, n, k;
+  int chunks_per_part;
+  int parts;
+  int roundtrip;
+  int transposed_out;
+};
+
+__global__ __launch_bounds__(512) void gemm_nn_lines_kernel(const LnArgs g) {
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // 3 stages; later 16 KB of parked sums, then the patch
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int n0 = blockIdx.x * 128;
+  const int m0 = blockIdx.y * 32;
+  const int nchunks_all = g.k >> 7;
+  const int c0 = blockIdx.z * g.chunks_per_part;
+  const int nchunks = min(g.chunks_per_part, nchunks_all - c0);
+  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.b), 0, g.k * g.n, 0x00020000);
+  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.a), 0, g.m * g.k, 0x00020000);
+  // staging: 20 instructions per chunk (16 of b's rows, 4 of a's rows), wavefront w issues numbers w, w + 8, w + 16
+  const int r8 = lane >> 3, piece = (lane & 7) ^ r8;
+  constexpr int kFar = static_cast<int>(0x80000000u);   // out of range whatever scalar offset is added: zeros
+  const int src0 = (8 * wave + r8) * g.n + n0 + piece * 16;
+  const int src1 = (8 * (wave + 8) + r8) * g.n + n0 + piece * 16;
+  // a's rows: swizzled by row / 2, since their readers take 16 bytes of 16 consecutive rows at once
+  const int apiece = (lane & 7) ^ ((4 * (wave & 1) + (r8 >> 1)) & 7);
+  const int src2 = m0 + 8 * wave + r8 < g.m ? (m0 + 8 * wave + r8) * g.k + apiece * 16 : kFar;
+  const unsigned lds0 = lds_addr(smem);
+  auto issue = [&](int c, int st) {
+    const unsigned dst = lds0 + st * kLnStage;
+    const int bo = (c0 + c) * 128 * g.n, ao = (c0 + c) * 128;
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, NITI_LDS_AT(dst + wave * 1024), 16, src0, bo, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, NITI_LDS_AT(dst + (wave + 8) * 1024), 16, src1, bo, 0, 0);
+    if (wave < 4) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, NITI_LDS_AT(dst + 16384 + wave * 1024), 16, src2, ao, 0, 0);
+  };
+  const int ft = wave & 3, kh = wave >> 2;
+  const int lr = lane & 31, lk = lane >> 5;
+  const int j = lane & 15, gg = (lane >> 4) & 1;
+  // b chunk row kh * 64 + s * 32 + lk * 16 + (j >> 1) (+ 8), bytes ft * 32 + gg * 16 + 8 (j & 1) .. + 8
+  const unsigned b_off = static_cast<unsigned>((kh * 64 + lk * 16 + (j >> 1)) * 128 + (((ft * 2 + gg) ^ (j >> 1)) << 4) + 8 * (j & 1));
+  // a chunk row lr, bytes kh * 64 + s * 32 + lk * 16 .. + 16
+  unsigned a_off[2];
+#pragma unroll
+  for (int sstep = 0; sstep < 2; ++sstep) a_off[sstep] = static_cast<unsigned>(16384 + lr * 128 + (((kh * 4 + sstep * 2 + lk) ^ ((lr >> 1) & 7)) << 4));
+  v16i acc;
+#pragma unroll
+  for (int e = 0; e < 16; ++e) acc[e] = 0;
+  issue(0, 0);
+  if (nchunks > 1) issue(1, 1);
+  for (int c = 0; c < nchunks; ++c) {
+    // younger than this chunk's loads: the next chunk's (3 per wavefront 0 - 3, 2 per wavefront 4 - 7)
+    if (c + 1 < nchunks) {
+      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
+      else __builtin_amdgcn_s_waitcnt(0x0F70 | 2);
+    } else {
+      __builtin_amdgcn_s_waitcnt(0x0F70);
+    }
+    km_sync();   // the chunk has landed for every wavefront, and the stage refilled below has been read by all
+    if (c + 2 < nchunks) issue(c + 2, (c + 2) % 3);
+    const unsigned base = lds0 + (c % 3) * kLnStage;
+    v2i lo[2], hi[2];
+    v4i fa[2];
+#pragma unroll
+    for (int sstep = 0; sstep < 2; ++sstep) {
+      lo[sstep] = lds_read_tr8<0>(base + b_off + sstep * 4096);
+      hi[sstep] = lds_read_tr8<1024>(base + b_off + sstep * 4096);
+      fa[sstep] = lds_read_b128(base + a_off[sstep]);
+    }
+    lds_settle<0>();
+#pragma unroll
+    for (int sstep = 0; sstep < 2; ++sstep) {
+      asm volatile("" : "+v"(fa[sstep]));
+      // MFMA A = 32 columns of c x 32 reduction steps, B = 32 rows of c x 32 steps
+      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lds_landed(lo[sstep], hi[sstep]), fa[sstep], acc, 0, 0, 0);
+    }
+  }
+  km_sync();   // every wavefront is done with the stages
+  int* const park = reinterpret_cast<int*>(smem) + ft * (16 * 64) + lane;
+  if (kh == 1) {
+#pragma unroll
+    for (int e = 0; e < 16; ++e) park[e * 64] = acc[e];
+  }
+  __syncthreads();
+  // element 4 q + e of a lane is column n0 + ft * 32 + 8 q + 4 (lane / 32) + e of row m0 + lane % 32
+  const bool last = g.parts == 1;
+  int32_t* const out = g.out + static_cast<long long>(blockIdx.z) * g.m * g.n;
+  int8_t* const patch = smem + 16384;                            // [32 rows][128 columns] of int32, clear of the parked sums
+  if (kh == 0) {
+    uint32_t lmax = 0;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+      int v = acc[e] + park[e * 64];
+      if (last && g.roundtrip) v = f32_roundtrip(v);
+      acc[e] = v;
+      const uint32_t u = uabs(v);                         // rows beyond m are sums of zeros
+      lmax = u > lmax ? u : lmax;
+    }
+    if (last && g.absmax != nullptr) fold_absmax(g.absmax, lmax);
+    if (g.transposed_out) {   // 32 lanes write 32 consecutive rows of one column: a line
+      if (m0 + lr < g.m) {
+#pragma unroll
+        for (int e = 0; e < 16; ++e)
+          out[static_cast<long long>(n0 + ft * 32 + 8 * (e >> 2) + 4 * lk + (e & 3)) * g.m + m0 + lr] = acc[e];
+      }
+    } else {
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<v4i*>(patch + lr * kLnPatchPitch + (ft * 32 + 8 * q + 4 * lk) * 4) =
+            v4i{acc[4 * q], acc[4 * q + 1], acc[4 * q + 2], acc[4 * q + 3]};
+    }
+  }
+  if (g.transposed_out) return;
+  __syncthreads();
+  const int row = tid >> 4, p16 = tid & 15;
+  if (m0 + row >= g.m) return;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    *reinterpret_cast<v4i*>(out + static_cast<long long>(m0 + row) * g.n + n0 + (p16 + 16 * i) * 4) =
+        *reinterpret_cast<const v4i*>(patch + row * kLnPatchPitch + (p16 + 16 * i) * 16);
+}
+
+// c[i] = sum over the parts of the partial results, four elements per thread
+__global__ __launch_bounds__(256) void km_reduce_parts_kernel(const int32_t* __restrict__ part, int32_t* __restrict__ c, long long quads, int parts,
+                                                              int roundtrip, uint32_t* absmax) {
+  const long long i = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+  uint32_t lmax = 0;
+  if (i < quads) {
+    v4i s = *reinterpret_cast<const v4i*>(part + 4 * i);
+    for (int p = 1; p < parts; ++p) {
+      const v4i v = *reinterpret_cast<const v4i*>(part + 4 * (static_cast<long long>(p) * quads + i));
+#pragma unroll
+      for (int e = 0; e < 4; ++e) s[e] += v[e];
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      if (roundtrip) s[e] = f32_roundtrip(s[e]);
+      const uint32_t u = uabs(s[e]);
+      lmax = u > lmax ? u : lmax;
+    }
+    *reinterpret_cast<v4i*>(c + 4 * i) = s;
+  }
+  if (absmax != nullptr) fold_absmax(absmax, lmax);
+}
+
 constexpr size_t km_lds(bool trans_a, int mt) {
   const size_t stage = trans_a ? static_cast<size_t>(kKmChunkTN) * 32 + static_cast<size_t>(kKmChunkTN) * (mt * 32 + 16)
                                : static_cast<size_t>(kKmChunkNN) * 32;
@@ -188,6 +349,33 @@ int km_launch(const KmArgs& g, hipStream_t stream) {
   return check_launch("gemm_kmajor");
 }
 
+// The whole-line kernel's plan for an NN product (after the TT form has been turned into one): 0 parts = not taken.
+struct LnPlan {
+  int parts, chunks_per_part;
+};
+LnPlan lines_plan(int m, int n, int k) {
+  LnPlan p{0, 0};
+  if (n % 128 != 0 || k % 128 != 0 || (m + 31) / 32 > 65535) return p;
+  if (static_cast<long long>(m) * k >= 0x7fffffffLL || static_cast<long long>(k) * n >= 0x7fffffffLL) return p;
+  static const bool off = [] {
+    const char* e = getenv("NITI_GEMM_LINES");
+    return e != nullptr && e[0] == '0';
+  }();
+  if (off) return p;
+  const long long tiles = static_cast<long long>(n / 128) * ((m + 31) / 32);
+  const int chunks = k / 128;
+  int parts = 1;
+  if (tiles < 192) {
+    parts = static_cast<int>((256 + tiles - 1) / tiles);
+    if (parts > chunks / 2) parts = chunks / 2;
+    if (parts > 32) parts = 32;
+    if (parts < 1) parts = 1;
+  }
+  p.chunks_per_part = (chunks + parts - 1) / parts;
+  p.parts = (chunks + p.chunks_per_part - 1) / p.chunks_per_part;
+  return p;
+}
+
 }  // namespace
 
 // Shapes the direct kernels take: 32-column tiles, whole reduction steps, 16-byte pieces of every row.
@@ -199,8 +387,21 @@ bool gemm_kmajor_shape(int trans_a, int trans_b, int m, int n, int k) {
   return (m + 127) / 128 <= 65535;
 }
 
+// bytes of partial results the whole-line kernel wants for this product (0: none, or another kernel takes it)
+size_t gemm_kmajor_workspace(int trans_a, int trans_b, int m, int n, int k) {
+  if (trans_b != 0) {
+    const int t = m;
+    m = n;
+    n = t;
+    trans_a = 0;
+  }
+  if (trans_a != 0) return 0;
+  const LnPlan p = lines_plan(m, n, k);
+  return p.parts > 1 ? static_cast<size_t>(p.parts) * m * n * 4 : 0;
+}
+
 int launch_gemm_kmajor(int trans_a, int trans_b, const int8_t* a, const int8_t* b, int32_t* c, int m, int n, int k, bool roundtrip,
-                       uint32_t* absmax, hipStream_t stream) {
+                       uint32_t* absmax, void* workspace, hipStream_t stream) {
   KmArgs g{a, b, c, absmax, m, n, k, roundtrip ? 1 : 0, 0};
   if (trans_b != 0) {   // rows of the kernel's product = n (rows of b), columns = m (columns of a)
     g.a = b;
@@ -209,6 +410,26 @@ int launch_gemm_kmajor(int trans_a, int trans_b, const int8_t* a, const int8_t* 
     g.n = m;
     g.transposed_out = 1;
     trans_a = 0;
+  }
+  if (trans_a == 0) {
+    const LnPlan p = lines_plan(g.m, g.n, k);
+    if (p.parts > 0) {
+      static bool attr_set[kDeviceSlots] = {};
+      bool& done = attr_set[device_slot()];
+      if (!done) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nn_lines_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLnLdsBytes) != hipSuccess)
+          return fail(NITI_ERR_LAUNCH, "gemm: cannot reserve %d bytes of LDS", kLnLdsBytes);
+        done = true;
+      }
+      LnArgs l{g.a, g.b, p.parts > 1 ? static_cast<int32_t*>(workspace) : c, absmax, g.m, g.n, k, p.chunks_per_part, p.parts, g.roundtrip, g.transposed_out};
+      hipLaunchKernelGGL(gemm_nn_lines_kernel, dim3(g.n / 128, (g.m + 31) / 32, p.parts), dim3(512), static_cast<size_t>(kLnLdsBytes), stream, l);
+      if (p.parts > 1) {
+        const long long quads = static_cast<long long>(g.m) * g.n / 4;
+        hipLaunchKernelGGL(km_reduce_parts_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, stream,
+                           static_cast<const int32_t*>(workspace), c, quads, p.parts, g.roundtrip, absmax);
+      }
+      return check_launch("gemm_nn_lines");
+    }
   }
   // few 128-row tiles and a long reduction: 32-row tiles whose eight wavefronts split the reduction
   const long long tiles128 = static_cast<long long>(g.n / 32) * ((g.m + 127) / 128);

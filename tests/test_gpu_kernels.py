@@ -690,9 +690,12 @@ def test_conv_wgrad(dev, case):
 
 # the last six take the kernel that reads operands with a slow reduction index as stored (n and k multiples of 32):
 # several staged chunks, a chunk tail, row counts that are not multiples of the 128-row tile, the three products of a
-# fully connected layer 8192 -> 1024 on a batch of 128
+# fully connected layer 8192 -> 1024 on a batch of 128; then shapes for the kernel that stages whole lines (n and k
+# multiples of 128, in the doubly transposed form m and k): a row tail, a reduction split unevenly over workgroups
+# (5 chunks in 2 parts), a single chunk, several tiles, a row tail in the transposed store
 GEMM_CASES = [(128, 10, 8192), (16, 16, 16), (128, 128, 64), (100, 10, 512), (7, 5, 3), (130, 70, 100), (128, 1024, 1024), (33, 12, 8192),
-              (48, 32, 32), (200, 64, 96), (160, 96, 2080), (64, 7, 1056), (128, 1024, 8192), (128, 8192, 1024), (1024, 8192, 128)]
+              (48, 32, 32), (200, 64, 96), (160, 96, 2080), (64, 7, 1056), (128, 1024, 8192), (128, 8192, 1024), (1024, 8192, 128),
+              (100, 128, 256), (40, 256, 640), (128, 128, 128), (96, 384, 1152), (256, 40, 640)]
 
 
 @pytest.mark.parametrize("mnk", GEMM_CASES)
@@ -713,15 +716,18 @@ def test_gemm(dev, mnk, ta, tb):
     assert int(am.cpu()) == po.absmax(ref)
 
 
+@pytest.mark.parametrize("mnk", [(160, 64, 2080), (160, 128, 2176), (384, 2048, 2176)])
 @pytest.mark.parametrize("ta,tb", [(False, False), (True, False), (True, True)])
-def test_gemm_f32_epilogue_above_2_24(dev, ta, tb):
+def test_gemm_f32_epilogue_above_2_24(dev, ta, tb, mnk):
     """Sums beyond 2**24 through the kernel that reads both operands as stored: with the flag every sum takes the
-    reference epilogue's int32 -> float32 -> int32 round trip (linear_combination_clamp.h:371-389), without it none."""
+    reference epilogue's int32 -> float32 -> int32 round trip (linear_combination_clamp.h:371-389), without it none.
+    The second shape takes the whole-line kernel with the reduction split over workgroups (the round trip then happens
+    where the parts are added), the third the same kernel without a split."""
     from niti_amd import ops
     from oracle import niti_oracle as po
-    _say("gemm f32 epilogue", ta, tb)
+    _say("gemm f32 epilogue", ta, tb, mnk)
     g = torch.Generator().manual_seed(411)
-    m, n, k = 160, 64, 2080
+    m, n, k = mnk
     A, B = ri8(g, m, k), ri8(g, k, n)
     A[:40] = 127
     B[:, :20] = 127
