@@ -290,13 +290,16 @@ int niti_conv2d_i8_wgrad_update(const int8_t* act, const int8_t* err, int8_t* w,
  * (pytorch/int8mm-extension/int8mm.cpp:9-14, int8mm_kernel.cu:8-34):
  *   c[m,n] = sum_k opA[m,k] * opB[k,n],  c row-major with leading dimension n.
  * trans_a == 0: a is [m,k] row-major; 1: a is [k,m].  trans_b == 0: b is [k,n]; 1: b is [n,k].
- * Operands are read as stored, one launch, no workspace: (trans_a=0, trans_b=1) with k % 16 == 0;
+ * Operands are read as stored, no operand copy: (trans_a=0, trans_b=1) with k % 16 == 0;
  * trans_b=0 - the form the reference's extension receives (trans_a=0) and the one with both
  * reduction indices slow (trans_a=1, m % 16 == 0) - with n % 32 == 0 and k % 32 == 0, through
  * transposing LDS reads; (trans_a=1, trans_b=1) with m % 32 == 0 and k % 32 == 0 the same way
  * (it fills the [n,m] buffer behind the transposed view that int8_mm returns, from lhs and rhs
- * as the reference passes them).  Other shapes first re-lay the operand(s) into the workspace
- * (niti_gemm_i8_workspace() bytes, 0 for the cases above).
+ * as the reference passes them).  One launch - except that the forms with trans_a == trans_b
+ * whose result has few tiles and whose reduction is long (n, k multiples of 128; in the doubly
+ * transposed form m, k) split the reduction over workgroups: the int32 parts go to the workspace
+ * and a second small launch adds them.  Other shapes first re-lay the operand(s) into the
+ * workspace.  niti_gemm_i8_workspace() reports the bytes either way (0 when none are needed).
  */
 size_t niti_gemm_i8_workspace(int trans_a, int trans_b, int m, int n, int k);
 int niti_gemm_i8(int trans_a, int trans_b, const int8_t* a, const int8_t* b, int32_t* c, int m, int n, int k,

@@ -133,9 +133,14 @@ def test_workspace_sizes(lib):
     assert lib.niti_gemm_i8_workspace(0, 1, 128, 10, 100) > 0
     # operands with a slow reduction index are read as stored when n and k are multiples of 32 (the transposed
     # first operand also needs m % 16 == 0, both transposed m % 32 == 0) ...
-    assert lib.niti_gemm_i8_workspace(0, 0, 128, 1024, 8192) == 0
+    # 32 tiles of 32 x 128 and 64 chunks of the reduction: split into 8 parts of int32 partial results
+    assert lib.niti_gemm_i8_workspace(0, 0, 128, 1024, 8192) == 8 * 128 * 1024 * 4
+    assert lib.niti_gemm_i8_workspace(1, 1, 1024, 128, 8192) == 8 * 128 * 1024 * 4
+    assert lib.niti_gemm_i8_workspace(0, 0, 128, 8192, 1024) == 0     # 256 tiles: no split
+    assert lib.niti_gemm_i8_workspace(0, 0, 128, 1056, 8192) == 0     # n not a multiple of 128: the 32-byte-piece kernel
     assert lib.niti_gemm_i8_workspace(1, 0, 128, 1024, 8192) == 0
-    assert lib.niti_gemm_i8_workspace(1, 1, 1024, 10, 8192) == 0
+    assert lib.niti_gemm_i8_workspace(1, 1, 1024, 10, 8192) == 32 * 10 * 1024 * 4   # 8 tiles: 32 parts of 2 chunks
+    assert lib.niti_gemm_i8_workspace(1, 1, 1056, 10, 8192) == 0
     # ... other shapes re-lay them: b [k,n] -> [n,k16]; a [k,m] -> [m,k16]
     assert lib.niti_gemm_i8_workspace(0, 0, 128, 1000, 8192) == 1000 * 8192
     assert lib.niti_gemm_i8_workspace(1, 1, 1000, 10, 8192) == 1000 * 8192
