@@ -392,12 +392,12 @@ __global__ __launch_bounds__(512) void fcw_dgrad_kernel(const FcwArgs a) {
 // in 32-byte pieces as well and stores 4-byte pieces.  Here (F and O multiples of 128) a workgroup owns 128 features x
 // 32 samples: per chunk of 128 reduction steps it stages w[o .. o+128)[f0 .. f0+128) and err[m0 .. m0+32)[o .. o+128) -
 // one whole line per row (buffer_load ... lds, pieces XOR-swizzled by the row) - through a ring of three stages with one
-// barrier per chunk; 8 wavefronts = 4 feature quarters x 2 halves of the chunk; the rounded bytes leave through an LDS
-// patch so that every sample's 128 features are one line.
+// barrier per chunk; 8 wavefronts = 4 feature quarters x 2 halves of the chunk; the sums pass through an LDS patch into a
+// row-major arrangement for the rounding.
 constexpr int kDgStage = 128 * 128 + 32 * 128;        // weight chunk + error chunk
 constexpr int kDgLdsBytes = 3 * kDgStage + 32 * 4;
 __global__ __launch_bounds__(512) void fcw_dgrad_lds_kernel(const FcwArgs a) {
-  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // 3 stages; later 16 KB of parked sums / the 4 KB patch
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // 3 stages; later 16 KB of parked sums / the 17 KB patch
   uint32_t* const words = reinterpret_cast<uint32_t*>(smem + 3 * kDgStage);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
@@ -480,28 +480,36 @@ __global__ __launch_bounds__(512) void fcw_dgrad_lds_kernel(const FcwArgs a) {
       lmax = u > lmax ? u : lmax;
     }
   }
+  // The rounding runs in a row-major arrangement - thread (row = tid / 16, piece = tid % 16) takes features
+  // 64 q + 4 piece .. + 4 (q = 0, 1) of one sample - so that sixteen lanes read 256 consecutive bytes of random integers;
+  // those are requested here, ahead of the range exchange.
+  const int row = tid >> 4, p16 = tid & 15;
+  const bool rin = m0 + row < a.M;
+  const long long at = static_cast<long long>(m0 + row) * a.F + f0 + p16 * 4;
+  const v4i zero = {0, 0, 0, 0};
+  v4i u[2] = {zero, zero};
+  if (a.method == NITI_ROUND_STOCHASTIC && rin) {
+#pragma unroll
+    for (int q = 0; q < 2; ++q) u[q] = *reinterpret_cast<const v4i*>(a.rand + at + q * 64);
+  }
   const int shift = grid_shift<8>(a, lmax, words, words + 8);   // its barriers also retire the parked sums
-  const int m = m0 + lr;
   const bool trunc = a.trunc != 0;
-  int8_t* const patch = smem + 16384;                            // [32 samples][128 features], clear of the parked sums
+  constexpr int kPitch = 128 * 4 + 16;
+  int8_t* const patch = smem + 16384;                            // [32 samples][128 features] of int32, clear of the parked sums
   if (kh == 0) {
-    const v4i zero = {0, 0, 0, 0};
 #pragma unroll
-    for (int g = 0; g < 4; ++g) {
-      const int fo = ft * 32 + 8 * g + 4 * lk;
-      v4i u = zero;
-      if (a.method == NITI_ROUND_STOCHASTIC && m < a.M) u = *reinterpret_cast<const v4i*>(a.rand + static_cast<long long>(m) * a.F + f0 + fo);
-      int r[4];
-#pragma unroll
-      for (int e = 0; e < 4; ++e) r[e] = round_any(acc[4 * g + e], shift, a.method, trunc, u[e]);
-      *reinterpret_cast<uint32_t*>(patch + lr * 128 + fo) = pack4_i8(r[0], r[1], r[2], r[3]);
-    }
+    for (int g = 0; g < 4; ++g)
+      *reinterpret_cast<v4i*>(patch + lr * kPitch + (ft * 32 + 8 * g + 4 * lk) * 4) = v4i{acc[4 * g], acc[4 * g + 1], acc[4 * g + 2], acc[4 * g + 3]};
   }
   __syncthreads();
-  if (tid < 256) {
-    const int row = tid >> 3, p16 = tid & 7;
-    if (m0 + row < a.M)
-      *reinterpret_cast<v4i*>(a.out8 + static_cast<long long>(m0 + row) * a.F + f0 + p16 * 16) = *reinterpret_cast<const v4i*>(patch + row * 128 + p16 * 16);
+  if (!rin) return;
+#pragma unroll
+  for (int q = 0; q < 2; ++q) {
+    const v4i sum = *reinterpret_cast<const v4i*>(patch + row * kPitch + (q * 64 + p16 * 4) * 4);
+    int r[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) r[e] = round_any(sum[e], shift, a.method, trunc, u[q][e]);
+    *reinterpret_cast<uint32_t*>(a.out8 + at + q * 64) = pack4_i8(r[0], r[1], r[2], r[3]);
   }
 }
 

@@ -1025,7 +1025,8 @@ def test_group_conv_first_layer_wgrad(dev):
 
 
 @pytest.mark.parametrize("case", [(128, 8192, 1024), (40, 256, 64), (300, 512, 96), (16, 64, 32), (64, 320, 32), (128, 1024, 2048),
-                                  (7, 4096, 128)])   # M, F, O
+                                  (7, 4096, 128), (40, 384, 384), (33, 128, 256)])   # M, F, O; the last two: a ring of three
+                                                                                     # stages that wraps, ragged sample tiles
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 def test_linear_any_width(dev, case, div_mode):
     """TiLinear's three passes as single launches on operands as stored, all rounding methods (stochastic rounding on
