@@ -475,6 +475,17 @@ def side_workloads(dev):
         fc[name + "_gbs"] = round(nbytes / t * 1e-3, 1)
         fc[name + "_frac_hbm"] = round(nbytes / t * 1e-3 / HBM_PEAK_GBS, 4)
         fc[name + "_tops"] = round(2.0 * M * Fin * O / t * 1e-6, 1)
+    # what the weight-gradient launch moves: both operands, the weights in and out, one random integer per weight
+    moved = O * M + M * Fin + 2 * O * Fin + 4 * O * Fin
+    fc["wgrad_moved_bytes"] = moved
+    fc["wgrad_moved_gbs"] = round(moved / fc["wgrad_us"] * 1e-3, 1)
+    fc["wgrad_moved_frac_hbm"] = round(moved / fc["wgrad_us"] * 1e-3 / HBM_PEAK_GBS, 4)
+    # the same three launches with the reference's default rounding (ti_torch.py:459-462: RoundShift for
+    # activations and errors, PstoShift for gradients - no random integers to read)
+    for name, fn in (("fwd_round", lambda: (fsync.zero_(), ops.linear_fwd_requant(A, W, 7, "round", sync=fsync))),
+                     ("dgrad_round", lambda: (fsync.zero_(), ops.linear_dgrad_requant(G, W, 7, "round", sync=fsync))),
+                     ("wgrad_psto", lambda: (fsync.zero_(), ops.linear_wgrad_update(G, A, Wu, 5, "psto", sync=fsync)))):
+        fc[name + "_us"] = round(max(_avg_us(fn) - t_fill, 1e-3), 2)
     # the drop-in int32 products of the extension boundary, operands as the reference hands them over
     # (ti_torch.py:246,259,263: [m,k] and [k,n] row-major, the result the transposed view of an [n,m] buffer)
     from niti_amd.shims import int8mm_cuda

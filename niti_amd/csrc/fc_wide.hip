@@ -578,12 +578,17 @@ __global__ __launch_bounds__(512) void fcw_wgrad_kernel(const FcwArgs a) {
       for (int t = 0; t < T; ++t) acc[t] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa, lds_landed(blo[t], bhi[t]), acc[t], 0, 0, 0);
     }
   }
-  // ---- out of the MFMA layout: lane (o = tid / 16, piece = tid % 16) takes features 64 q + 4 piece .. + 4 (q = 0 .. 3) of
-  // one weight row, so that 16 lanes' random integers are 256 consecutive bytes
+  // ---- out of the MFMA layout: lane (o = tid / 16, piece = tid % 16) takes 16 features of one weight row - with
+  // stochastic rounding features 64 q + 4 piece .. + 4 (q = 0 .. 3), so that 16 lanes' random integers are 256
+  // consecutive bytes; otherwise 16 piece .. + 16, so that a lane moves 16 bytes of weights at once
+  const bool sto = a.method == NITI_ROUND_STOCHASTIC;
   const int lr = lane & 31;
   const int orow = tid >> 4, piece = tid & 15;
   int fin[T][16];
   uint32_t lmax = 0;
+  const int src_off = sto ? (piece >> 3) * (32 * kWgPatchPitch) + orow * kWgPatchPitch + (piece & 7) * 16
+                          : (piece >> 1) * (32 * kWgPatchPitch) + orow * kWgPatchPitch + (piece & 1) * 64;
+  const int src_step = sto ? 2 * 32 * kWgPatchPitch : 16;
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     sync_mem();                                              // tiles (or the previous patch) have been read
@@ -593,10 +598,10 @@ __global__ __launch_bounds__(512) void fcw_wgrad_kernel(const FcwArgs a) {
       *reinterpret_cast<v4i*>(patch + lr * kWgPatchPitch + (8 * g + 4 * lk) * 4) =
           v4i{acc[t][4 * g], acc[t][4 * g + 1], acc[t][4 * g + 2], acc[t][4 * g + 3]};
     __syncthreads();
-    const int8_t* src = act_t + (piece >> 3) * (32 * kWgPatchPitch) + orow * kWgPatchPitch + (piece & 7) * 16;
+    const int8_t* src = act_t + src_off;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const v4i v = *reinterpret_cast<const v4i*>(src + q * (2 * 32 * kWgPatchPitch));
+      const v4i v = *reinterpret_cast<const v4i*>(src + q * src_step);
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         fin[t][4 * q + e] = v[e];
@@ -607,28 +612,54 @@ __global__ __launch_bounds__(512) void fcw_wgrad_kernel(const FcwArgs a) {
   }
   const int shift = grid_shift<8>(a, lmax, words, words + 8);
   const bool trunc = a.trunc != 0;
+  if (sto) {
+#pragma unroll
+    for (int t = 0; t < T; ++t) {
+      const int o = o0 + t * 32 + orow;
+      if (o >= a.O) continue;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int f = f0 + q * 64 + piece * 4;
+        if (f >= a.F) continue;                              // F is a multiple of 16: four features are inside or outside
+        const long long at = static_cast<long long>(o) * a.F + f;
+        const uint32_t wold = *reinterpret_cast<const uint32_t*>(a.w + at);
+        const v4i u = *reinterpret_cast<const v4i*>(a.rand + at);
+        int r[4], wn[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          r[e] = round_any(fin[t][4 * q + e], shift, NITI_ROUND_STOCHASTIC, trunc, u[e]);
+          const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * e)) & 0xFFu));
+          wn[e] = clip127(wo - r[e]);
+        }
+        *reinterpret_cast<uint32_t*>(a.w + at) = pack4_i8(wn[0], wn[1], wn[2], wn[3]);
+        if (a.out8 != nullptr) *reinterpret_cast<uint32_t*>(a.out8 + at) = pack4_i8(r[0], r[1], r[2], r[3]);
+      }
+    }
+    return;
+  }
+  const int f = f0 + piece * 16;
+  if (f >= a.F) return;
 #pragma unroll
   for (int t = 0; t < T; ++t) {
     const int o = o0 + t * 32 + orow;
     if (o >= a.O) continue;
+    const long long at = static_cast<long long>(o) * a.F + f;
+    const v4i wold = *reinterpret_cast<const v4i*>(a.w + at);
+    v4i wnew, g8;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-      const int f = f0 + q * 64 + piece * 4;
-      if (f >= a.F) continue;                                // F is a multiple of 16: four features are inside or outside
-      const long long at = static_cast<long long>(o) * a.F + f;
-      const uint32_t wold = *reinterpret_cast<const uint32_t*>(a.w + at);
-      v4i u = zero;
-      if (a.method == NITI_ROUND_STOCHASTIC) u = *reinterpret_cast<const v4i*>(a.rand + at);
       int r[4], wn[4];
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        r[e] = round_any(fin[t][4 * q + e], shift, a.method, trunc, u[e]);
-        const int wo = static_cast<int>(static_cast<int8_t>((wold >> (8 * e)) & 0xFFu));
+        r[e] = round_any(fin[t][4 * q + e], shift, a.method, trunc, 0);
+        const int wo = static_cast<int>(static_cast<int8_t>((static_cast<uint32_t>(wold[q]) >> (8 * e)) & 0xFFu));
         wn[e] = clip127(wo - r[e]);
       }
-      *reinterpret_cast<uint32_t*>(a.w + at) = pack4_i8(wn[0], wn[1], wn[2], wn[3]);
-      if (a.out8 != nullptr) *reinterpret_cast<uint32_t*>(a.out8 + at) = pack4_i8(r[0], r[1], r[2], r[3]);
+      wnew[q] = static_cast<int>(pack4_i8(wn[0], wn[1], wn[2], wn[3]));
+      g8[q] = static_cast<int>(pack4_i8(r[0], r[1], r[2], r[3]));
     }
+    *reinterpret_cast<v4i*>(a.w + at) = wnew;
+    if (a.out8 != nullptr) *reinterpret_cast<v4i*>(a.out8 + at) = g8;
   }
 }
 
