@@ -303,25 +303,32 @@ __global__ __launch_bounds__(512) void gemm_nn_lines_kernel(const LnArgs g) {
         *reinterpret_cast<const v4i*>(patch + row * kLnPatchPitch + (p16 + 16 * i) * 16);
 }
 
-// c[i] = sum over the parts of the partial results, four elements per thread
-__global__ __launch_bounds__(256) void km_reduce_parts_kernel(const int32_t* __restrict__ part, int32_t* __restrict__ c, long long quads, int parts,
+// c[i] = sum over the parts of the partial results: two elements per thread (the result is small - many short
+// wavefronts cover the device better than few long ones), the loads of eight parts in flight together
+__global__ __launch_bounds__(256) void km_reduce_parts_kernel(const int32_t* __restrict__ part, int32_t* __restrict__ c, long long pairs, int parts,
                                                               int roundtrip, uint32_t* absmax) {
   const long long i = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
   uint32_t lmax = 0;
-  if (i < quads) {
-    v4i s = *reinterpret_cast<const v4i*>(part + 4 * i);
-    for (int p = 1; p < parts; ++p) {
-      const v4i v = *reinterpret_cast<const v4i*>(part + 4 * (static_cast<long long>(p) * quads + i));
+  if (i < pairs) {
+    v2i s = {0, 0};
+    for (int p0 = 0; p0 < parts; p0 += 8) {
+      v2i v[8];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) s[e] += v[e];
+      for (int u = 0; u < 8; ++u) {
+        const int p = p0 + u < parts ? p0 + u : p0;          // a repeated part is not added below
+        v[u] = *reinterpret_cast<const v2i*>(part + 2 * (static_cast<long long>(p) * pairs + i));
+      }
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (p0 + u < parts) s += v[u];
     }
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
+    for (int e = 0; e < 2; ++e) {
       if (roundtrip) s[e] = f32_roundtrip(s[e]);
       const uint32_t u = uabs(s[e]);
       lmax = u > lmax ? u : lmax;
     }
-    *reinterpret_cast<v4i*>(c + 4 * i) = s;
+    *reinterpret_cast<v2i*>(c + 2 * i) = s;
   }
   if (absmax != nullptr) fold_absmax(absmax, lmax);
 }
@@ -424,9 +431,9 @@ int launch_gemm_kmajor(int trans_a, int trans_b, const int8_t* a, const int8_t* 
       LnArgs l{g.a, g.b, p.parts > 1 ? static_cast<int32_t*>(workspace) : c, absmax, g.m, g.n, k, p.chunks_per_part, p.parts, g.roundtrip, g.transposed_out};
       hipLaunchKernelGGL(gemm_nn_lines_kernel, dim3(g.n / 128, (g.m + 31) / 32, p.parts), dim3(512), static_cast<size_t>(kLnLdsBytes), stream, l);
       if (p.parts > 1) {
-        const long long quads = static_cast<long long>(g.m) * g.n / 4;
-        hipLaunchKernelGGL(km_reduce_parts_kernel, dim3(static_cast<unsigned>((quads + 255) / 256)), dim3(256), 0, stream,
-                           static_cast<const int32_t*>(workspace), c, quads, p.parts, g.roundtrip, absmax);
+        const long long pairs = static_cast<long long>(g.m) * g.n / 2;
+        hipLaunchKernelGGL(km_reduce_parts_kernel, dim3(static_cast<unsigned>((pairs + 255) / 256)), dim3(256), 0, stream,
+                           static_cast<const int32_t*>(workspace), c, pairs, p.parts, g.roundtrip, absmax);
       }
       return check_launch("gemm_nn_lines");
     }
