@@ -21,6 +21,7 @@
 
 #include "common.h"
 #include "lds_asm.h"
+#include "nn_lines.h"
 #include "requant_math.h"
 
 namespace niti {
@@ -390,92 +391,25 @@ __global__ __launch_bounds__(512) void fcw_dgrad_kernel(const FcwArgs a) {
 // ---- data gradient, operands through LDS as whole lines -----------------------------------------------------------
 // The kernel above stages 32-byte pieces of the weight rows (a quarter of every line it fetches), takes the error rows
 // in 32-byte pieces as well and stores 4-byte pieces.  Here (F and O multiples of 128) a workgroup owns 128 features x
-// 32 samples: per chunk of 128 reduction steps it stages w[o .. o+128)[f0 .. f0+128) and err[m0 .. m0+32)[o .. o+128) -
-// one whole line per row (buffer_load ... lds, pieces XOR-swizzled by the row) - through a ring of three stages with one
-// barrier per chunk; 8 wavefronts = 4 feature quarters x 2 halves of the chunk; the sums pass through an LDS patch into a
-// row-major arrangement for the rounding.
-constexpr int kDgStage = 128 * 128 + 32 * 128;        // weight chunk + error chunk
-constexpr int kDgLdsBytes = 3 * kDgStage + 32 * 4;
+// 32 samples of dx = err w and runs the whole-line product of nn_lines.h over all of O; the sums pass through an LDS
+// patch into a row-major arrangement for the rounding.
+constexpr int kDgLdsBytes = kLinesLdsBytes + 32 * 4;
 __global__ __launch_bounds__(512) void fcw_dgrad_lds_kernel(const FcwArgs a) {
-  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // 3 stages; later 16 KB of parked sums / the 17 KB patch
-  uint32_t* const words = reinterpret_cast<uint32_t*>(smem + 3 * kDgStage);
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // the stages; later 16 KB of parked sums / the 17 KB patch
+  uint32_t* const words = reinterpret_cast<uint32_t*>(smem + kLinesLdsBytes);
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int f0 = blockIdx.x * 128;
   const int m0 = blockIdx.y * 32;
-  const int nchunks = a.O >> 7;
-  const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(a.w, 0, a.O * a.F, 0x00020000);
-  const __amdgpu_buffer_rsrc_t re = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.err), 0, a.M * a.O, 0x00020000);
-  // staging: 20 instructions per chunk (16 of weight rows, 4 of error rows), wavefront w issues numbers w, w + 8, w + 16
-  const int r8 = lane >> 3, piece = (lane & 7) ^ r8;
-  constexpr int kFar = static_cast<int>(0x80000000u);   // out of range whatever scalar offset is added: zeros
-  const int src0 = (8 * wave + r8) * a.F + f0 + piece * 16;                 // weight rows 8 w ..
-  const int src1 = (8 * (wave + 8) + r8) * a.F + f0 + piece * 16;           // weight rows 64 + 8 w ..
-  // error rows (wavefronts 0 - 3): swizzled by row / 2, since their readers below take 16 bytes of 16 consecutive rows at once
-  const int epiece = (lane & 7) ^ ((4 * (wave & 1) + (r8 >> 1)) & 7);
-  const int src2 = m0 + 8 * wave + r8 < a.M ? (m0 + 8 * wave + r8) * a.O + epiece * 16 : kFar;
-  const unsigned lds0 = lds_addr(smem);
-  auto issue = [&](int c, int st) {
-    const unsigned dst = lds0 + st * kDgStage;
-    const int wo = c * 128 * a.F, eo = c * 128;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst + wave * 1024), 16, src0, wo, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst + (wave + 8) * 1024), 16, src1, wo, 0, 0);
-    if (wave < 4) __builtin_amdgcn_raw_ptr_buffer_load_lds(re, NITI_LDS_AT(dst + 16384 + wave * 1024), 16, src2, eo, 0, 0);
-  };
-  // fragments
   const int ft = wave & 3, kh = wave >> 2;
   const int lr = lane & 31, lk = lane >> 5;
-  const int j = lane & 15, gg = (lane >> 4) & 1;
-  // weight chunk row kh * 64 + s * 32 + lk * 16 + (j >> 1) (+ 8), bytes ft * 32 + gg * 16 + 8 (j & 1) .. + 8
-  const unsigned a_off = static_cast<unsigned>((kh * 64 + lk * 16 + (j >> 1)) * 128 + (((ft * 2 + gg) ^ (j >> 1)) << 4) + 8 * (j & 1));
-  // error chunk row lr, bytes kh * 64 + s * 32 + lk * 16 .. + 16
-  unsigned b_off[2];
-#pragma unroll
-  for (int sstep = 0; sstep < 2; ++sstep) b_off[sstep] = static_cast<unsigned>(16384 + lr * 128 + (((kh * 4 + sstep * 2 + lk) ^ ((lr >> 1) & 7)) << 4));
-  v16i acc;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = 0;
-  issue(0, 0);
-  if (nchunks > 1) issue(1, 1);
-  for (int c = 0; c < nchunks; ++c) {
-    // younger than this chunk's loads: the next chunk's (3 per wavefront 0 - 3, 2 per wavefront 4 - 7)
-    if (c + 1 < nchunks) {
-      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
-      else __builtin_amdgcn_s_waitcnt(0x0F70 | 2);
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-    }
-    sync_mem();   // the chunk has landed for every wavefront, and the stage refilled below has been read by all
-    if (c + 2 < nchunks) issue(c + 2, (c + 2) % 3);
-    const unsigned base = lds0 + (c % 3) * kDgStage;
-    v2i lo[2], hi[2];
-    v4i fb[2];
-#pragma unroll
-    for (int sstep = 0; sstep < 2; ++sstep) {
-      lo[sstep] = lds_read_tr8<0>(base + a_off + sstep * 4096);
-      hi[sstep] = lds_read_tr8<1024>(base + a_off + sstep * 4096);
-      fb[sstep] = lds_read_b128(base + b_off[sstep]);
-    }
-    lds_settle<0>();
-#pragma unroll
-    for (int sstep = 0; sstep < 2; ++sstep) {
-      asm volatile("" : "+v"(fb[sstep]));
-      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lds_landed(lo[sstep], hi[sstep]), fb[sstep], acc, 0, 0, 0);
-    }
-  }
-  sync_mem();   // every wavefront is done with the stages
-  int* const park = reinterpret_cast<int*>(smem) + ft * (16 * 64) + lane;
-  if (kh == 1) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) park[e * 64] = acc[e];
-  }
-  __syncthreads();
+  v16i acc = lines_product(a.err, a.w, a.M, a.F, a.O, m0, f0, 0, a.O >> 7, smem);
+  lines_add_halves(acc, smem);
   uint32_t lmax = 0;
   if (kh == 0) {
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      acc[e] += park[e * 64];
       const uint32_t u = uabs(acc[e]);                 // samples beyond M are sums of zeros
       lmax = u > lmax ? u : lmax;
     }

@@ -14,6 +14,7 @@
 // No operand is copied into another layout and the output is written once.
 #include "common.h"
 #include "lds_asm.h"
+#include "nn_lines.h"
 
 namespace niti {
 namespace {
@@ -168,14 +169,10 @@ __global__ __launch_bounds__(512) void gemm_kmajor_kernel(const KmArgs g) {
 // ---- NN form, both operands through LDS as whole 128-byte lines ------------------------------------------------------
 // The kernel above stages b in 32-byte pieces of its rows and takes a in 32-byte pieces as well; the path from L2 into
 // a compute unit moves such pieces at a quarter of the rate of whole lines.  Here (n and k multiples of 128) a workgroup
-// owns 32 rows x 128 columns of c and a range of the reduction: per chunk of 128 steps it stages b[k .. k+128)[n0 ..
-// n0+128) and a[m0 .. m0+32)[k .. k+128), one whole line per row (buffer_load ... lds, 16-byte pieces XOR-swizzled by
-// the row), through a ring of three stages with one barrier per chunk.  8 wavefronts = 4 column quarters x 2 halves of
-// the chunk.  blockIdx.z splits the reduction when the tiles alone would leave most of the device idle: the parts then
-// write int32 partial results and km_reduce_parts_kernel adds them.
-constexpr int kLnStage = 128 * 128 + 32 * 128;        // b chunk + a chunk
+// owns 32 rows x 128 columns of c and a range of the reduction, and runs the whole-line product of nn_lines.h over it.
+// blockIdx.z splits the reduction when the tiles alone would leave most of the device idle: the parts then write int32
+// partial results and km_reduce_parts_kernel adds them.
 constexpr int kLnPatchPitch = 128 * 4 + 16;
-constexpr int kLnLdsBytes = 3 * kLnStage;
 
 struct LnArgs {
   const int8_t* a;
@@ -190,81 +187,18 @@ struct LnArgs {
 };
 
 __global__ __launch_bounds__(512) void gemm_nn_lines_kernel(const LnArgs g) {
-  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // 3 stages; later 16 KB of parked sums, then the patch
+  extern __shared__ __attribute__((aligned(16))) int8_t smem[];   // the stages; later 16 KB of parked sums, then the patch
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int n0 = blockIdx.x * 128;
   const int m0 = blockIdx.y * 32;
-  const int nchunks_all = g.k >> 7;
   const int c0 = blockIdx.z * g.chunks_per_part;
-  const int nchunks = min(g.chunks_per_part, nchunks_all - c0);
-  const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.b), 0, g.k * g.n, 0x00020000);
-  const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(g.a), 0, g.m * g.k, 0x00020000);
-  // staging: 20 instructions per chunk (16 of b's rows, 4 of a's rows), wavefront w issues numbers w, w + 8, w + 16
-  const int r8 = lane >> 3, piece = (lane & 7) ^ r8;
-  constexpr int kFar = static_cast<int>(0x80000000u);   // out of range whatever scalar offset is added: zeros
-  const int src0 = (8 * wave + r8) * g.n + n0 + piece * 16;
-  const int src1 = (8 * (wave + 8) + r8) * g.n + n0 + piece * 16;
-  // a's rows: swizzled by row / 2, since their readers take 16 bytes of 16 consecutive rows at once
-  const int apiece = (lane & 7) ^ ((4 * (wave & 1) + (r8 >> 1)) & 7);
-  const int src2 = m0 + 8 * wave + r8 < g.m ? (m0 + 8 * wave + r8) * g.k + apiece * 16 : kFar;
-  const unsigned lds0 = lds_addr(smem);
-  auto issue = [&](int c, int st) {
-    const unsigned dst = lds0 + st * kLnStage;
-    const int bo = (c0 + c) * 128 * g.n, ao = (c0 + c) * 128;
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, NITI_LDS_AT(dst + wave * 1024), 16, src0, bo, 0, 0);
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(rb, NITI_LDS_AT(dst + (wave + 8) * 1024), 16, src1, bo, 0, 0);
-    if (wave < 4) __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, NITI_LDS_AT(dst + 16384 + wave * 1024), 16, src2, ao, 0, 0);
-  };
+  const int nchunks = min(g.chunks_per_part, (g.k >> 7) - c0);
   const int ft = wave & 3, kh = wave >> 2;
   const int lr = lane & 31, lk = lane >> 5;
-  const int j = lane & 15, gg = (lane >> 4) & 1;
-  // b chunk row kh * 64 + s * 32 + lk * 16 + (j >> 1) (+ 8), bytes ft * 32 + gg * 16 + 8 (j & 1) .. + 8
-  const unsigned b_off = static_cast<unsigned>((kh * 64 + lk * 16 + (j >> 1)) * 128 + (((ft * 2 + gg) ^ (j >> 1)) << 4) + 8 * (j & 1));
-  // a chunk row lr, bytes kh * 64 + s * 32 + lk * 16 .. + 16
-  unsigned a_off[2];
-#pragma unroll
-  for (int sstep = 0; sstep < 2; ++sstep) a_off[sstep] = static_cast<unsigned>(16384 + lr * 128 + (((kh * 4 + sstep * 2 + lk) ^ ((lr >> 1) & 7)) << 4));
-  v16i acc;
-#pragma unroll
-  for (int e = 0; e < 16; ++e) acc[e] = 0;
-  issue(0, 0);
-  if (nchunks > 1) issue(1, 1);
-  for (int c = 0; c < nchunks; ++c) {
-    // younger than this chunk's loads: the next chunk's (3 per wavefront 0 - 3, 2 per wavefront 4 - 7)
-    if (c + 1 < nchunks) {
-      if (wave < 4) __builtin_amdgcn_s_waitcnt(0x0F70 | 3);
-      else __builtin_amdgcn_s_waitcnt(0x0F70 | 2);
-    } else {
-      __builtin_amdgcn_s_waitcnt(0x0F70);
-    }
-    km_sync();   // the chunk has landed for every wavefront, and the stage refilled below has been read by all
-    if (c + 2 < nchunks) issue(c + 2, (c + 2) % 3);
-    const unsigned base = lds0 + (c % 3) * kLnStage;
-    v2i lo[2], hi[2];
-    v4i fa[2];
-#pragma unroll
-    for (int sstep = 0; sstep < 2; ++sstep) {
-      lo[sstep] = lds_read_tr8<0>(base + b_off + sstep * 4096);
-      hi[sstep] = lds_read_tr8<1024>(base + b_off + sstep * 4096);
-      fa[sstep] = lds_read_b128(base + a_off[sstep]);
-    }
-    lds_settle<0>();
-#pragma unroll
-    for (int sstep = 0; sstep < 2; ++sstep) {
-      asm volatile("" : "+v"(fa[sstep]));
-      // MFMA A = 32 columns of c x 32 reduction steps, B = 32 rows of c x 32 steps
-      acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(lds_landed(lo[sstep], hi[sstep]), fa[sstep], acc, 0, 0, 0);
-    }
-  }
-  km_sync();   // every wavefront is done with the stages
-  int* const park = reinterpret_cast<int*>(smem) + ft * (16 * 64) + lane;
-  if (kh == 1) {
-#pragma unroll
-    for (int e = 0; e < 16; ++e) park[e * 64] = acc[e];
-  }
-  __syncthreads();
+  v16i acc = lines_product(g.a, g.b, g.m, g.n, g.k, m0, n0, c0, nchunks, smem);
+  lines_add_halves(acc, smem);
   // element 4 q + e of a lane is column n0 + ft * 32 + 8 q + 4 (lane / 32) + e of row m0 + lane % 32
   const bool last = g.parts == 1;
   int32_t* const out = g.out + static_cast<long long>(blockIdx.z) * g.m * g.n;
@@ -273,7 +207,7 @@ __global__ __launch_bounds__(512) void gemm_nn_lines_kernel(const LnArgs g) {
     uint32_t lmax = 0;
 #pragma unroll
     for (int e = 0; e < 16; ++e) {
-      int v = acc[e] + park[e * 64];
+      int v = acc[e];
       if (last && g.roundtrip) v = f32_roundtrip(v);
       acc[e] = v;
       const uint32_t u = uabs(v);                         // rows beyond m are sums of zeros
@@ -424,12 +358,12 @@ int launch_gemm_kmajor(int trans_a, int trans_b, const int8_t* a, const int8_t* 
       static bool attr_set[kDeviceSlots] = {};
       bool& done = attr_set[device_slot()];
       if (!done) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nn_lines_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLnLdsBytes) != hipSuccess)
-          return fail(NITI_ERR_LAUNCH, "gemm: cannot reserve %d bytes of LDS", kLnLdsBytes);
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(gemm_nn_lines_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLinesLdsBytes) != hipSuccess)
+          return fail(NITI_ERR_LAUNCH, "gemm: cannot reserve %d bytes of LDS", kLinesLdsBytes);
         done = true;
       }
       LnArgs l{g.a, g.b, p.parts > 1 ? static_cast<int32_t*>(workspace) : c, absmax, g.m, g.n, k, p.chunks_per_part, p.parts, g.roundtrip, g.transposed_out};
-      hipLaunchKernelGGL(gemm_nn_lines_kernel, dim3(g.n / 128, (g.m + 31) / 32, p.parts), dim3(512), static_cast<size_t>(kLnLdsBytes), stream, l);
+      hipLaunchKernelGGL(gemm_nn_lines_kernel, dim3(g.n / 128, (g.m + 31) / 32, p.parts), dim3(512), static_cast<size_t>(kLinesLdsBytes), stream, l);
       if (p.parts > 1) {
         const long long pairs = static_cast<long long>(g.m) * g.n / 2;
         hipLaunchKernelGGL(km_reduce_parts_kernel, dim3(static_cast<unsigned>((pairs + 255) / 256)), dim3(256), 0, stream,
