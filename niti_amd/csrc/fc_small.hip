@@ -17,7 +17,10 @@
 // All of them keep their int32 sums in registers across the tensor-wide range: every workgroup publishes its
 // largest magnitude in a slot of its own and reads all slots (all workgroups resident - checked by the host - and
 // the wait bounded by a wall-clock limit), as the convolution kernels do.
+#include <stdlib.h>
+
 #include "common.h"
+#include "lds_asm.h"
 #include "loss_math.h"
 #include "requant_math.h"
 #include "rng.h"
@@ -80,16 +83,61 @@ __device__ inline uint32_t exchange_range(const FcArgs& a, uint32_t bmax) {
 // ---- forward ------------------------------------------------------------------------------------------
 // One workgroup of 16 wavefronts per tile of 16 samples; wavefront w reduces over features [w * kchunk, (w+1) * kchunk).
 // kHead: dropout on the activations (mask bytes 0x00 / 0xFF in dynamic LDS, F bytes) and the loss gradient.
-template <bool kHead>
+// kLds (F and kchunk multiples of 128): the fragments do not come straight from memory - 64-byte pieces of the rows,
+// which the path from L2 into a compute unit moves at a third of the rate of whole 128-byte lines, and that path is what
+// bounds a workgroup that pulls 26 rows of F bytes - but every wavefront stages its share one line per row at a time
+// (buffer_load ... lds: an instruction moves eight rows' lines, lane -> (row lane / 8, 16-byte piece lane % 8), pieces
+// XOR-swizzled by the row, every instruction's kilobyte 16 bytes further on, so that the fragment reads spread over the
+// banks) in two buffers of its own: no barrier in the loop, the next line on its way while this one multiplies.
+constexpr int kFsInstrBytes = 1024 + 16;
+constexpr int kFsStage = 4 * kFsInstrBytes;            // 16 weight rows + 16 samples, one line each
+constexpr int kFsStagesBytes = 16 * 2 * kFsStage;      // 16 wavefronts x 2 buffers
+template <bool kHead, bool kLds = false>
 __global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
   __shared__ int part[16][256];
   __shared__ __attribute__((aligned(16))) int8_t logits[16][16];   // kHead: the tile's rounded logits
-  extern __shared__ __attribute__((aligned(16))) unsigned char keep[];
+  extern __shared__ __attribute__((aligned(16))) unsigned char keep_base[];   // kLds: the stages come first, then the mask
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int mt = blockIdx.x;
   const bool drop = kHead && a.dropout != 0;
   const bool draws = kHead && (a.dropout == 2 || (a.target != nullptr && a.loss_rand == nullptr));
+  unsigned char* const keep = kLds ? keep_base + kFsStagesBytes : keep_base;
+  // kLds: the first line is requested before anything else, so that it travels while the mask is made
+  const int k0 = wave * a.kchunk;
+  [[maybe_unused]] int nlines = 0;
+  [[maybe_unused]] int src[4] = {0, 0, 0, 0};
+  [[maybe_unused]] unsigned stage0 = 0;
+  [[maybe_unused]] const __amdgpu_buffer_rsrc_t rw = __builtin_amdgcn_make_buffer_rsrc(a.w, 0, a.O * a.F, 0x00020000);
+  [[maybe_unused]] const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<int8_t*>(a.act), 0, a.M * a.F, 0x00020000);
+  auto issue = [&](int line, int buf) {
+    const int kb = k0 + line * 128;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const unsigned dst = stage0 + buf * kFsStage + j * kFsInstrBytes;
+      if (j < 2) __builtin_amdgcn_raw_ptr_buffer_load_lds(rw, NITI_LDS_AT(dst), 16, src[j], kb, 0, 0);
+      else __builtin_amdgcn_raw_ptr_buffer_load_lds(ra, NITI_LDS_AT(dst), 16, src[j], kb, 0, 0);
+    }
+  };
+  if constexpr (kLds) {
+    nlines = k0 < a.F ? (min(k0 + a.kchunk, a.F) - k0) >> 7 : 0;
+    const int r8 = lane >> 3, piece = (lane & 7) ^ r8;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                      // instruction j: rows 8 j .. 8 j + 7 of the panel (16 weight rows, 16 samples)
+      const int prow = 8 * j + r8;
+      const int g = prow < 16 ? prow : mt * 16 + prow - 16;
+      const bool in = prow < 16 ? g < a.O : g < a.M;
+      src[j] = in ? g * a.F + piece * 16 : static_cast<int>(0x80000000u);   // out of range whatever scalar offset is added: zeros
+    }
+    stage0 = lds_addr(keep_base) + wave * (2 * kFsStage);
+    if (nlines > 0) issue(0, 0);
+  }
+  // the sample's target class is wanted at the very end, behind a chain of waits: requested now
+  long long target_of_row = -1;
+  if (kHead && a.target != nullptr && wave < 4) {
+    const int trow = mt * 16 + wave * 4 + (lane >> 4);
+    if (trow < a.M) target_of_row = a.target[trow];
+  }
   RngDraw draw{};
   if (draws) draw = rng_read(a.rng);
   if (drop) {
@@ -117,13 +165,47 @@ __global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
   }
   const int row = lane & 15, kg = lane >> 4;           // operand row (sample / output feature), 16-byte piece of a 64-step
   const int m = mt * 16 + row;
-  const int k0 = wave * a.kchunk;
   const int k1 = min(k0 + a.kchunk, a.F);
   const int8_t* pa = a.act + static_cast<long long>(m) * a.F;
   const int8_t* pw = a.w + static_cast<long long>(row) * a.F;
   const bool va = m < a.M, vw = row < a.O;
   v4i acc = {0, 0, 0, 0};
   const v4i zero = {0, 0, 0, 0};
+  if constexpr (kLds) {
+    // fragments: lane (row, kg) of 64-step s reads piece 4 s + kg of its row's line
+    const unsigned frow = (row >> 3) * kFsInstrBytes + (row & 7) * 128;
+    unsigned fpiece[2];
+#pragma unroll
+    for (int sstep = 0; sstep < 2; ++sstep) fpiece[sstep] = static_cast<unsigned>(((4 * sstep + kg) ^ (row & 7)) * 16);
+    const unsigned keep0 = lds_addr(keep) + k0 + kg * 16;
+    for (int line = 0; line < nlines; ++line) {
+      const int buf = line & 1;
+      if (line + 1 < nlines) {
+        issue(line + 1, buf ^ 1);
+        __builtin_amdgcn_s_waitcnt(0x0F70 | 4);                      // vmcnt(4): this line has landed, the next one is on its way
+      } else {
+        __builtin_amdgcn_s_waitcnt(0x0F70);                          // vmcnt(0)
+      }
+      const unsigned base = stage0 + buf * kFsStage + frow;
+      v4i fw[2], fa[2], fk[2];
+#pragma unroll
+      for (int sstep = 0; sstep < 2; ++sstep) {
+        fw[sstep] = lds_read_b128(base + fpiece[sstep]);
+        fa[sstep] = lds_read_b128(base + 2 * kFsInstrBytes + fpiece[sstep]);
+        if (drop) fk[sstep] = lds_read_b128(keep0 + line * 128 + sstep * 64);
+      }
+      lds_settle<0>();
+#pragma unroll
+      for (int sstep = 0; sstep < 2; ++sstep) {
+        asm volatile("" : "+v"(fw[sstep]), "+v"(fa[sstep]));
+        if (drop) {
+          asm volatile("" : "+v"(fk[sstep]));
+          fa[sstep] &= fk[sstep];
+        }
+        acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(fa[sstep], fw[sstep], acc, 0, 0, 0);
+      }
+    }
+  } else
   for (int kb = k0; kb < k1; kb += 256) {                 // four 64-steps at a time, their loads in flight together
     v4i fa[4], fw[4];
 #pragma unroll
@@ -208,7 +290,7 @@ __global__ __launch_bounds__(1024) void fc_fwd_requant_kernel(const FcArgs a) {
       float g = nm * 2048.0f / fsum;
       const long long tsum = group_sum(valid ? static_cast<long long>(g) : 0LL);   // ti_loss.py:34
       if (valid) {
-        if (j == a.target[row]) g = g - static_cast<float>(tsum);
+        if (j == target_of_row) g = g - static_cast<float>(tsum);
         const int x = static_cast<int>(g);   // .type(torch.int32)
         const long long idx = static_cast<long long>(row) * a.O + j;
         const int u = a.loss_rand != nullptr ? a.loss_rand[idx] & 15 : static_cast<int>(rng_word(draw, kRngStreamLoss, static_cast<uint32_t>(idx)) & 15u);
@@ -671,6 +753,29 @@ int resident_blocks(const void* kernel, int threads = 256) {
 // forward: reduction elements per wavefront (a multiple of 256), sixteen wavefronts per 16-sample tile
 int fwd_chunk(int F) { return ((F + 15) / 16 + 255) / 256 * 256; }
 
+// The forward kernel's LDS-staged form: taken when F is a multiple of 128, its stages (and the dropout mask) fit beside
+// the kernel's static LDS and one workgroup per compute unit covers the grid.  NITI_FC_LDS=0 pins the other form.
+template <bool kHead>
+bool fwd_lds_ok(int F, long long nb, size_t mask_bytes, size_t* lds) {
+  *lds = static_cast<size_t>(kFsStagesBytes) + mask_bytes;
+  const char* e = getenv("NITI_FC_LDS");
+  if ((e != nullptr && e[0] == '0') || F % 128 != 0 || *lds + 16384 + 256 + 64 > 160 * 1024) return false;
+  static int resident_of[kDeviceSlots] = {};
+  int& resident = resident_of[device_slot()];
+  if (resident == 0) {
+    // counted with the largest allocation the kernel takes, so the answer holds for every call
+    constexpr int kMost = 160 * 1024 - 16384 - 256 - 64;
+    int dev = 0, cus = 0, per_cu = 0;
+    const void* k = reinterpret_cast<const void*>(fc_fwd_requant_kernel<kHead, true>);
+    if (hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, kMost) == hipSuccess && hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+        hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k, 1024, kMost) == hipSuccess)
+      resident = cus * per_cu;
+    if (resident == 0) resident = -1;
+  }
+  return nb <= resident;
+}
+
 long long blocks_of(int which, int M, int O, int F) {
   if (M <= 0 || O <= 0 || F <= 0 || O > kMaxOut) return 0;
   if (which == NITI_FC_FORWARD) {
@@ -754,7 +859,11 @@ extern "C" int niti_fc_i8_fwd_requant(const int8_t* act, const int8_t* w, int8_t
   if (resident == 0) resident = resident_blocks(reinterpret_cast<const void*>(fc_fwd_requant_kernel<false>), 1024);
   if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "fc_fwd_requant: %lld workgroups do not fit on the device at once (%d)", nb, resident);
   a.kchunk = fwd_chunk(F);
-  hipLaunchKernelGGL(fc_fwd_requant_kernel<false>, dim3(static_cast<unsigned>(nb)), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
+  size_t lds_staged = 0;
+  if (fwd_lds_ok<false>(F, nb, 0, &lds_staged))
+    hipLaunchKernelGGL((fc_fwd_requant_kernel<false, true>), dim3(static_cast<unsigned>(nb)), dim3(1024), lds_staged, static_cast<hipStream_t>(stream), a);
+  else
+    hipLaunchKernelGGL((fc_fwd_requant_kernel<false, false>), dim3(static_cast<unsigned>(nb)), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
   return check_launch("fc_fwd_requant");
 }
 
@@ -861,7 +970,11 @@ extern "C" int niti_head_i8_forward(const int8_t* act, const int8_t* w, int8_t* 
   }
   if (nb > resident) return fail(NITI_ERR_UNSUPPORTED, "head_forward: %lld workgroups do not fit on the device at once (%d)", nb, resident);
   a.kchunk = fwd_chunk(F);
-  hipLaunchKernelGGL(fc_fwd_requant_kernel<true>, dim3(static_cast<unsigned>(nb)), dim3(1024), lds, static_cast<hipStream_t>(stream), a);
+  size_t lds_staged = 0;
+  if (fwd_lds_ok<true>(F, nb, lds, &lds_staged))
+    hipLaunchKernelGGL((fc_fwd_requant_kernel<true, true>), dim3(static_cast<unsigned>(nb)), dim3(1024), lds_staged, static_cast<hipStream_t>(stream), a);
+  else
+    hipLaunchKernelGGL((fc_fwd_requant_kernel<true, false>), dim3(static_cast<unsigned>(nb)), dim3(1024), lds, static_cast<hipStream_t>(stream), a);
   return check_launch("head_forward");
 }
 
