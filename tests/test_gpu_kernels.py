@@ -577,7 +577,8 @@ def test_conv_wgrad_update(dev, case, div_mode, launches, monkeypatch):
             assert torch.equal(wp.cpu(), ops.conv_filter_prepare(w16_ref, N, Q, Q).cpu())
 
 
-@pytest.mark.parametrize("case", [(128, 10, 8192), (5, 3, 64), (33, 16, 272), (512, 10, 1024), (1, 1, 16), (100, 7, 4000)])
+@pytest.mark.parametrize("case", [(128, 10, 8192), (5, 3, 64), (33, 16, 272), (512, 10, 1024), (1, 1, 16), (100, 7, 4000), (37, 10, 384),
+                                  (48, 16, 128)])
 @pytest.mark.parametrize("div_mode", ["floor", "trunc"])
 def test_fc_few_outputs(dev, case, div_mode):
     """TiLinear's three passes as one launch each (few output features) against GEMM + requantisation of the oracle."""
