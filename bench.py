@@ -376,14 +376,21 @@ def mfma_probe(dev):
     rnd = torch.randint(-127, 128, (1 << 20,), generator=g, dtype=torch.int8).to(dev)
     zero = torch.zeros(1 << 20, dtype=torch.int8, device=dev)
     ops.mfma_probe(const)                              # clocks up
-    zt, zg = ops.mfma_probe(zero)
-    ct, cg = ops.mfma_probe(const)
-    rt, rg = ops.mfma_probe(rnd)
+    # one workgroup (8 wavefronts) per compute unit: two wavefronts per SIMD, each issuing its run of products back to
+    # back.  With two workgroups per compute unit the same loop reaches two thirds of this (four wavefronts of equal
+    # priority take turns on a SIMD's matrix unit, and the changes of wavefront cost it idle clocks).
+    one = dict(workgroups=256, iters=2400)
+    zt, zg = ops.mfma_probe(zero, **one)
+    ct, cg = ops.mfma_probe(const, **one)
+    rt, rg = ops.mfma_probe(rnd, **one)
+    rt2, rg2 = ops.mfma_probe(rnd)
     return {"zero_operands_tops": round(zt, 1), "zero_operands_clock_ghz": round(zg, 2),
             "constant_operands_tops": round(ct, 1), "constant_operands_clock_ghz": round(cg, 2),
             "random_operands_tops": round(rt, 1), "random_operands_clock_ghz": round(rg, 2),
-            "note": "512 workgroups x 8 wavefronts x 1200 x 12 v_mfma_i32_32x32x32_i8 on register operands; clock = shader "
-                    "cycle counter against the 100 MHz wall clock inside the loop"}
+            "random_operands_two_workgroups_per_cu_tops": round(rt2, 1), "random_operands_two_workgroups_per_cu_clock_ghz": round(rg2, 2),
+            "note": "256 workgroups (one per compute unit) x 8 wavefronts x 2400 x 12 v_mfma_i32_32x32x32_i8 on register operands; "
+                    "clock = shader cycle counter against the 100 MHz wall clock inside the loop; the last pair is the same loop "
+                    "with 512 workgroups x 1200"}
 
 
 def side_workloads(dev):
