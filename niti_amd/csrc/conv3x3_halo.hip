@@ -371,7 +371,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       for (int e = 0; e < 16; ++e) acc[i][j][e] = 0;
 
   // one filter row: 12 (6) MFMAs from the activation tile sa and the three taps at sw
-  auto filter_row = [&](const int8_t* sa, const int8_t* sw, int r) {
+  auto filter_row = [&](const int8_t* sa, const int8_t* sw, int r, auto&& behind_first_tap) {
     const int roff = r * G::RP * 32;
     // pixels under the centre column of this filter row; the fragment layout is lane -> (pixel lane % 32,
     // 16 channels lane / 32), so the pixel to the left is one lane down and the one to the right one lane up
@@ -422,6 +422,9 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
     for (int i = 0; i < NWF; ++i)
 #pragma unroll
       for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[0][i], pc[j], acc[i][j], 0, 0, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    behind_first_tap();
+    __builtin_amdgcn_sched_barrier(0);
     v4i ps[PT];
 #pragma unroll
     for (int j = 0; j < PT; ++j)
@@ -445,7 +448,7 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
   // are inline assembly and run one filter row ahead of the products: row r + 1 is requested, then the wait leaves
   // exactly those requests in flight, then row r multiplies - so only the first row of a stage waits for LDS.  (Left
   // to itself the compiler keeps the fragments in few registers and alternates read, wait, product.)
-  auto stage_rows = [&](unsigned saa, unsigned swa) {
+  auto stage_rows = [&](unsigned saa, unsigned swa, auto&& behind_first_row) {
     constexpr int PER_TAP = NWF * (kWT ? 2 : 1);
     constexpr int ROW_READS = PT + 3 * PER_TAP;
     static_assert(ROW_READS <= 15, "the wait counter holds 15");
@@ -514,6 +517,10 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
 #pragma unroll
         for (int j = 0; j < PT; ++j) acc[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wf[2][i], ps[j], acc[i][j], 0, 0, 0);
       __builtin_amdgcn_sched_barrier(0);   // the next row's requests and wait stay behind these products
+      if constexpr (r == 0) {
+        behind_first_row();
+        __builtin_amdgcn_sched_barrier(0);
+      }
     });
   };
 
@@ -542,12 +549,14 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
           hc_wait_vmcnt_pair<WL + G::ACT_LOADS>(wfull);
         }
         hc_sync();
-        if (t + 2 < nst) {
-          const int c2 = r == 0 ? ci : ci + 1, r2 = r == 0 ? 2 : r - 1;
-          issue_w(c2, r2, (t + 2) % G::WSTAGES);
-        }
-        if (r == 0 && more) issue_act(ci + 1, (ci + 1) & 1);
-        filter_row(sa, w_buf + (t % G::WSTAGES) * G::W_BYTES, r);
+        // the next loads go out behind the first tap's products (see the other pipeline below)
+        filter_row(sa, w_buf + (t % G::WSTAGES) * G::W_BYTES, r, [&] {
+          if (t + 2 < nst) {
+            const int c2 = r == 0 ? ci : ci + 1, r2 = r == 0 ? 2 : r - 1;
+            issue_w(c2, r2, (t + 2) % G::WSTAGES);
+          }
+          if (r == 0 && more) issue_act(ci + 1, (ci + 1) & 1);
+        });
       }
     }
   } else {
@@ -561,10 +570,15 @@ __global__ __launch_bounds__(512, 4) void conv3x3_halo_kernel(const HaloArgs a) 
       else
         hc_wait_vmcnt<0>();
       hc_sync();
-      if (ci + 1 < a.cslices) issue_act(ci + 1, (ci + 1) & 1);
-      if (ci + 2 < a.cslices) issue_w(ci + 2, 0, (ci + 2) % G::WSTAGES);
+      // The next loads go out behind the first filter row's products, not right behind the barrier: a wavefront
+      // issues in order, the memory pipeline takes a few hundred clocks to accept a stage's load instructions (32-byte
+      // pieces: 32 requests each), and right behind the barrier all eight wavefronts would spend them at the same
+      // time with nothing queued on the matrix units.
       const int8_t* sw = w_buf + (ci % G::WSTAGES) * G::W_BYTES;
-      stage_rows(lds_addr(sa), lds_addr(sw));
+      stage_rows(lds_addr(sa), lds_addr(sw), [&] {
+        if (ci + 1 < a.cslices) issue_act(ci + 1, (ci + 1) & 1);
+        if (ci + 2 < a.cslices) issue_w(ci + 2, 0, (ci + 2) % G::WSTAGES);
+      });
     }
   }
 
