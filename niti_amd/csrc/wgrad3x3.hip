@@ -84,8 +84,11 @@ __device__ inline WorkItem die_local_work_item() {
 // sum_q err[q] act[q+s-1] = sum_q' err[q'-s+1] act[q'] -, once per reduction step for all three filter rows (8 byte
 // shifts instead of 24 per nine MFMAs), and every filter row reads one aligned activation fragment (b_base then names
 // the pixels themselves, halo column + 1): 8 instead of 11 LDS reads.
-template <int Q, int BR, int HR, int ROWB, bool kShiftTaps, int NB, bool kShiftErr = false, int KS = 4>
-__device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const int (&b_base)[NB], v16i (&acc)[9]) {
+// behind_first: run once behind the first step's products - the caller's load instructions for a later stage.  A
+// wavefront issues in order and the memory pipeline takes a few hundred clocks to accept a stage's loads; right behind
+// the stage barrier all eight wavefronts would spend them at the same time with nothing queued on the matrix units.
+template <int Q, int BR, int HR, int ROWB, bool kShiftTaps, int NB, bool kShiftErr = false, int KS = 4, class F>
+__device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const int (&b_base)[NB], v16i (&acc)[9], F&& behind_first) {
   v2i alo[2], ahi[2];   // [reduction step & 1]
   v2i rd[2][NB];        // [row step & 1]
   v4i af[2];
@@ -149,6 +152,10 @@ __device__ inline void wgrad_stage(unsigned sbase, const int (&a_base)[2], const
       }
     }
     __builtin_amdgcn_sched_barrier(0);   // the next row's requests and wait stay behind these products
+    if constexpr (step == 0) {
+      behind_first();
+      __builtin_amdgcn_sched_barrier(0);
+    }
   });
 }
 
@@ -298,8 +305,9 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_kernel(const WgradArgs a) {
     if (it + STAGES - 2 < nb) wg_wait_vmcnt<(STAGES - 2) * G::NL>();
     else wg_wait_vmcnt<0>();
     wg_sync();
-    if (it + STAGES - 1 < nb) issue(band_begin + it + STAGES - 1, (it + STAGES - 1) % STAGES);
-    wgrad_stage<Q, BR, G::HR, G::RP * 64, true, NB>(lds_addr(smem + (it % STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
+    wgrad_stage<Q, BR, G::HR, G::RP * 64, true, NB>(lds_addr(smem + (it % STAGES) * G::STAGE_BYTES), a_base, b_base, acc, [&] {
+      if (it + STAGES - 1 < nb) issue(band_begin + it + STAGES - 1, (it + STAGES - 1) % STAGES);
+    });
   }
 
   // ---- partial sums: acc[t][4g+e] = dw[k0+wk*32+8g+4*lk+e][tap t][c0+wc*32+(lane&31)]
@@ -805,8 +813,9 @@ __global__ __launch_bounds__(512, 1) void wgrad3x3_narrow_kernel(const WgradArgs
     if (it + G::STAGES - 2 < nb) wg_wait_vmcnt<(G::STAGES - 2) * G::NL>();
     else wg_wait_vmcnt<0>();
     wg_sync();
-    if (it + G::STAGES - 1 < nb) issue(band_begin + it + G::STAGES - 1, (it + G::STAGES - 1) % G::STAGES);
-    wgrad_stage<Q, BR, G::HR, G::RP * 32, kShiftTaps, NB, kShiftErr, kHalfK ? 2 : 4>(lds_addr(smem + (it % G::STAGES) * G::STAGE_BYTES), a_base, b_base, acc);
+    wgrad_stage<Q, BR, G::HR, G::RP * 32, kShiftTaps, NB, kShiftErr, kHalfK ? 2 : 4>(
+        lds_addr(smem + (it % G::STAGES) * G::STAGE_BYTES), a_base, b_base, acc,
+        [&] { if (it + G::STAGES - 1 < nb) issue(band_begin + it + G::STAGES - 1, (it + G::STAGES - 1) % G::STAGES); });
   }
 
   // ---- add the two pixel halves: half 1 -> LDS -> half 0 -> memory.  Slot layout [value][lane].
