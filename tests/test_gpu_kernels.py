@@ -1117,3 +1117,50 @@ def test_conv_dgrad_requant_unpool(dev, case):
         y, sh, _ = ops.conv2d_dgrad_requant(ed, wd, 1, 1, method=method, relu_mask=pd, unpool=(xd, "first"),
                                             forward_filter=ops.conv_filter_prepare(wd, N, Q, Q), shift_out=so, shift_hint=True)
         assert int(so.cpu()) == sh_ref and torch.equal(y.cpu(), co.maxpool_bwd(pooled, dx, pool_in, 2, 2, 0, "first")), method
+
+
+@pytest.mark.parametrize("seed", [11, 12, 13])
+def test_whole_line_kernels_on_drawn_shapes(dev, seed):
+    """The kernels that stage whole 128-byte lines (int32 GEMM with a slow reduction index in both storage forms, TiLinear
+    forward and data gradient) on shapes drawn per seed: row counts that leave ragged tiles, one to a dozen chunks of the
+    reduction (so the split over workgroups comes out even, uneven and absent), against the oracle's int8mm and
+    act_calc / err_calc."""
+    import random
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    rnd = random.Random(seed)
+    g = torch.Generator().manual_seed(7000 + seed)
+    for _ in range(4):
+        m = rnd.choice([1, 7, 31, 33, 64, 100, 128, 200, 257])
+        n, k = 128 * rnd.randint(1, 6), 128 * rnd.randint(1, 12)
+        _say("whole_line gemm", seed, m, n, k)
+        A, B = ri8(g, m, k), ri8(g, k, n)
+        ref = po.int8mm(A, B)
+        am = ops.new_scalar_u32(dev)
+        assert torch.equal(ops.gemm(A.to(dev), B.to(dev), False, False, absmax=am).cpu(), ref)
+        assert int(am.cpu()) == po.absmax(ref)
+        am = ops.new_scalar_u32(dev)
+        assert torch.equal(ops.gemm(B.to(dev), A.to(dev), True, True, absmax=am).cpu(), ref.t().contiguous())   # [n,m] = B^T A^T
+        assert int(am.cpu()) == po.absmax(ref)
+    for _ in range(3):
+        M = rnd.choice([1, 5, 16, 31, 33, 64, 100, 160])
+        Fi, O = 128 * rnd.randint(1, 8), 128 * rnd.randint(1, 6)
+        _say("whole_line linear", seed, M, Fi, O)
+        act, w, err = ri8(g, M, Fi), ri8(g, O, Fi), ri8(g, M, O, lo=-60, hi=60)
+        for method in ("round", "sto"):
+            ud = torch.randint(0, 1 << 24, (M, Fi), generator=g, dtype=torch.int32)
+            uf = torch.randint(0, 1 << 24, (M, O), generator=g, dtype=torch.int32)
+
+            def low(u, acc):
+                s = max(po.bitwidth_int(po.absmax(acc)) - 7, 0)
+                return u & ((1 << s) - 1) if s > 0 else torch.zeros_like(u)
+            sto = method == "sto"
+            assert ops.linear_sync_words("dgrad", M, O, Fi) and ops.linear_sync_words("forward", M, O, Fi)
+            acc = po.int8mm(err, w)
+            ref, sh = po.err_calc(acc, method, "floor", rand=low(ud, acc) if sto else None)
+            y, s2, sync = ops.linear_dgrad_requant(err.to(dev), w.to(dev), 7, method, "floor", rand=ud.to(dev) if sto else None)
+            assert torch.equal(y.cpu(), ref) and int(s2.cpu()) == sh and int(sync.cpu()[1]) == 0, (M, Fi, O, method)
+            acc = po.int8mm(act, w.t().contiguous())
+            ref, _ = po.act_calc(acc, 0, method, "floor", rand=low(uf, acc) if sto else None)
+            y, _, sync = ops.linear_fwd_requant(act.to(dev), w.to(dev), 7, method, "floor", rand=uf.to(dev) if sto else None)
+            assert torch.equal(y.cpu(), ref) and int(sync.cpu()[1]) == 0, (M, Fi, O, method)
