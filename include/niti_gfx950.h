@@ -477,6 +477,19 @@ int niti_head_i8_backward(const int8_t* err, const int8_t* act, const int8_t* dr
                           uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out, int32_t* grad_shift_out,
                           const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act, int exp_act_bias,
                           int32_t* err_exp_out, int32_t* grad_exp_out, void* stream);
+/*
+ * niti_head_i8_backward with the backward pass of the 2 x 2 / stride-2 max-pool whose flattened output act is
+ * (ti_vgg.py:33-37: TiMaxpool2d, TiFlat in front of the classifier; ti_torch.py:302-316, int8pool_kernel.cu:84-138):
+ * act [M][P][Q][C] = maxpool(pool_in [M][2P][2Q][C]), F = P Q C, C a multiple of 64.  unpooled [M][2P][2Q][C] receives
+ * what niti_maxpool_i8_bwd(act, dx8, pool_in, ...) would write, pool_flags = NITI_TIES_FIRST / NITI_TIES_ALL, optionally
+ * | NITI_POOL_BWD_RELU.  dx8 may be null here (only the routed gradient is wanted).
+ */
+int niti_head_i8_backward_unpool(const int8_t* err, const int8_t* act, const int8_t* drop_mask, int8_t* w, int8_t* dx8, int M,
+                                 int O, int F, int err_bits, int err_method, int grad_bits, int grad_method, int div_mode,
+                                 int bw_mode, uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out,
+                                 int32_t* grad_shift_out, const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act,
+                                 int exp_act_bias, int32_t* err_exp_out, int32_t* grad_exp_out, const int8_t* pool_in,
+                                 int8_t* unpooled, int P, int Q, int C, int pool_flags, void* stream);
 
 /*
  * Grouped int8 convolution with float32 output, replaces int8conv_cuda.group_conv

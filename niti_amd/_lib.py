@@ -81,6 +81,8 @@ SIGNATURES = {
                                   _vp, _vp, _vp, _vp, _vp]),
     "niti_head_i8_backward": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp,
                                    _vp, _vp, _vp, _i, _vp, _vp, _vp]),
+    "niti_head_i8_backward_unpool": (_i, [_vp, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _i, _i, _vp, _sz, _vp, _vp, _vp,
+                                   _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _vp]),
     "niti_mfma_probe_i8": (_i, [_vp, _sz, _i, _i, _vp, _vp, _vp]),
     "niti_group_conv_i8_f32": (_i, [_vp, _vp, _vp] + [_i] * 12 + [_vp]),
 }

@@ -522,6 +522,11 @@ struct HeadBwdArgs {
   int exp_act_bias;
   int32_t* err_exp_out;
   int32_t* grad_exp_out;
+  // backward pass of the 2 x 2 max-pool whose flattened output act is ([M][P][Q][C], F = P Q C, C a multiple of 64)
+  const int8_t* pool_in;   // [M][2P][2Q][C], or null
+  int8_t* unpooled;        // [M][2P][2Q][C]
+  int pool_q, pool_c;
+  int pool_ties_all, pool_relu;
 };
 
 __device__ inline int byte_of(uint32_t w, int b) { return static_cast<int>(static_cast<int8_t>((w >> (8 * b)) & 0xFFu)); }
@@ -574,7 +579,7 @@ __device__ inline void wait_slot_pairs(uint32_t* slots, int nb, long long spin_l
   max_hi = wave_max_u32(ghi);
 }
 
-__global__ __launch_bounds__(1024) void fc_head_bwd_kernel(const HeadBwdArgs a) {
+__global__ __launch_bounds__(1024, 8) void fc_head_bwd_kernel(const HeadBwdArgs a) {
   // both products run on v_mfma_i32_16x16x64_i8, whose operands are rows with the reduction index in consecutive bytes
   __shared__ __attribute__((aligned(16))) uint32_t err_s[kHeadMaxM * 4];               // [m][o]: 16 bytes per sample
   __shared__ __attribute__((aligned(16))) uint32_t err_t[kMaxOut * kHeadGroups];       // [o][m]
@@ -713,6 +718,21 @@ __global__ __launch_bounds__(1024) void fc_head_bwd_kernel(const HeadBwdArgs a) 
     if (a.err_exp_out != nullptr) *a.err_exp_out = e_err;
     if (a.grad_exp_out != nullptr) *a.grad_exp_out = sw + e_err + (a.exp_act != nullptr ? *a.exp_act : 0) + a.exp_act_bias;   // ti_torch.py:18
   }
+  // the pool window of this thread's (sample, 16 channels) is requested here, ahead of the rounding and the stores of the
+  // two gradients (any earlier and the kernel needs more registers than let two workgroups share a compute unit)
+  const bool unpool = a.pool_in != nullptr && t < a.M * 4;
+  long long px0 = 0, prowb = 0;
+  v4i py = zero, px[4] = {zero, zero, zero, zero};
+  if (unpool) {
+    const int m = t >> 2, piece = t & 3;
+    const int pp = f0 / a.pool_c, c = f0 - pp * a.pool_c + piece * 16;
+    const int ph = pp / a.pool_q, pw = pp - ph * a.pool_q;
+    prowb = static_cast<long long>(2 * a.pool_q) * a.pool_c;
+    px0 = ((static_cast<long long>(m) * 2 * (a.F / (a.pool_q * a.pool_c)) + 2 * ph) * 2 * a.pool_q + 2 * pw) * a.pool_c + c;
+    py = *reinterpret_cast<const v4i*>(a.act + static_cast<long long>(m) * a.F + f0 + piece * 16);
+    px[0] = *reinterpret_cast<const v4i*>(a.pool_in + px0);
+    px[1] = *reinterpret_cast<const v4i*>(a.pool_in + px0 + a.pool_c);
+  }
   const bool trunc = a.trunc != 0;
   const bool psto_d = a.err_method == NITI_ROUND_PSEUDO_STOCHASTIC, psto_w = a.grad_method == NITI_ROUND_PSEUDO_STOCHASTIC;
   {
@@ -722,7 +742,9 @@ __global__ __launch_bounds__(1024) void fc_head_bwd_kernel(const HeadBwdArgs a) 
       for (int blk = 0; blk < 4; ++blk) {
         const uint32_t r4 = pack4_i8(round_to_i8(dacc[blk][0], shift_d, psto_d, trunc), round_to_i8(dacc[blk][1], shift_d, psto_d, trunc),
                                      round_to_i8(dacc[blk][2], shift_d, psto_d, trunc), round_to_i8(dacc[blk][3], shift_d, psto_d, trunc));
-        *reinterpret_cast<uint32_t*>(a.dx8 + static_cast<long long>(m) * a.F + f0 + 16 * blk + 4 * kg) = r4 & keep_s[4 * blk + kg];   // ti_torch.py:454
+        const uint32_t kept = r4 & keep_s[4 * blk + kg];   // ti_torch.py:454
+        if (a.dx8 != nullptr) *reinterpret_cast<uint32_t*>(a.dx8 + static_cast<long long>(m) * a.F + f0 + 16 * blk + 4 * kg) = kept;
+        if (a.pool_in != nullptr) act_t[m * (kHeadSlab / 4) + 4 * blk + kg] = kept;   // [m][64 bytes]: the transposed activations are done with
       }
     }
   }
@@ -739,6 +761,37 @@ __global__ __launch_bounds__(1024) void fc_head_bwd_kernel(const HeadBwdArgs a) 
         if (a.g8 != nullptr) a.g8[at] = static_cast<int8_t>(r);
       }
     }
+  }
+  if (a.pool_in == nullptr) return;
+  // ---- the max-pool's backward pass for the slab (64 channels of one pooled pixel): thread (sample, 16 channels)
+  // routes its 16 gradients to the window positions that hold the maximum (int8pool_kernel.cu:84-138; the first in scan
+  // order, or all of them), zeroed where the pool's input is not positive when the ReLU in front leaves that to it
+  __syncthreads();
+  if (unpool) {
+    const int m = t >> 2, piece = t & 3;
+    const long long x0 = px0, rowb = prowb;
+    const v4i y = py;
+    const v4i d = *reinterpret_cast<const v4i*>(act_t + m * (kHeadSlab / 4) + piece * 4);
+    px[2] = *reinterpret_cast<const v4i*>(a.pool_in + px0 + prowb);   // the window's second row: requested late, for want of registers
+    px[3] = *reinterpret_cast<const v4i*>(a.pool_in + px0 + prowb + a.pool_c);
+    const v4i (&x)[4] = px;
+    v4i o[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      uint32_t taken = 0;   // bytes whose gradient an earlier position of the window (scan order) already received
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const uint32_t eq = equal_bytes(static_cast<uint32_t>(x[k][e]), static_cast<uint32_t>(y[e]));
+        uint32_t keep = a.pool_ties_all ? eq : eq & ~taken;
+        if (a.pool_relu) keep &= positive_bytes(static_cast<uint32_t>(x[k][e]));
+        o[k][e] = static_cast<int>(static_cast<uint32_t>(d[e]) & keep);
+        taken |= eq;
+      }
+    }
+    *reinterpret_cast<v4i*>(a.unpooled + x0) = o[0];
+    *reinterpret_cast<v4i*>(a.unpooled + x0 + a.pool_c) = o[1];
+    *reinterpret_cast<v4i*>(a.unpooled + x0 + rowb) = o[2];
+    *reinterpret_cast<v4i*>(a.unpooled + x0 + rowb + a.pool_c) = o[3];
   }
 }
 
@@ -978,14 +1031,26 @@ extern "C" int niti_head_i8_forward(const int8_t* act, const int8_t* w, int8_t* 
   return check_launch("head_forward");
 }
 
-extern "C" int niti_head_i8_backward(const int8_t* err, const int8_t* act, const int8_t* drop_mask, int8_t* w, int8_t* dx8, int M, int O,
-                                     int F, int err_bits, int err_method, int grad_bits, int grad_method, int div_mode, int bw_mode,
-                                     uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out, int32_t* grad_shift_out,
-                                     const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act, int exp_act_bias,
-                                     int32_t* err_exp_out, int32_t* grad_exp_out, void* stream) {
+static int head_backward(const int8_t* err, const int8_t* act, const int8_t* drop_mask, int8_t* w, int8_t* dx8, int M, int O,
+                         int F, int err_bits, int err_method, int grad_bits, int grad_method, int div_mode, int bw_mode,
+                         uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out, int32_t* grad_shift_out,
+                         const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act, int exp_act_bias,
+                         int32_t* err_exp_out, int32_t* grad_exp_out, const int8_t* pool_in, int8_t* unpooled, int P, int Q, int C,
+                         int pool_flags, void* stream) {
   clear_error();
   if (M <= 0 || O <= 0 || F <= 0) return fail(NITI_ERR_INVALID_ARG, "head_backward: non-positive extent");
-  if (err == nullptr || act == nullptr || w == nullptr || dx8 == nullptr || sync == nullptr) return fail(NITI_ERR_INVALID_ARG, "head_backward: null pointer");
+  if (err == nullptr || act == nullptr || w == nullptr || sync == nullptr || (dx8 == nullptr && pool_in == nullptr))
+    return fail(NITI_ERR_INVALID_ARG, "head_backward: null pointer");
+  int ties = 0;
+  if (pool_in != nullptr) {
+    ties = pool_flags & ~NITI_POOL_BWD_RELU;
+    if (ties != NITI_TIES_FIRST && ties != NITI_TIES_ALL) return fail(NITI_ERR_INVALID_ARG, "head_backward_unpool: ties=%d", ties);
+    if (unpooled == nullptr || !aligned16(pool_in) || !aligned16(unpooled))
+      return fail(NITI_ERR_INVALID_ARG, "head_backward_unpool: the pool's input and the result must be 16-byte aligned arrays");
+    if (P <= 0 || Q <= 0 || C <= 0 || C % kHeadSlab != 0 || static_cast<long long>(P) * Q * C != F)
+      return fail(NITI_ERR_UNSUPPORTED, "head_backward_unpool: F=%d is not P=%d x Q=%d x C=%d with C a multiple of %d", F, P, Q, C, kHeadSlab);
+    if (4LL * M * F >= 0x7fffffffLL) return fail(NITI_ERR_UNSUPPORTED, "head_backward_unpool: more than 2^31 elements");
+  }
   if (err_bits < 1 || err_bits > 7 || grad_bits < 1 || grad_bits > 7)
     return fail(NITI_ERR_INVALID_ARG, "head_backward: err_bits=%d grad_bits=%d outside 1..7", err_bits, grad_bits);
   for (const int method : {err_method, grad_method})
@@ -997,7 +1062,7 @@ extern "C" int niti_head_i8_backward(const int8_t* err, const int8_t* act, const
   if (nb == 0)
     return fail(NITI_ERR_UNSUPPORTED, "head_backward: M=%d O=%d F=%d outside the kernel (M <= %d, O <= %d, F a multiple of %d); use the separate passes",
                 M, O, F, kHeadMaxM, kMaxOut, kHeadSlab);
-  if (!aligned16(act) || !aligned16(w) || !aligned16(dx8) || (drop_mask != nullptr && !aligned16(drop_mask)))
+  if (!aligned16(act) || !aligned16(w) || (dx8 != nullptr && !aligned16(dx8)) || (drop_mask != nullptr && !aligned16(drop_mask)))
     return fail(NITI_ERR_INVALID_ARG, "head_backward: act, w, dx8 and the mask must be 16-byte aligned");
   const size_t need = niti_head_i8_sync_words(1, M, O, F);
   if (sync_words < need) return fail(NITI_ERR_WORKSPACE, "head_backward: needs %zu zeroed sync words, got %zu", need, sync_words);
@@ -1032,6 +1097,41 @@ extern "C" int niti_head_i8_backward(const int8_t* err, const int8_t* act, const
   a.exp_act_bias = exp_act_bias;
   a.err_exp_out = err_exp_out;
   a.grad_exp_out = grad_exp_out;
+  a.pool_in = pool_in;
+  a.unpooled = unpooled;
+  a.pool_q = Q;
+  a.pool_c = C;
+  a.pool_ties_all = ties == NITI_TIES_ALL ? 1 : 0;
+  a.pool_relu = (pool_flags & NITI_POOL_BWD_RELU) != 0 ? 1 : 0;
   hipLaunchKernelGGL(fc_head_bwd_kernel, dim3(static_cast<unsigned>(nb)), dim3(1024), 0, static_cast<hipStream_t>(stream), a);
   return check_launch("head_backward");
+}
+
+extern "C" int niti_head_i8_backward(const int8_t* err, const int8_t* act, const int8_t* drop_mask, int8_t* w, int8_t* dx8, int M, int O,
+                                     int F, int err_bits, int err_method, int grad_bits, int grad_method, int div_mode, int bw_mode,
+                                     uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out, int32_t* grad_shift_out,
+                                     const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act, int exp_act_bias,
+                                     int32_t* err_exp_out, int32_t* grad_exp_out, void* stream) {
+  if (dx8 == nullptr) {
+    clear_error();
+    return fail(NITI_ERR_INVALID_ARG, "head_backward: null pointer");
+  }
+  return head_backward(err, act, drop_mask, w, dx8, M, O, F, err_bits, err_method, grad_bits, grad_method, div_mode, bw_mode, sync, sync_words,
+                       g8_out, err_shift_out, grad_shift_out, exp_err, exp_w, exp_act, exp_act_bias, err_exp_out, grad_exp_out, nullptr, nullptr,
+                       0, 0, 0, 0, stream);
+}
+
+extern "C" int niti_head_i8_backward_unpool(const int8_t* err, const int8_t* act, const int8_t* drop_mask, int8_t* w, int8_t* dx8, int M,
+                                            int O, int F, int err_bits, int err_method, int grad_bits, int grad_method, int div_mode,
+                                            int bw_mode, uint32_t* sync, size_t sync_words, int8_t* g8_out, int32_t* err_shift_out,
+                                            int32_t* grad_shift_out, const int32_t* exp_err, const int32_t* exp_w, const int32_t* exp_act,
+                                            int exp_act_bias, int32_t* err_exp_out, int32_t* grad_exp_out, const int8_t* pool_in,
+                                            int8_t* unpooled, int P, int Q, int C, int pool_flags, void* stream) {
+  if (pool_in == nullptr) {
+    clear_error();
+    return fail(NITI_ERR_INVALID_ARG, "head_backward_unpool: null pointer");
+  }
+  return head_backward(err, act, drop_mask, w, dx8, M, O, F, err_bits, err_method, grad_bits, grad_method, div_mode, bw_mode, sync, sync_words,
+                       g8_out, err_shift_out, grad_shift_out, exp_err, exp_w, exp_act, exp_act_bias, err_exp_out, grad_exp_out, pool_in, unpooled,
+                       P, Q, C, pool_flags, stream);
 }

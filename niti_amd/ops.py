@@ -815,10 +815,13 @@ def head_forward(act, w, target_bits=7, method="round", div_mode="floor", bw_mod
 
 def head_backward(err, act, w, err_bits=7, err_method="psto", grad_bits=5, grad_method="psto", div_mode="floor", bw_mode="int",
                   drop_mask=None, want_grad=False, sync=None, exp_err=None, exp_w=None, exp_act=None, exp_act_bias=0,
-                  err_exp_out=None, grad_exp_out=None):
+                  err_exp_out=None, grad_exp_out=None, unpool=None):
     """Classifier backward in one launch (niti_head_i8_backward): err [M,O], act [M,F] (in front of the dropout),
     w [O,F] (updated in place), ``drop_mask`` int8 [F] of 0 / 1 or None.  Returns (dx8 [M,F] with the mask applied,
-    rounded gradient [O,F] or None, err shift, grad shift, sync)."""
+    rounded gradient [O,F] or None, err shift, grad shift, sync).
+    ``unpool`` = (pool_in [M,2P,2Q,C], ties, relu): act is the flattened output of a 2 x 2 max-pool over pool_in; the launch
+    also routes dx8 through that pool's backward pass (niti_head_i8_backward_unpool) and a sixth element is returned:
+    the gradient [M,2P,2Q,C]."""
     _chk_dev(err, act, w, drop_mask, sync, exp_err, exp_w, exp_act, err_exp_out, grad_exp_out)
     if (err.dtype != torch.int8 or act.dtype != torch.int8 or w.dtype != torch.int8 or err.dim() != 2 or act.dim() != 2
             or w.dim() != 2 or err.shape[0] != act.shape[0] or tuple(w.shape) != (err.shape[1], act.shape[1])):
@@ -839,6 +842,22 @@ def head_backward(err, act, w, err_bits=7, err_method="psto", grad_bits=5, grad_
     dx = torch.empty((M, F), dtype=torch.int8, device=err.device)
     g8 = torch.empty_like(w) if want_grad else None
     shifts = torch.empty(2, dtype=torch.int32, device=err.device)
+    if unpool is not None:
+        pool_in, ties, relu = unpool
+        _chk_dev(pool_in)
+        if pool_in.dtype != torch.int8 or pool_in.dim() != 4 or not pool_in.is_contiguous() or pool_in.shape[0] != M:
+            raise RuntimeError("head_backward: unpool wants the pool's contiguous int8 input [M,2P,2Q,C]")
+        H2, W2, C = pool_in.shape[1:]
+        if H2 % 2 or W2 % 2 or (H2 // 2) * (W2 // 2) * C != F:
+            raise RuntimeError("head_backward: the pool's input %s does not pool to %d features" % (tuple(pool_in.shape), F))
+        out = torch.empty_like(pool_in)
+        st = L.lib().niti_head_i8_backward_unpool(
+            _ptr(err), _ptr(act), _ptr(drop_mask), _ptr(w), _ptr(dx), M, O, F, err_bits, L.ROUND[err_method], grad_bits,
+            L.ROUND[grad_method], L.DIV[div_mode], L.BW[bw_mode], _ptr(sync), sync.numel(), _ptr(g8), _ptr(shifts[0:1]),
+            _ptr(shifts[1:2]), _ptr(exp_err), _ptr(exp_w), _ptr(exp_act), int(exp_act_bias), _ptr(err_exp_out), _ptr(grad_exp_out),
+            _ptr(pool_in), _ptr(out), H2 // 2, W2 // 2, C, L.TIES[ties] | (L.POOL_BWD_RELU if relu else 0), _stream(err))
+        L.check(st, "niti_head_i8_backward_unpool")
+        return dx, g8, shifts[0:1], shifts[1:2], sync, out
     st = L.lib().niti_head_i8_backward(_ptr(err), _ptr(act), _ptr(drop_mask), _ptr(w), _ptr(dx), M, O, F, err_bits,
                                        L.ROUND[err_method], grad_bits, L.ROUND[grad_method], L.DIV[div_mode], L.BW[bw_mode],
                                        _ptr(sync), sync.numel(), _ptr(g8), _ptr(shifts[0:1]), _ptr(shifts[1:2]), _ptr(exp_err),

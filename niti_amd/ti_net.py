@@ -58,6 +58,14 @@ class TiNet(Module):
                 # plain attributes, not sub-modules: the two layers refer to each other
                 layers[-1].__dict__["drop_below"] = layers[-2]
                 layers[-2].__dict__["head"] = layers[-1]
+            # 2x2 / stride-2 max-pool -> TiFlat -> [TiDropout ->] classifier: the classifier's backward launch routes its
+            # data gradient through that pool's backward pass as well
+            j = len(layers) - 2
+            if j >= 0 and isinstance(layers[j], ti_torch.TiDropout):
+                j -= 1
+            if (j >= 1 and isinstance(layers[j], ti_torch.TiFlat) and isinstance(layers[j - 1], ti_torch.TiMaxpool2d)
+                    and (layers[j - 1].kernel_size, layers[j - 1].stride, layers[j - 1].padding) == (2, 2, 0)):
+                layers[-1].__dict__["pool_below"] = layers[j - 1]
         return self
 
     def forward(self, x, target=None):

@@ -683,16 +683,25 @@ class TiLinear(UpdateWeight):
         mask = self._dropped     # the forward pass read ``act`` through this mask: act_in is the tensor in front of the dropout
         if not KEEP_INT32_GRAD and self._head("backward", M, (ERROR_ROUND_METHOD, GRAD_ROUND_METHOD), (rand, grad_rand)):
             exps = torch.empty(2, dtype=torch.int32, device=dev)
+            # the 2x2 max-pool whose flattened output this layer read (TiNet.fuse): its backward pass in the same launch
+            pool = self.__dict__.get("pool_below")
+            unpool = None
+            if (pool is not None and getattr(pool, "act_out", None) is not None and pool.act_out.data_ptr() == act.data_ptr()
+                    and pool.act_out.numel() == act.numel() and pool.act_in.dim() == 4 and pool.act_in.is_contiguous()
+                    and pool.act_in.dtype == torch.int8 and pool.act_in.shape[3] % 64 == 0):
+                unpool = (pool.act_in, POOL_TIES, pool.relu_below)
             done = self._try("head-backward", M, lambda: ops.head_backward(
                 err_in, act, self.weight, BITWIDTH, _method_name(ERROR_ROUND_METHOD), GRAD_BITWIDTH, _method_name(GRAD_ROUND_METHOD),
                 DIV_MODE, BW_MODE, drop_mask=mask, want_grad=self.keep_grad, exp_err=self.err_exp_in, exp_w=self._wexp(),
                 exp_act=_exp_tensor(self.act_in_exp, dev), exp_act_bias=1 if mask is not None else 0,
-                err_exp_out=exps[0:1], grad_exp_out=exps[1:2]))
+                err_exp_out=exps[0:1], grad_exp_out=exps[1:2], unpool=unpool))
             if done is not None:
                 self.err_exp, self.grad_exp = exps[0:1], exps[1:2]
                 self.grad, self.grad_shift, self.grad_int32acc = done[1], done[3], None
                 if mask is not None:
                     self.drop_below.bwd_done = done[0]     # masked already
+                if unpool is not None:
+                    pool.bwd_routed = (done[0], done[5])
                 return done[0], self.err_exp
         if mask is not None:     # the separate passes want the masked activations and their exponent
             act, self.act_in_exp = ops.mask_features(act, mask, _exp_tensor(self.act_in_exp, dev), 1)
@@ -772,6 +781,7 @@ class TiMaxpool2d(Module):
         self.relu_below = False     # the ReLU in front of this layer leaves its backward pass to this layer
         self.preset = None          # (input tensor, pooled tensor) left by the convolution that computed both
         self.bwd_done = None        # the error tensor a convolution behind this layer has already routed through it
+        self.bwd_routed = None      # (error tensor, routed result) left by the classifier behind this layer
 
     def forward(self, input):
         self.act_in, exp_in = input
@@ -788,6 +798,9 @@ class TiMaxpool2d(Module):
         done, self.bwd_done = self.bwd_done, None
         if done is not None and done is err_in:
             return input        # the data gradient behind this layer wrote its result through this pooling already
+        routed, self.bwd_routed = self.bwd_routed, None
+        if routed is not None and routed[0].data_ptr() == err_in.data_ptr() and routed[0].numel() == err_in.numel():
+            return routed[1], err_exp     # the classifier's backward launch has run this pass
         err_out = ops.maxpool_bwd(self.act_out, err_in.contiguous(), self.act_in, self.kernel_size, self.stride,
                                   self.padding, POOL_TIES, relu=self.relu_below)
         return err_out, err_exp

@@ -209,3 +209,38 @@ def test_head_backward(dev, case, div_mode):
             assert int(eo.cpu()[0]) == dsh - 7 and int(eo.cpu()[1]) == gsh + dsh - 7 - 4 + (1 if use_mask else 0)
     assert ops.head_sync_words("backward", 257, 10, 512) == 0 and ops.head_sync_words("backward", 128, 17, 512) == 0
     assert ops.head_sync_words("backward", 128, 10, 96) == 0 and ops.head_sync_words("forward", 128, 17, 512) == 0
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", [(128, 10, 4, 4, 512), (37, 7, 2, 3, 64), (256, 16, 1, 1, 128)])   # M, O, P, Q, C
+@pytest.mark.parametrize("ties", ["first", "all"])
+def test_head_backward_unpool(dev, case, ties):
+    """niti_head_i8_backward_unpool: the classifier's backward launch followed through the 2 x 2 max-pool in front of it,
+    against niti_head_i8_backward's data gradient routed by the oracle's max-pool backward (+ the ReLU mask).  The pool's
+    input has few distinct values: many windows with several equal maxima, many non-positive maxima."""
+    from niti_amd import ops
+    from oracle import niti_oracle as po
+    M, O, P, Q, C = case
+    F = P * Q * C
+    _say("head_backward_unpool", case, ties)
+    g = torch.Generator().manual_seed(7300 + M + O + F)
+    x = ri8(g, M, 2 * P, 2 * Q, C, lo=-3, hi=5)
+    y = po.maxpool_fwd(x)
+    act = y.reshape(M, F).contiguous()
+    w, err = ri8(g, O, F), ri8(g, M, O, lo=-40, hi=40)
+    mask = torch.randint(0, 2, (F,), generator=g, dtype=torch.int8)
+    for relu in (False, True):
+        for use_mask in (False, True):
+            wd = w.to(dev).clone()
+            dx, _, _, _, sync, routed = ops.head_backward(err.to(dev), act.to(dev), wd, 7, "round", 5, "psto", "floor",
+                                                          drop_mask=mask.to(dev) if use_mask else None,
+                                                          unpool=(x.to(dev), ties, relu))
+            wd2 = w.to(dev).clone()
+            dx_plain, _, _, _, _ = ops.head_backward(err.to(dev), act.to(dev), wd2, 7, "round", 5, "psto", "floor",
+                                                     drop_mask=mask.to(dev) if use_mask else None)
+            assert int(sync.cpu()[1]) == 0
+            assert torch.equal(dx.cpu(), dx_plain.cpu()) and torch.equal(wd.cpu(), wd2.cpu())
+            ref = po.maxpool_bwd(y, dx_plain.cpu().reshape(M, P, Q, C), x, ties=ties)
+            if relu:
+                ref = torch.where(x > 0, ref, torch.zeros_like(ref))
+            assert torch.equal(routed.cpu(), ref.to(torch.int8)), (relu, use_mask)
